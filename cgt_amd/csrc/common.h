@@ -1,0 +1,51 @@
+// Shared helpers of the cgt_amd HIP library (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdio>
+#include "cgt_amd.h"
+
+#define CGT_API extern "C" __attribute__((visibility("default")))
+
+namespace cgt_amd {
+
+// Per-thread message of the last failure; read through cgt_amd_last_error().
+void set_error(const char* fmt, ...);
+void clear_error();
+
+inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
+
+constexpr int kWave = 64;    // CDNA wavefront width
+constexpr int kNumXCD = 8;   // MI355X: 8 accelerator dies, each with its own L2
+
+inline long cdiv(long a, long b) { return (a + b - 1) / b; }
+
+}  // namespace cgt_amd
+
+#define CGT_HIP_TRY(expr)                                                          \
+    do {                                                                           \
+        hipError_t e_ = (expr);                                                    \
+        if (e_ != hipSuccess) {                                                    \
+            cgt_amd::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), \
+                               __FILE__, __LINE__);                                \
+            return CGT_AMD_ERR_HIP;                                                \
+        }                                                                          \
+    } while (0)
+
+#define CGT_ARG_CHECK(cond, ...)                \
+    do {                                        \
+        if (!(cond)) {                          \
+            cgt_amd::set_error(__VA_ARGS__);    \
+            return CGT_AMD_ERR_ARG;             \
+        }                                       \
+    } while (0)
+
+// After a kernel launch: surface launch-configuration errors as a status.
+#define CGT_LAUNCH_CHECK(name)                                                     \
+    do {                                                                           \
+        hipError_t e_ = hipGetLastError();                                         \
+        if (e_ != hipSuccess) {                                                    \
+            cgt_amd::set_error("launch of %s failed: %s", name, hipGetErrorString(e_)); \
+            return CGT_AMD_ERR_HIP;                                                \
+        }                                                                          \
+    } while (0)

@@ -1,0 +1,281 @@
+// im2col / col2im for gfx950.  Both are HBM-bound copies / ordered sums.
+//
+// Layouts (as in CGT): image [B,C,H,W]; column buffer [B,m,n,Z] with
+// Z = C*kh*kw ordered (channel, kernel row, kernel col).
+//
+// im2col: one workgroup owns (image b, output row h, a chunk of channels).
+//   It stages the kh input rows of its channels into LDS with coalesced row
+//   reads (zero padded left/right/top/bottom, so the inner loop has no bounds
+//   tests), then streams the output row: consecutive lanes write consecutive
+//   z, so every store instruction covers one contiguous run of the column
+//   buffer.  Each input element is read from HBM kh/sh times at most (the
+//   neighbouring rows' workgroups run at the same time and share L2).
+//
+// col2im: gather form of the reference's scatter loop.  Each image pixel sums
+//   its taps in ascending (kernel row, kernel col) order, which for a fixed
+//   channel is ascending z -- the order the sequential reference adds them in
+//   -- so no atomics are needed and the result is bit-identical.
+#include "common.h"
+
+namespace cgt_amd {
+
+// Geometry known at compile time (hot shapes) ...
+template <int KH, int KW, int PH, int PW, int SH, int SW>
+struct StaticGeom {
+    __host__ __device__ constexpr int kh() const { return KH; }
+    __host__ __device__ constexpr int kw() const { return KW; }
+    __host__ __device__ constexpr int ph() const { return PH; }
+    __host__ __device__ constexpr int pw() const { return PW; }
+    __host__ __device__ constexpr int sh() const { return SH; }
+    __host__ __device__ constexpr int sw() const { return SW; }
+};
+// ... or only at run time (anything else).
+struct DynGeom {
+    int kh_, kw_, ph_, pw_, sh_, sw_;
+    __host__ __device__ int kh() const { return kh_; }
+    __host__ __device__ int kw() const { return kw_; }
+    __host__ __device__ int ph() const { return ph_; }
+    __host__ __device__ int pw() const { return pw_; }
+    __host__ __device__ int sh() const { return sh_; }
+    __host__ __device__ int sw() const { return sw_; }
+};
+
+constexpr int kIm2colThreads = 256;
+constexpr int kIm2colWaves = kIm2colThreads / kWave;
+
+// VEC: 4 consecutive z per lane, 16-byte stores (needs Z%4==0, chunk*kh*kw%4==0).
+template <class G, bool VEC>
+__global__ __launch_bounds__(kIm2colThreads) void im2col_rows_kernel(
+    G g, const float* __restrict__ im, float* __restrict__ col, int C, int H, int W, int m, int n,
+    int chunk, int nchunks) {
+    extern __shared__ float tile[];  // [cc*kh][Wp], Wp = W + 2*pw
+
+    const int KH = g.kh(), KW = g.kw();
+    const int Wp = W + 2 * g.pw();
+    const long bid = blockIdx.x;
+    const int ck = (int)(bid % nchunks);
+    const int h = (int)((bid / nchunks) % m);
+    const long b = bid / ((long)nchunks * m);
+    const int c0 = ck * chunk;
+    const int cc = min(chunk, C - c0);
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+
+    // stage rows: LDS row r = (c, ho) <- image row h*sh - ph + ho of channel c0+c
+    const int nrows = cc * KH;
+    const int hbase = h * g.sh() - g.ph();
+    for (int r = wave; r < nrows; r += kIm2colWaves) {
+        const int c = r / KH, ho = r - c * KH;
+        const int hp = hbase + ho;
+        const bool rowok = hp >= 0 && hp < H;
+        const float* src = im + ((b * C + c0 + c) * (long)H + (rowok ? hp : 0)) * W;
+        float* dst = tile + r * Wp;
+        for (int x = lane; x < Wp; x += kWave) {
+            const int wp = x - g.pw();
+            dst[x] = (rowok && wp >= 0 && wp < W) ? src[wp] : 0.0f;
+        }
+    }
+    __syncthreads();
+
+    const int KK = KH * KW;
+    const int zc_n = cc * KK;                // z's this workgroup writes per output pixel
+    const long Z = (long)C * KK;
+    float* orow = col + ((b * m + h) * (long)n) * Z + (long)c0 * KK;
+    for (int w = wave; w < n; w += kIm2colWaves) {
+        float* out = orow + (long)w * Z;
+        const int xbase = w * g.sw();
+        if (VEC) {
+            for (int z4 = lane * 4; z4 < zc_n; z4 += kWave * 4) {
+                float v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int zc = z4 + j;
+                    const int c = zc / KK, r = zc - c * KK;
+                    const int ho = r / KW, wo = r - ho * KW;
+                    v[j] = tile[(c * KH + ho) * Wp + xbase + wo];
+                }
+                *reinterpret_cast<float4*>(out + z4) = make_float4(v[0], v[1], v[2], v[3]);
+            }
+        } else {
+            for (int zc = lane; zc < zc_n; zc += kWave) {
+                const int c = zc / KK, r = zc - c * KK;
+                const int ho = r / KW, wo = r - ho * KW;
+                out[zc] = tile[(c * KH + ho) * Wp + xbase + wo];
+            }
+        }
+    }
+}
+
+// Fallback for rows too wide for LDS staging: one thread per output element.
+template <class G>
+__global__ __launch_bounds__(256) void im2col_direct_kernel(
+    G g, const float* __restrict__ im, float* __restrict__ col, long total, int C, int H, int W,
+    int m, int n) {
+    const int KH = g.kh(), KW = g.kw();
+    const long Z = (long)C * KH * KW;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const int z = (int)(idx % Z);
+        long t = idx / Z;
+        const int w = (int)(t % n);
+        t /= n;
+        const int h = (int)(t % m);
+        const long b = t / m;
+        const int c = z / (KH * KW), r = z - c * (KH * KW);
+        const int ho = r / KW, wo = r - ho * KW;
+        const int hp = h * g.sh() - g.ph() + ho, wp = w * g.sw() - g.pw() + wo;
+        float v = 0.0f;
+        if (hp >= 0 && hp < H && wp >= 0 && wp < W) v = im[((b * C + c) * (long)H + hp) * W + wp];
+        col[idx] = v;
+    }
+}
+
+// One thread per image pixel; taps added in ascending (ho, wo).
+template <class G>
+__global__ __launch_bounds__(256) void col2im_gather_kernel(
+    G g, const float* __restrict__ col, float* __restrict__ im, long total, int C, int H, int W,
+    int m, int n) {
+    const int KH = g.kh(), KW = g.kw();
+    const long Z = (long)C * KH * KW;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const int wp = (int)(idx % W);
+        long t = idx / W;
+        const int hp = (int)(t % H);
+        t /= H;
+        const int c = (int)(t % C);
+        const long b = t / C;
+        float acc = 0.0f;
+        for (int ho = 0; ho < KH; ++ho) {
+            const int hh = hp + g.ph() - ho;
+            if (hh < 0) break;
+            const int h = hh / g.sh();
+            if (h * g.sh() != hh || h >= m) continue;
+            for (int wo = 0; wo < KW; ++wo) {
+                const int ww = wp + g.pw() - wo;
+                if (ww < 0) break;
+                const int w = ww / g.sw();
+                if (w * g.sw() != ww || w >= n) continue;
+                acc += col[((b * m + h) * (long)n + w) * Z + (c * KH + ho) * KW + wo];
+            }
+        }
+        im[idx] = acc;
+    }
+}
+
+static int check_geom(const char* what, long B, long C, long H, long W, int kh, int kw, int ph,
+                      int pw, int sh, int sw, long* m, long* n) {
+    CGT_ARG_CHECK(B >= 0 && C >= 0 && H >= 0 && W >= 0, "%s: negative shape", what);
+    CGT_ARG_CHECK(kh > 0 && kw > 0 && sh > 0 && sw > 0 && ph >= 0 && pw >= 0,
+                  "%s: bad geometry k=(%d,%d) p=(%d,%d) s=(%d,%d)", what, kh, kw, ph, pw, sh, sw);
+    CGT_ARG_CHECK(H + 2 * ph >= kh && W + 2 * pw >= kw, "%s: kernel larger than padded image", what);
+    *m = (H + 2 * ph - kh) / sh + 1;
+    *n = (W + 2 * pw - kw) / sw + 1;
+    CGT_ARG_CHECK(C * H * W < (1L << 31) && (*m) * (*n) * C * kh * kw < (1L << 40) &&
+                      H < (1 << 24) && W < (1 << 24) && C < (1 << 24),
+                  "%s: shape too large", what);
+    return CGT_AMD_OK;
+}
+
+static int gcd4(int v) { return (v % 4 == 0) ? 4 : (v % 2 == 0) ? 2 : 1; }
+
+template <class G>
+static int launch_im2col(G g, const float* im, long B, int C, int H, int W, int m, int n,
+                         float* col, hipStream_t st) {
+    const int KK = g.kh() * g.kw();
+    const long Z = (long)C * KK;
+    const int Wp = W + 2 * g.pw();
+    const long row_bytes = (long)g.kh() * Wp * sizeof(float);  // LDS per channel
+    const long lds_budget = 32 * 1024;
+    if (row_bytes <= 64 * 1024 && B * m < (1L << 31) / 64) {
+        int chunk = (int)(lds_budget / row_bytes);
+        if (chunk < 1) chunk = 1;
+        if (chunk > C) chunk = C;
+        // 16-byte stores need every chunk's z-run to start and end on a
+        // multiple of 4 floats: Z % 4 == 0 and (chunk*kh*kw) % 4 == 0.
+        bool vec = (Z % 4 == 0) && (reinterpret_cast<uintptr_t>(col) % 16 == 0);
+        if (vec && chunk < C) {
+            const int step = 4 / gcd4(KK);       // smallest channel count with (step*KK) % 4 == 0
+            if (chunk >= step) chunk = chunk / step * step;
+            else vec = false;
+        }
+        const int nchunks = (int)cdiv(C, chunk);
+        const size_t lds = (size_t)chunk * row_bytes;
+        const long blocks = B * m * nchunks;
+        if (blocks == 0) return CGT_AMD_OK;
+        if (vec)
+            im2col_rows_kernel<G, true><<<dim3((unsigned)blocks), dim3(kIm2colThreads), lds, st>>>(
+                g, im, col, C, H, W, m, n, chunk, nchunks);
+        else
+            im2col_rows_kernel<G, false><<<dim3((unsigned)blocks), dim3(kIm2colThreads), lds, st>>>(
+                g, im, col, C, H, W, m, n, chunk, nchunks);
+        CGT_LAUNCH_CHECK("im2col_rows_kernel");
+        return CGT_AMD_OK;
+    }
+    const long total = B * m * n * Z;
+    if (total == 0) return CGT_AMD_OK;
+    long blocks = cdiv(total, 256);
+    if (blocks > 1 << 20) blocks = 1 << 20;
+    im2col_direct_kernel<G><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(g, im, col, total, C, H, W, m, n);
+    CGT_LAUNCH_CHECK("im2col_direct_kernel");
+    return CGT_AMD_OK;
+}
+
+template <class G>
+static int launch_col2im(G g, const float* col, long B, int C, int H, int W, int m, int n,
+                         float* im, hipStream_t st) {
+    const long total = B * C * H * W;
+    if (total == 0) return CGT_AMD_OK;
+    long blocks = cdiv(total, 256);
+    if (blocks > 1 << 20) blocks = 1 << 20;
+    col2im_gather_kernel<G><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(g, col, im, total, C, H, W, m, n);
+    CGT_LAUNCH_CHECK("col2im_gather_kernel");
+    return CGT_AMD_OK;
+}
+
+// Geometries compiled with constant index math: (kh, kw, ph, pw, sh, sw).
+#define CGT_STATIC_GEOMS(X) \
+    X(3, 3, 1, 1, 1, 1)     \
+    X(5, 5, 2, 2, 1, 1)     \
+    X(11, 11, 0, 0, 4, 4)   \
+    X(3, 3, 0, 0, 1, 1)     \
+    X(1, 1, 0, 0, 1, 1)
+
+}  // namespace cgt_amd
+
+using namespace cgt_amd;
+
+CGT_API int cgt_amd_im2col_f32(const float* im, long B, long C, long H, long W, int kh, int kw,
+                               int ph, int pw, int sh, int sw, float* col, void* stream) {
+    long m, n;
+    int rc = check_geom("im2col", B, C, H, W, kh, kw, ph, pw, sh, sw, &m, &n);
+    if (rc) return rc;
+    if (B * m * n * C == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(im && col, "im2col: null pointer");
+    hipStream_t st = as_stream(stream);
+#define X(KH, KW, PH, PW, SH, SW)                                                     \
+    if (kh == KH && kw == KW && ph == PH && pw == PW && sh == SH && sw == SW)         \
+        return launch_im2col(StaticGeom<KH, KW, PH, PW, SH, SW>(), im, B, (int)C, (int)H, (int)W, \
+                             (int)m, (int)n, col, st);
+    CGT_STATIC_GEOMS(X)
+#undef X
+    return launch_im2col(DynGeom{kh, kw, ph, pw, sh, sw}, im, B, (int)C, (int)H, (int)W, (int)m,
+                         (int)n, col, st);
+}
+
+CGT_API int cgt_amd_col2im_f32(const float* col, long B, long C, long H, long W, int kh, int kw,
+                               int ph, int pw, int sh, int sw, float* im, void* stream) {
+    long m, n;
+    int rc = check_geom("col2im", B, C, H, W, kh, kw, ph, pw, sh, sw, &m, &n);
+    if (rc) return rc;
+    if (B * C * H * W == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(im && col, "col2im: null pointer");
+    hipStream_t st = as_stream(stream);
+#define X(KH, KW, PH, PW, SH, SW)                                                     \
+    if (kh == KH && kw == KW && ph == PH && pw == PW && sh == SH && sw == SW)         \
+        return launch_col2im(StaticGeom<KH, KW, PH, PW, SH, SW>(), col, B, (int)C, (int)H, (int)W, \
+                             (int)m, (int)n, im, st);
+    CGT_STATIC_GEOMS(X)
+#undef X
+    return launch_col2im(DynGeom{kh, kw, ph, pw, sh, sw}, col, B, (int)C, (int)H, (int)W, (int)m,
+                         (int)n, im, st);
+}

@@ -1,0 +1,244 @@
+// Cross-channel local response normalisation for gfx950.  HBM-bound.
+//
+// Arrays are [N,C,H,W]; the window runs along C, so neighbours in the window
+// are H*W floats apart while neighbours in a wavefront (consecutive pixels)
+// are adjacent: every load/store instruction is one contiguous run.
+//
+// A thread owns one pixel (n, p) and a run of channels; it walks the run with
+// the window held in registers, so x is read once (plus a halo of size-1
+// channels per run), scale and top are written once, in a single fused pass:
+// 3 array passes forward, 5 backward.  The window sum is taken directly over
+// the registers (not as the reference's running add/subtract), which is more
+// accurate and independent of the walk direction.
+#include "common.h"
+#include <algorithm>
+
+namespace cgt_amd {
+
+constexpr int kLrnThreads = 256;
+
+__device__ __forceinline__ float pow_neg_beta(float s, float nbeta) {
+    // s >= k > 0.  exp2(nbeta*log2(s)) on the hardware transcendental units:
+    // relative error ~1e-6 for the scale range LRN produces.
+    return __builtin_amdgcn_exp2f(nbeta * __builtin_amdgcn_logf(s));
+}
+
+// SIZE > 0: window length known at compile time (ring in registers).
+template <int SIZE>
+__global__ __launch_bounds__(kLrnThreads) void lrn_fwd_kernel(
+    const float* __restrict__ x, float* __restrict__ top, float* __restrict__ scale, int C,
+    int HW, int crun, float aos, float nbeta, float kconst) {
+    constexpr int PRE = (SIZE - 1) / 2, POST = SIZE - PRE - 1;
+    const int p = blockIdx.x * kLrnThreads + threadIdx.x;
+    if (p >= HW) return;
+    const long n = blockIdx.z;
+    const int cs = blockIdx.y * crun, ce = min(C, cs + crun);
+    const float* xp = x + n * C * (long)HW + p;
+    float* tp = top + n * C * (long)HW + p;
+    float* sp = scale + n * C * (long)HW + p;
+
+    float ring[SIZE];  // ring[j] = x[c - PRE + j]
+#pragma unroll
+    for (int j = 1; j < SIZE; ++j) {
+        const int c = cs - PRE + j - 1;
+        ring[j] = (c >= 0 && c < C) ? xp[(long)c * HW] : 0.0f;
+    }
+#pragma unroll 4
+    for (int c = cs; c < ce; ++c) {
+#pragma unroll
+        for (int j = 0; j < SIZE - 1; ++j) ring[j] = ring[j + 1];
+        const int ch = c + POST;
+        ring[SIZE - 1] = (ch < C) ? xp[(long)ch * HW] : 0.0f;
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < SIZE; ++j) acc += ring[j] * ring[j];
+        const float s = kconst + acc * aos;
+        sp[(long)c * HW] = s;
+        tp[(long)c * HW] = ring[PRE] * pow_neg_beta(s, nbeta);
+    }
+}
+
+// Any window length: re-reads the window through the cache.
+__global__ __launch_bounds__(kLrnThreads) void lrn_fwd_generic_kernel(
+    const float* __restrict__ x, float* __restrict__ top, float* __restrict__ scale, int C,
+    int HW, int crun, int size, float aos, float nbeta, float kconst) {
+    const int pre = (size - 1) / 2, post = size - pre - 1;
+    const int p = blockIdx.x * kLrnThreads + threadIdx.x;
+    if (p >= HW) return;
+    const long n = blockIdx.z;
+    const int cs = blockIdx.y * crun, ce = min(C, cs + crun);
+    const long base = n * C * (long)HW + p;
+    for (int c = cs; c < ce; ++c) {
+        float acc = 0.0f;
+        const int lo = max(0, c - pre), hi = min(C - 1, c + post);
+        for (int cc = lo; cc <= hi; ++cc) {
+            const float v = x[base + (long)cc * HW];
+            acc += v * v;
+        }
+        const float s = kconst + acc * aos;
+        scale[base + (long)c * HW] = s;
+        top[base + (long)c * HW] = x[base + (long)c * HW] * pow_neg_beta(s, nbeta);
+    }
+}
+
+template <int SIZE>
+__global__ __launch_bounds__(kLrnThreads) void lrn_bwd_kernel(
+    const float* __restrict__ x, const float* __restrict__ top, const float* __restrict__ scale,
+    const float* __restrict__ top_diff, float* __restrict__ bottom_diff, int C, int HW, int crun,
+    float nbeta, float ratio) {
+    // transposed window: [c - PRE, c + POST]
+    constexpr int PRE = SIZE - (SIZE + 1) / 2, POST = SIZE - PRE - 1;
+    const int p = blockIdx.x * kLrnThreads + threadIdx.x;
+    if (p >= HW) return;
+    const long n = blockIdx.z;
+    const int cs = blockIdx.y * crun, ce = min(C, cs + crun);
+    const long base = n * C * (long)HW + p;
+    const float* xp = x + base;
+    const float* tp = top + base;
+    const float* sp = scale + base;
+    const float* dp = top_diff + base;
+    float* bp = bottom_diff + base;
+
+    float tr[SIZE];       // tr[j] = (td*top/scale)[c - PRE + j]
+    float dr[POST + 1];   // dr[j] = td[c + j]
+    float sr[POST + 1];   // sr[j] = scale[c + j]
+#pragma unroll
+    for (int j = 1; j < SIZE; ++j) {
+        const int c = cs - PRE + j - 1;
+        float d = 0.0f, s = 1.0f, t = 0.0f;
+        if (c >= 0 && c < C) {
+            d = dp[(long)c * HW];
+            s = sp[(long)c * HW];
+            t = tp[(long)c * HW];
+        }
+        tr[j] = d * t / s;
+        if (j - 1 >= PRE) {       // channel >= cs: also feeds the centre rings
+            dr[j - PRE] = d;
+            sr[j - PRE] = s;
+        }
+    }
+#pragma unroll 4
+    for (int c = cs; c < ce; ++c) {
+#pragma unroll
+        for (int j = 0; j < SIZE - 1; ++j) tr[j] = tr[j + 1];
+#pragma unroll
+        for (int j = 0; j < POST; ++j) {
+            dr[j] = dr[j + 1];
+            sr[j] = sr[j + 1];
+        }
+        const int ch = c + POST;
+        float d = 0.0f, s = 1.0f, t = 0.0f;
+        if (ch < C) {
+            d = dp[(long)ch * HW];
+            s = sp[(long)ch * HW];
+            t = tp[(long)ch * HW];
+        }
+        tr[SIZE - 1] = d * t / s;
+        dr[POST] = d;
+        sr[POST] = s;
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < SIZE; ++j) acc += tr[j];
+        bp[(long)c * HW] = dr[0] * pow_neg_beta(sr[0], nbeta) - ratio * xp[(long)c * HW] * acc;
+    }
+}
+
+__global__ __launch_bounds__(kLrnThreads) void lrn_bwd_generic_kernel(
+    const float* __restrict__ x, const float* __restrict__ top, const float* __restrict__ scale,
+    const float* __restrict__ top_diff, float* __restrict__ bottom_diff, int C, int HW, int crun,
+    int size, float nbeta, float ratio) {
+    const int pre = size - (size + 1) / 2, post = size - pre - 1;
+    const int p = blockIdx.x * kLrnThreads + threadIdx.x;
+    if (p >= HW) return;
+    const long n = blockIdx.z;
+    const int cs = blockIdx.y * crun, ce = min(C, cs + crun);
+    const long base = n * C * (long)HW + p;
+    for (int c = cs; c < ce; ++c) {
+        float acc = 0.0f;
+        const int lo = max(0, c - pre), hi = min(C - 1, c + post);
+        for (int cc = lo; cc <= hi; ++cc) {
+            const long i = base + (long)cc * HW;
+            acc += top_diff[i] * top[i] / scale[i];
+        }
+        const long i = base + (long)c * HW;
+        bottom_diff[i] = top_diff[i] * pow_neg_beta(scale[i], nbeta) - ratio * x[i] * acc;
+    }
+}
+
+static int check_lrn(const char* what, long N, long C, long H, long W, int size) {
+    CGT_ARG_CHECK(N >= 0 && C >= 0 && H >= 0 && W >= 0, "%s: negative shape", what);
+    CGT_ARG_CHECK(size >= 1 && size <= C, "%s: need 1 <= size <= C, got size=%d C=%ld", what, size, C);
+    CGT_ARG_CHECK(H * W < (1L << 31) && C < (1L << 31) && N < 65536, "%s: shape too large", what);
+    return CGT_AMD_OK;
+}
+
+// channels per thread run: short enough to fill the chip, long enough that the
+// halo re-read (size-1 channels per run) stays small.
+static int pick_crun(long N, int C, int HW, int size) {
+    const long pix_blocks = cdiv(HW, kLrnThreads) * N;
+    int crun = C;
+    const int min_run = std::max(8 * size, 16);
+    while (crun > min_run && pix_blocks * cdiv(C, crun) < 2048) crun = (crun + 1) / 2;
+    return crun;
+}
+
+}  // namespace cgt_amd
+
+using namespace cgt_amd;
+
+CGT_API int cgt_amd_lrn_fwd_f32(const float* x, long N, long C, long H, long W, int size,
+                                double alpha, double beta, double k, float* top, float* scale,
+                                void* stream) {
+    if (N * C * H * W == 0 && N >= 0 && C >= 0 && H >= 0 && W >= 0 && size >= 1) return CGT_AMD_OK;
+    int rc = check_lrn("lrn_fwd", N, C, H, W, size);
+    if (rc) return rc;
+    CGT_ARG_CHECK(x && top && scale, "lrn_fwd: null pointer");
+    CGT_ARG_CHECK(k > 0, "lrn_fwd: k must be positive");
+    const int HW = (int)(H * W);
+    const int crun = pick_crun(N, (int)C, HW, size);
+    dim3 grid((unsigned)cdiv(HW, kLrnThreads), (unsigned)cdiv(C, crun), (unsigned)N), block(kLrnThreads);
+    hipStream_t st = as_stream(stream);
+    const float aos = (float)(alpha / size), nbeta = (float)(-beta), kc = (float)k;
+#define LRN_FWD_CASE(S)                                                                           \
+    case S:                                                                                       \
+        lrn_fwd_kernel<S><<<grid, block, 0, st>>>(x, top, scale, (int)C, HW, crun, aos, nbeta, kc); \
+        break;
+    switch (size) {
+        LRN_FWD_CASE(1) LRN_FWD_CASE(2) LRN_FWD_CASE(3) LRN_FWD_CASE(4) LRN_FWD_CASE(5)
+        LRN_FWD_CASE(6) LRN_FWD_CASE(7) LRN_FWD_CASE(8) LRN_FWD_CASE(9)
+        default:
+            lrn_fwd_generic_kernel<<<grid, block, 0, st>>>(x, top, scale, (int)C, HW, crun, size, aos, nbeta, kc);
+    }
+#undef LRN_FWD_CASE
+    CGT_LAUNCH_CHECK("lrn_fwd_kernel");
+    return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_lrn_bwd_f32(const float* x, const float* top, const float* scale,
+                                const float* top_diff, long N, long C, long H, long W, int size,
+                                double alpha, double beta, float* bottom_diff, void* stream) {
+    if (N * C * H * W == 0 && N >= 0 && C >= 0 && H >= 0 && W >= 0 && size >= 1) return CGT_AMD_OK;
+    int rc = check_lrn("lrn_bwd", N, C, H, W, size);
+    if (rc) return rc;
+    CGT_ARG_CHECK(x && top && scale && top_diff && bottom_diff, "lrn_bwd: null pointer");
+    const int HW = (int)(H * W);
+    const int crun = pick_crun(N, (int)C, HW, size);
+    dim3 grid((unsigned)cdiv(HW, kLrnThreads), (unsigned)cdiv(C, crun), (unsigned)N), block(kLrnThreads);
+    hipStream_t st = as_stream(stream);
+    const float nbeta = (float)(-beta), ratio = (float)(2. * alpha * beta / size);
+#define LRN_BWD_CASE(S)                                                                      \
+    case S:                                                                                  \
+        lrn_bwd_kernel<S><<<grid, block, 0, st>>>(x, top, scale, top_diff, bottom_diff, (int)C, \
+                                                  HW, crun, nbeta, ratio);                   \
+        break;
+    switch (size) {
+        LRN_BWD_CASE(1) LRN_BWD_CASE(2) LRN_BWD_CASE(3) LRN_BWD_CASE(4) LRN_BWD_CASE(5)
+        LRN_BWD_CASE(6) LRN_BWD_CASE(7) LRN_BWD_CASE(8) LRN_BWD_CASE(9)
+        default:
+            lrn_bwd_generic_kernel<<<grid, block, 0, st>>>(x, top, scale, top_diff, bottom_diff,
+                                                           (int)C, HW, crun, size, nbeta, ratio);
+    }
+#undef LRN_BWD_CASE
+    CGT_LAUNCH_CHECK("lrn_bwd_kernel");
+    return CGT_AMD_OK;
+}

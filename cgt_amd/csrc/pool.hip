@@ -1,0 +1,236 @@
+// Max pooling with argmax, and its pullback, for gfx950.  HBM-bound.
+//
+// Planes are independent, so the (n,c) axis is flattened.  A workgroup owns a
+// run of whole planes: it stages them into LDS as one flat, contiguous,
+// coalesced read (the run is contiguous in memory whatever H*W is), computes
+// the outputs from LDS, and writes them as one flat contiguous run.
+//
+// Forward: window scan in (h, w) order, strict '>', from -FLT_MAX; mask is the
+// in-plane index h*W + w.  Pullback: gather form of the reference's scatter --
+// each input cell visits the windows that cover it in ascending (ph, pw) and
+// adds top_diff where the mask names it, which reproduces the sequential add
+// order bit-for-bit without atomics.
+#include "common.h"
+#include <algorithm>
+#include <cfloat>
+
+namespace cgt_amd {
+
+struct PoolGeom {
+    int kh, kw, ph, pw, sh, sw;
+};
+
+constexpr int kPoolThreads = 256;
+
+// planes_per_wg planes per workgroup; LDS holds their inputs.
+__global__ __launch_bounds__(kPoolThreads) void max_pool_fwd_kernel(
+    PoolGeom g, const float* __restrict__ bottom, float* __restrict__ top, int* __restrict__ mask,
+    long nplanes, int H, int W, int PH, int PW, int planes_per_wg) {
+    extern __shared__ float tile[];
+    const long p0 = (long)blockIdx.x * planes_per_wg;
+    const long left = nplanes - p0;
+    const int np = left < planes_per_wg ? (int)left : planes_per_wg;
+    const int HW = H * W, PP = PH * PW;
+    const float* src = bottom + p0 * HW;
+    const int nin = np * HW;
+    for (int i = threadIdx.x; i < nin; i += kPoolThreads) tile[i] = src[i];
+    __syncthreads();
+
+    const int nout = np * PP;
+    float* tdst = top + p0 * PP;
+    int* mdst = mask + p0 * PP;
+    for (int o = threadIdx.x; o < nout; o += kPoolThreads) {
+        const int pl = o / PP, r = o - pl * PP;
+        const int y = r / PW, x = r - y * PW;
+        int hs = y * g.sh - g.ph, ws = x * g.sw - g.pw;
+        const int he = min(hs + g.kh, H), we = min(ws + g.kw, W);
+        hs = max(hs, 0);
+        ws = max(ws, 0);
+        const float* pt = tile + pl * HW;
+        float best = -FLT_MAX;
+        int arg = -1;
+        for (int h = hs; h < he; ++h)
+            for (int w = ws; w < we; ++w) {
+                const float v = pt[h * W + w];
+                if (v > best) {
+                    best = v;
+                    arg = h * W + w;
+                }
+            }
+        tdst[o] = best;
+        mdst[o] = arg;
+    }
+}
+
+// Plane too large for LDS: read through the cache hierarchy.
+__global__ __launch_bounds__(kPoolThreads) void max_pool_fwd_direct_kernel(
+    PoolGeom g, const float* __restrict__ bottom, float* __restrict__ top, int* __restrict__ mask,
+    long total, int H, int W, int PH, int PW) {
+    const long PP = (long)PH * PW;
+    for (long o = (long)blockIdx.x * blockDim.x + threadIdx.x; o < total;
+         o += (long)gridDim.x * blockDim.x) {
+        const long pl = o / PP;
+        const int r = (int)(o - pl * PP);
+        const int y = r / PW, x = r - y * PW;
+        int hs = y * g.sh - g.ph, ws = x * g.sw - g.pw;
+        const int he = min(hs + g.kh, H), we = min(ws + g.kw, W);
+        hs = max(hs, 0);
+        ws = max(ws, 0);
+        const float* pt = bottom + pl * H * W;
+        float best = -FLT_MAX;
+        int arg = -1;
+        for (int h = hs; h < he; ++h)
+            for (int w = ws; w < we; ++w) {
+                const float v = pt[h * W + w];
+                if (v > best) {
+                    best = v;
+                    arg = h * W + w;
+                }
+            }
+        top[o] = best;
+        mask[o] = arg;
+    }
+}
+
+__device__ __forceinline__ int floordiv(int a, int b) {  // b > 0
+    int q = a / b;
+    return (a % b != 0 && a < 0) ? q - 1 : q;
+}
+
+// LDS holds mask and top_diff of the workgroup's planes.
+__global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_kernel(
+    PoolGeom g, const int* __restrict__ mask, const float* __restrict__ top_diff,
+    float* __restrict__ bottom_diff, long nplanes, int H, int W, int PH, int PW,
+    int planes_per_wg) {
+    extern __shared__ float tile[];
+    const long p0 = (long)blockIdx.x * planes_per_wg;
+    const long left = nplanes - p0;
+    const int np = left < planes_per_wg ? (int)left : planes_per_wg;
+    const int HW = H * W, PP = PH * PW;
+    const int nout = np * PP;
+    float* td = tile;
+    int* mk = reinterpret_cast<int*>(tile + planes_per_wg * PP);
+    for (int i = threadIdx.x; i < nout; i += kPoolThreads) {
+        td[i] = top_diff[p0 * PP + i];
+        mk[i] = mask[p0 * PP + i];
+    }
+    __syncthreads();
+
+    const int nin = np * HW;
+    float* dst = bottom_diff + p0 * HW;
+    for (int i = threadIdx.x; i < nin; i += kPoolThreads) {
+        const int pl = i / HW, cell = i - pl * HW;
+        const int h = cell / W, w = cell - h * W;
+        // windows covering (h, w): ph*sh - pad <= h < ph*sh - pad + kh
+        const int y0 = max(0, floordiv(h + g.ph - g.kh, g.sh) + 1), y1 = min(PH - 1, (h + g.ph) / g.sh);
+        const int x0 = max(0, floordiv(w + g.pw - g.kw, g.sw) + 1), x1 = min(PW - 1, (w + g.pw) / g.sw);
+        float acc = 0.0f;
+        for (int y = y0; y <= y1; ++y)
+            for (int x = x0; x <= x1; ++x) {
+                const int o = pl * PP + y * PW + x;
+                if (mk[o] == cell) acc += td[o];
+            }
+        dst[i] = acc;
+    }
+}
+
+__global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_direct_kernel(
+    PoolGeom g, const int* __restrict__ mask, const float* __restrict__ top_diff,
+    float* __restrict__ bottom_diff, long total, int H, int W, int PH, int PW) {
+    const long HW = (long)H * W, PP = (long)PH * PW;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (long)gridDim.x * blockDim.x) {
+        const long pl = i / HW;
+        const int cell = (int)(i - pl * HW);
+        const int h = cell / W, w = cell - h * W;
+        const int y0 = max(0, floordiv(h + g.ph - g.kh, g.sh) + 1), y1 = min(PH - 1, (h + g.ph) / g.sh);
+        const int x0 = max(0, floordiv(w + g.pw - g.kw, g.sw) + 1), x1 = min(PW - 1, (w + g.pw) / g.sw);
+        float acc = 0.0f;
+        for (int y = y0; y <= y1; ++y)
+            for (int x = x0; x <= x1; ++x) {
+                const long o = pl * PP + y * PW + x;
+                if (mask[o] == cell) acc += top_diff[o];
+            }
+        bottom_diff[i] = acc;
+    }
+}
+
+static int check_pool(const char* what, long N, long C, long H, long W, int kh, int kw, int ph,
+                      int pw, int sh, int sw, long PH, long PW) {
+    CGT_ARG_CHECK(N >= 0 && C >= 0 && H >= 0 && W >= 0 && PH >= 0 && PW >= 0, "%s: negative shape", what);
+    CGT_ARG_CHECK(kh > 0 && kw > 0 && sh > 0 && sw > 0 && ph >= 0 && pw >= 0,
+                  "%s: bad geometry k=(%d,%d) p=(%d,%d) s=(%d,%d)", what, kh, kw, ph, pw, sh, sw);
+    CGT_ARG_CHECK(H * W < (1L << 31) && PH * PW < (1L << 31), "%s: plane too large", what);
+    // every window must start inside the padded image, as the op's shape rule guarantees
+    CGT_ARG_CHECK(PH == 0 || (PH - 1) * sh - ph < H, "%s: PH=%ld does not fit H=%ld", what, PH, H);
+    CGT_ARG_CHECK(PW == 0 || (PW - 1) * sw - pw < W, "%s: PW=%ld does not fit W=%ld", what, PW, W);
+    return CGT_AMD_OK;
+}
+
+}  // namespace cgt_amd
+
+using namespace cgt_amd;
+
+CGT_API long cgt_amd_pool_outsize(long H, int k, int pad, int stride) {
+    if (stride <= 0) return 0;
+    long num = H + 2L * pad - k;
+    if (num <= 0) return 0;
+    return (num + stride - 1) / stride;
+}
+
+CGT_API int cgt_amd_max_pool_f32(const float* bottom, long N, long C, long H, long W, int kh,
+                                 int kw, int ph, int pw, int sh, int sw, long PH, long PW,
+                                 float* top, int* mask, void* stream) {
+    int rc = check_pool("max_pool", N, C, H, W, kh, kw, ph, pw, sh, sw, PH, PW);
+    if (rc) return rc;
+    const long nplanes = N * C;
+    if (nplanes * PH * PW == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(bottom && top && mask, "max_pool: null pointer");
+    PoolGeom g{kh, kw, ph, pw, sh, sw};
+    hipStream_t st = as_stream(stream);
+    const long plane_bytes = H * W * (long)sizeof(float);
+    if (plane_bytes <= 48 * 1024) {
+        int ppw = (int)std::max(1L, (16 * 1024) / std::max(1L, plane_bytes));
+        const long blocks = cdiv(nplanes, ppw);
+        max_pool_fwd_kernel<<<dim3((unsigned)blocks), dim3(kPoolThreads), (size_t)ppw * plane_bytes, st>>>(
+            g, bottom, top, mask, nplanes, (int)H, (int)W, (int)PH, (int)PW, ppw);
+        CGT_LAUNCH_CHECK("max_pool_fwd_kernel");
+    } else {
+        const long total = nplanes * PH * PW;
+        long blocks = std::min(cdiv(total, (long)kPoolThreads), 1L << 20);
+        max_pool_fwd_direct_kernel<<<dim3((unsigned)blocks), dim3(kPoolThreads), 0, st>>>(
+            g, bottom, top, mask, total, (int)H, (int)W, (int)PH, (int)PW);
+        CGT_LAUNCH_CHECK("max_pool_fwd_direct_kernel");
+    }
+    return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_max_pool_pullback_f32(const int* mask, const float* top_diff, long N, long C,
+                                          long H, long W, int kh, int kw, int ph, int pw, int sh,
+                                          int sw, long PH, long PW, float* bottom_diff,
+                                          void* stream) {
+    int rc = check_pool("max_pool_pullback", N, C, H, W, kh, kw, ph, pw, sh, sw, PH, PW);
+    if (rc) return rc;
+    const long nplanes = N * C;
+    if (nplanes * H * W == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(bottom_diff, "max_pool_pullback: null pointer");
+    hipStream_t st = as_stream(stream);
+    if (PH * PW == 0) return cgt_amd_fill_u32(bottom_diff, 0u, nplanes * H * W, stream);
+    CGT_ARG_CHECK(mask && top_diff, "max_pool_pullback: null pointer");
+    PoolGeom g{kh, kw, ph, pw, sh, sw};
+    const long out_bytes = PH * PW * 2 * (long)sizeof(float);  // top_diff + mask per plane
+    if (out_bytes <= 48 * 1024) {
+        int ppw = (int)std::max(1L, (16 * 1024) / out_bytes);
+        const long blocks = cdiv(nplanes, ppw);
+        max_pool_bwd_kernel<<<dim3((unsigned)blocks), dim3(kPoolThreads), (size_t)ppw * out_bytes, st>>>(
+            g, mask, top_diff, bottom_diff, nplanes, (int)H, (int)W, (int)PH, (int)PW, ppw);
+        CGT_LAUNCH_CHECK("max_pool_bwd_kernel");
+    } else {
+        const long total = nplanes * H * W;
+        long blocks = std::min(cdiv(total, (long)kPoolThreads), 1L << 20);
+        max_pool_bwd_direct_kernel<<<dim3((unsigned)blocks), dim3(kPoolThreads), 0, st>>>(
+            g, mask, top_diff, bottom_diff, total, (int)H, (int)W, (int)PH, (int)PW);
+        CGT_LAUNCH_CHECK("max_pool_bwd_direct_kernel");
+    }
+    return CGT_AMD_OK;
+}

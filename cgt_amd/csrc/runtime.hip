@@ -1,0 +1,150 @@
+// Runtime entry points: device memory for cgtGPU arrays, copies, streams,
+// events, error reporting.
+#include "common.h"
+#include <cstring>
+
+namespace cgt_amd {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+void clear_error() { g_err[0] = 0; }
+
+__global__ void fill_u32_kernel(unsigned int* __restrict__ dst, unsigned int v, long n) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    long stride = (long)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) dst[i] = v;
+}
+
+}  // namespace cgt_amd
+
+using namespace cgt_amd;
+
+CGT_API int cgt_amd_version(void) { return 100; }
+
+CGT_API const char* cgt_amd_last_error(void) { return g_err; }
+
+CGT_API int cgt_amd_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return n;
+}
+
+CGT_API int cgt_amd_device_name(char* buf, int buflen) {
+    CGT_ARG_CHECK(buf && buflen > 0, "device_name: bad buffer");
+    int dev = 0;
+    CGT_HIP_TRY(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    CGT_HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    snprintf(buf, buflen, "%s %s CUs=%d clock=%dMHz", prop.gcnArchName, prop.name,
+             prop.multiProcessorCount, prop.clockRate / 1000);
+    return CGT_AMD_OK;
+}
+
+CGT_API void* cgt_amd_alloc(long nbytes) {
+    if (nbytes < 0) {
+        set_error("alloc: negative size %ld", nbytes);
+        return nullptr;
+    }
+    void* p = nullptr;
+    // A zero-byte array still needs a distinct non-null pointer.
+    hipError_t e = hipMalloc(&p, nbytes > 0 ? (size_t)nbytes : 16);
+    if (e != hipSuccess) {
+        set_error("hipMalloc(%ld) failed: %s", nbytes, hipGetErrorString(e));
+        return nullptr;
+    }
+    return p;
+}
+
+CGT_API int cgt_amd_free(void* ptr) {
+    if (!ptr) return CGT_AMD_OK;
+    CGT_HIP_TRY(hipFree(ptr));
+    return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_memcpy(int dest_devtype, int src_devtype, void* dest, const void* src,
+                           long nbytes) {
+    CGT_ARG_CHECK(nbytes >= 0, "memcpy: negative size");
+    if (nbytes == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(dest && src, "memcpy: null pointer");
+    if (dest_devtype == CGT_AMD_CPU && src_devtype == CGT_AMD_CPU) {
+        memcpy(dest, src, (size_t)nbytes);
+        return CGT_AMD_OK;
+    }
+    hipMemcpyKind kind;
+    if (src_devtype == CGT_AMD_CPU && dest_devtype == CGT_AMD_GPU) kind = hipMemcpyHostToDevice;
+    else if (src_devtype == CGT_AMD_GPU && dest_devtype == CGT_AMD_CPU) kind = hipMemcpyDeviceToHost;
+    else if (src_devtype == CGT_AMD_GPU && dest_devtype == CGT_AMD_GPU) kind = hipMemcpyDeviceToDevice;
+    else {
+        set_error("memcpy: invalid devtypes %d <- %d", dest_devtype, src_devtype);
+        return CGT_AMD_ERR_ARG;
+    }
+    CGT_HIP_TRY(hipMemcpy(dest, src, (size_t)nbytes, kind));
+    return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_fill_u32(void* dst, unsigned int value, long count, void* stream) {
+    CGT_ARG_CHECK(count >= 0, "fill: negative count");
+    if (count == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(dst, "fill: null pointer");
+    long blocks = cdiv(count, 256);
+    if (blocks > 4096) blocks = 4096;
+    fill_u32_kernel<<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(
+        static_cast<unsigned int*>(dst), value, count);
+    CGT_LAUNCH_CHECK("fill_u32");
+    return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_synchronize(void* stream) {
+    if (stream) CGT_HIP_TRY(hipStreamSynchronize(as_stream(stream)));
+    else CGT_HIP_TRY(hipDeviceSynchronize());
+    return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_stream_create(void** stream) {
+    CGT_ARG_CHECK(stream, "stream_create: null");
+    hipStream_t s;
+    CGT_HIP_TRY(hipStreamCreate(&s));  // default priority only
+    *stream = s;
+    return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_stream_destroy(void* stream) {
+    if (stream) CGT_HIP_TRY(hipStreamDestroy(as_stream(stream)));
+    return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_event_create(void** event) {
+    CGT_ARG_CHECK(event, "event_create: null");
+    hipEvent_t e;
+    CGT_HIP_TRY(hipEventCreate(&e));
+    *event = e;
+    return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_event_destroy(void* event) {
+    if (event) CGT_HIP_TRY(hipEventDestroy(static_cast<hipEvent_t>(event)));
+    return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_event_record(void* event, void* stream) {
+    CGT_ARG_CHECK(event, "event_record: null");
+    CGT_HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(event), as_stream(stream)));
+    return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_event_elapsed_ms(void* start, void* stop, float* ms) {
+    CGT_ARG_CHECK(start && stop && ms, "event_elapsed: null");
+    CGT_HIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
+    CGT_HIP_TRY(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+    return CGT_AMD_OK;
+}

@@ -1,0 +1,198 @@
+"""Direct calls of the C ABI on device arrays -- one function per hot-path op.
+
+These apply the same shape rules as the reference Ops (cited per function) and
+hand raw pointers to libcgt_amd.so.  Outputs may be passed in (`out=`) to be
+reused across calls, as the reference interpreter reuses them
+(src/execution.cpp:260-263); every kernel overwrites its output fully.
+"""
+import ctypes
+
+import numpy as np
+
+from . import capi
+from .gpuarray import GpuArray, empty
+
+
+def _geom(kernel, pad, stride):
+    (kh, kw), (ph, pw), (sh, sw) = kernel, pad, stride
+    return [int(v) for v in (kh, kw, ph, pw, sh, sw)]
+
+
+def _out(out, shape, dtype=np.float32):
+    if out is None:
+        return empty(shape, dtype)
+    if out.shape != tuple(shape) or out.dtype != np.dtype(dtype):
+        raise ValueError("out has shape %s dtype %s, expected %s %s" % (out.shape, out.dtype, tuple(shape), dtype))
+    return out
+
+
+def _f32(*arrays):
+    for a in arrays:
+        if a.dtype != np.float32:
+            raise TypeError("expected float32 device array, got %s" % a.dtype)
+
+
+def conv_outsize(H, k, pad, stride):
+    """(H + 2*pad - k) // stride + 1 (reference cgt/nn_ops/im2col.py:39-40)."""
+    return (H + 2 * pad - k) // stride + 1
+
+
+def pool_outsize(H, k, pad, stride):
+    """ceil((H + 2*pad - k) / stride), no +1 (reference cgt/nn_ops/max_pool_2d.py:40-41)."""
+    return int(capi.lib().cgt_amd_pool_outsize(H, k, pad, stride))
+
+
+def im2col(x, kernel, pad, stride, out=None, stream=None):
+    """Im2Col op (reference cgt/nn_ops/im2col.py:25-62): [B,C,H,W] -> [B,m,n,C*kh*kw]."""
+    _f32(x)
+    B, C, H, W = x.shape
+    g = _geom(kernel, pad, stride)
+    m, n = conv_outsize(H, g[0], g[2], g[4]), conv_outsize(W, g[1], g[3], g[5])
+    col = _out(out, (B, m, n, C * g[0] * g[1]))
+    capi.check(capi.lib().cgt_amd_im2col_f32(x.ptr, B, C, H, W, *g, col.ptr, stream))
+    return col
+
+
+def col2im(col, imshape, kernel, pad, stride, out=None, stream=None):
+    """Col2Im op (reference cgt/nn_ops/im2col.py:64-93): adjoint of im2col."""
+    _f32(col)
+    B, C, H, W = (int(s) for s in imshape)
+    g = _geom(kernel, pad, stride)
+    m, n = conv_outsize(H, g[0], g[2], g[4]), conv_outsize(W, g[1], g[3], g[5])
+    if col.shape != (B, m, n, C * g[0] * g[1]):
+        raise ValueError("col has shape %s, expected %s" % (col.shape, (B, m, n, C * g[0] * g[1])))
+    im = _out(out, (B, C, H, W))
+    capi.check(capi.lib().cgt_amd_col2im_f32(col.ptr, B, C, H, W, *g, im.ptr, stream))
+    return im
+
+
+def max_pool(x, kernel, pad, stride, out=None, stream=None):
+    """MaxPool op (reference cgt/nn_ops/max_pool_2d.py:22-53): returns (pool, int32 mask)."""
+    _f32(x)
+    N, C, H, W = x.shape
+    g = _geom(kernel, pad, stride)
+    PH, PW = pool_outsize(H, g[0], g[2], g[4]), pool_outsize(W, g[1], g[3], g[5])
+    top = _out(out[0] if out else None, (N, C, PH, PW))
+    mask = _out(out[1] if out else None, (N, C, PH, PW), np.int32)
+    capi.check(capi.lib().cgt_amd_max_pool_f32(x.ptr, N, C, H, W, *g, PH, PW, top.ptr, mask.ptr, stream))
+    return top, mask
+
+
+def max_pool_pullback(xshape, mask, gtop, kernel, pad, stride, out=None, stream=None):
+    """MaxPoolPullback op (reference cgt/nn_ops/max_pool_2d.py:55-72)."""
+    _f32(gtop)
+    if mask.dtype != np.int32:
+        raise TypeError("mask must be int32")
+    N, C, H, W = (int(s) for s in xshape)
+    g = _geom(kernel, pad, stride)
+    PH, PW = mask.shape[2:]
+    if mask.shape != gtop.shape or mask.shape[:2] != (N, C):
+        raise ValueError("mask %s / gtop %s do not match x %s" % (mask.shape, gtop.shape, xshape))
+    gb = _out(out, (N, C, H, W))
+    capi.check(capi.lib().cgt_amd_max_pool_pullback_f32(mask.ptr, gtop.ptr, N, C, H, W, *g, PH, PW,
+                                                        gb.ptr, stream))
+    return gb
+
+
+def lrn_fwd(x, size, alpha, beta, k=1.0, out=None, stream=None):
+    """CrossChannelLRNForward op (reference cgt/nn_ops/cross_channel_lrn.py:15-63):
+    returns (top, scale).  k=1 is the reference; other k is an extension."""
+    _f32(x)
+    N, C, H, W = x.shape
+    top = _out(out[0] if out else None, x.shape)
+    scale = _out(out[1] if out else None, x.shape)
+    capi.check(capi.lib().cgt_amd_lrn_fwd_f32(x.ptr, N, C, H, W, int(size), float(alpha), float(beta),
+                                              float(k), top.ptr, scale.ptr, stream))
+    return top, scale
+
+
+def lrn_bwd(x, top, scale, gtop, size, alpha, beta, out=None, stream=None):
+    """CrossChannelLRNBackward op (reference cgt/nn_ops/cross_channel_lrn.py:65-104)."""
+    _f32(x, top, scale, gtop)
+    N, C, H, W = x.shape
+    for a in (top, scale, gtop):
+        if a.shape != x.shape:
+            raise ValueError("LRN backward operands must share x's shape")
+    gb = _out(out, x.shape)
+    capi.check(capi.lib().cgt_amd_lrn_bwd_f32(x.ptr, top.ptr, scale.ptr, gtop.ptr, N, C, H, W, int(size),
+                                              float(alpha), float(beta), gb.ptr, stream))
+    return gb
+
+
+def mul22(A, B, tA=False, tB=False, out=None, stream=None):
+    """Mul22 op (reference cgt/core.py:2129-2229): C = op(A) . op(B); M, N, K and
+    leading dimensions as in its op body (2196-2205)."""
+    _f32(A, B)
+    if A.ndim != 2 or B.ndim != 2:
+        raise ValueError("Mul22 takes matrices")
+    M = A.shape[1] if tA else A.shape[0]
+    K = A.shape[0] if tA else A.shape[1]
+    N = B.shape[0] if tB else B.shape[1]
+    Kb = B.shape[1] if tB else B.shape[0]
+    if K != Kb:
+        raise ValueError("shape mismatch at matrix-matrix multiplication: %s %s" % (A.shape, B.shape))
+    C = _out(out, (M, N))
+    capi.check(capi.lib().cgt_amd_sgemm(int(tA), int(tB), M, N, K, A.ptr, A.shape[1], B.ptr, B.shape[1],
+                                        C.ptr, N, stream))
+    return C
+
+
+def batched_mul22(A, B, tA=False, tB=False, out=None, stream=None):
+    """BatchedMul22 op (reference cgt/core.py:2231-2288)."""
+    _f32(A, B)
+    if A.ndim != 3 or B.ndim != 3 or A.shape[0] != B.shape[0]:
+        raise ValueError("BatchedMul22 takes [P,.,.] arrays with equal P")
+    P = A.shape[0]
+    M = A.shape[2] if tA else A.shape[1]
+    K = A.shape[1] if tA else A.shape[2]
+    N = B.shape[1] if tB else B.shape[2]
+    Kb = B.shape[2] if tB else B.shape[1]
+    if K != Kb:
+        raise ValueError("shape mismatch at batched matrix multiplication: %s %s" % (A.shape, B.shape))
+    C = _out(out, (P, M, N))
+    capi.check(capi.lib().cgt_amd_sgemm_batched(int(tA), int(tB), P, M, N, K,
+                                                A.ptr, A.shape[2], A.shape[1] * A.shape[2],
+                                                B.ptr, B.shape[2], B.shape[1] * B.shape[2],
+                                                C.ptr, N, M * N, stream))
+    return C
+
+
+def transpose4(x, axes, out=None, stream=None):
+    """Transpose op for 4-d arrays (reference cgt/core.py:1559-1594)."""
+    _f32(x)
+    axes = tuple(int(a) for a in axes)
+    res = _out(out, tuple(x.shape[a] for a in axes))
+    shp = (ctypes.c_long * 4)(*x.shape)
+    ax = (ctypes.c_int * 4)(*axes)
+    capi.check(capi.lib().cgt_amd_transpose4_f32(x.ptr, shp, ax, res.ptr, stream))
+    return res
+
+
+def conv2d(x, f, pad=(0, 0), stride=(1, 1), stream=None, keep=None):
+    """conv2d forward as the reference composes it on its CPU path
+    (cgt/nn.py:95-100): im2col -> [B*m*n, Z] -> Mul22(False, True) with the
+    filters as [L, Z] -> [B, m, n, L] -> Transpose{0,3,1,2}.
+    `keep`, if a dict, receives the column buffer for the backward pass."""
+    L, K, r, c = f.shape
+    col = im2col(x, (r, c), pad, stride, stream=stream)
+    B, m, n, Z = col.shape
+    y = mul22(col.reshape(B * m * n, Z), f.reshape(L, Z), False, True, stream=stream)
+    if keep is not None:
+        keep["col"] = col
+    return transpose4(y.reshape(B, m, n, L), (0, 3, 1, 2), stream=stream)
+
+
+def conv2d_pullback(x, f, gy, pad=(0, 0), stride=(1, 1), col=None, stream=None):
+    """Gradients (gx, gf) of conv2d, following the graph the reference's autodiff
+    derives: Transpose{0,2,3,1} of gy (cgt/core.py:1569-1570); for Mul22(F,T)
+    (core.py:2160-2162) gcol = Mul22(F,F)[gc, f_LZ] -> Col2Im (im2col.py:34-35)
+    and gf = Mul22(T,F)[gc, col]."""
+    L, K, r, c = f.shape
+    if col is None:
+        col = im2col(x, (r, c), pad, stride, stream=stream)
+    B, m, n, Z = col.shape
+    gc = transpose4(gy, (0, 2, 3, 1), stream=stream).reshape(B * m * n, L)
+    gcol = mul22(gc, f.reshape(L, Z), False, False, stream=stream)
+    gx = col2im(gcol.reshape(B, m, n, Z), x.shape, (r, c), pad, stride, stream=stream)
+    gf = mul22(gc, col.reshape(B * m * n, Z), True, False, stream=stream).reshape(f.shape)
+    return gx, gf

@@ -1,0 +1,181 @@
+/*
+ * cgt_amd -- C ABI of the MI355X (gfx950) implementation of CGT's native CNN
+ * hot path: im2col / col2im, the Mul22 / BatchedMul22 fp32 GEMM, max-pool
+ * forward / pullback with argmax, cross-channel LRN forward / backward.
+ *
+ * These are the device-side launchers a CGT op body calls after it has
+ * unpacked its cgtArray arguments, the role `launchker_$function(raw
+ * pointers, ints...)` plays in the reference's two-translation-unit GPU ops
+ * (cgt/nn_ops/cross_channel_lrn.py:24-55).  Plain pointers and sizes only.
+ *
+ * Conventions
+ *   - every data pointer is DEVICE memory, fp32 contiguous row-major unless
+ *     noted; argmax masks are int32; sizes are `long` as in cgtArray::shape().
+ *   - `stream` is a hipStream_t passed as void*; NULL is the default stream.
+ *     Launches are asynchronous; nothing here synchronises.
+ *   - return value: CGT_AMD_OK or an error code; cgt_amd_last_error() gives
+ *     the message for the calling thread.  (The reference's CUDA_CHECK only
+ *     prints, include/cgt_cuda.h:11-21; a status is returned here instead.)
+ *   - outputs are fully overwritten on every call: the interpreter reuses
+ *     output buffers between calls without clearing them
+ *     (src/execution.cpp:260-263).
+ */
+#ifndef CGT_AMD_H
+#define CGT_AMD_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CGT_AMD_OK 0
+#define CGT_AMD_ERR_ARG 1     /* bad shape / geometry / null pointer      */
+#define CGT_AMD_ERR_HIP 2     /* a HIP runtime call failed                */
+#define CGT_AMD_ERR_NOMEM 3   /* workspace allocation failed              */
+#define CGT_AMD_ERR_NODEVICE 4
+
+/* devtype values of cgt_amd_memcpy, numerically equal to the reference's
+ * cgtDevtype { cgtCPU, cgtGPU } (include/cgt_common.h:68-71). */
+#define CGT_AMD_CPU 0
+#define CGT_AMD_GPU 1
+
+/* ---------------------------------------------------------------- runtime */
+
+/* Library version (major*100 + minor). */
+int cgt_amd_version(void);
+
+/* Message of the last error on the calling thread ("" if none). */
+const char *cgt_amd_last_error(void);
+
+/* Number of visible HIP devices (0 if none / no driver); never fails. */
+int cgt_amd_device_count(void);
+
+/* Device name of the current device, e.g. "gfx950..." into buf. */
+int cgt_amd_device_name(char *buf, int buflen);
+
+/* Device allocation for cgtGPU arrays.  Replaces the cudaMalloc / cudaFree
+ * branches of cgt_alloc / cgt_free (src/cgt_common.cpp:110-136).
+ * cgt_amd_alloc returns NULL on failure. */
+void *cgt_amd_alloc(long nbytes);
+int cgt_amd_free(void *ptr);
+
+/* Synchronous copy between host and device memory.  Replaces the cudaMemcpy
+ * branch of cgt_memcpy (src/cgt_common.cpp:138-153). */
+int cgt_amd_memcpy(int dest_devtype, int src_devtype, void *dest, const void *src, long nbytes);
+
+/* Asynchronous fill of `count` 32-bit words with `value` (a fill kernel, safe
+ * to capture in a HIP graph). */
+int cgt_amd_fill_u32(void *dst, unsigned int value, long count, void *stream);
+
+/* Block the host until `stream` (NULL: the whole device) has drained. */
+int cgt_amd_synchronize(void *stream);
+
+/* Stream and event helpers so a host without its own HIP binding can time
+ * launches on the stream they were issued to. */
+int cgt_amd_stream_create(void **stream);
+int cgt_amd_stream_destroy(void *stream);
+int cgt_amd_event_create(void **event);
+int cgt_amd_event_destroy(void *event);
+int cgt_amd_event_record(void *event, void *stream);
+int cgt_amd_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for stop */
+
+/* ---------------------------------------------------------------- im2col / col2im */
+
+/* Patch extraction.  im [B,C,H,W] -> col [B,m,n,Z], Z = C*kh*kw ordered
+ * (channel, kernel row, kernel col), m = (H+2*ph-kh)/sh + 1, n likewise;
+ * taps outside the image are 0.  Bit-exact copy.
+ * Replaces im2col_cpu (include/im2col.h:6-28) and the per-image loop of the
+ * Im2Col op body (cgt/nn_ops/im2col.py:50-61). */
+int cgt_amd_im2col_f32(const float *im, long B, long C, long H, long W,
+                       int kh, int kw, int ph, int pw, int sh, int sw,
+                       float *col, void *stream);
+
+/* Adjoint of im2col.  col [B,m,n,Z] -> im [B,C,H,W]; every pixel is the sum of
+ * its taps taken in ascending Z order starting from +0, which is the order
+ * the reference's sequential loop produces, so results are bit-identical.
+ * Replaces col2im_cpu (include/im2col.h:30-50) and the Col2Im op body
+ * (cgt/nn_ops/im2col.py:80-92). */
+int cgt_amd_col2im_f32(const float *col, long B, long C, long H, long W,
+                       int kh, int kw, int ph, int pw, int sh, int sw,
+                       float *im, void *stream);
+
+/* ---------------------------------------------------------------- max pooling */
+
+/* Pooled extent of the MaxPool op: ceil((H + 2*pad - k) / stride), no "+1"
+ * (cgt/nn_ops/max_pool_2d.py:40-41).  Returns 0 when the window does not fit. */
+long cgt_amd_pool_outsize(long H, int k, int pad, int stride);
+
+/* Max pooling with argmax.  bottom [N,C,H,W] -> top, mask [N,C,PH,PW].
+ * Window rows/cols outside the image are skipped; the first maximum in
+ * (h, w) scan order wins (strict >, starting from -FLT_MAX); mask holds
+ * h*W + w within the (n,c) plane, or -1 if no cell exceeded -FLT_MAX.
+ * Replaces max_pool<float> (include/pooling.h:24-71). */
+int cgt_amd_max_pool_f32(const float *bottom, long N, long C, long H, long W,
+                         int kh, int kw, int ph, int pw, int sh, int sw,
+                         long PH, long PW, float *top, int *mask, void *stream);
+
+/* Pool pullback.  bottom_diff [N,C,H,W] = 0, then += top_diff at the cell each
+ * mask entry names; cells named by several windows add in ascending (ph, pw)
+ * order, bit-identical to the reference's sequential loop.  `mask` must be the
+ * output of cgt_amd_max_pool_f32 for the same geometry (each entry lies inside
+ * its own window); entries of -1 contribute nothing.
+ * Replaces max_pool_pullback<float> (include/pooling.h:73-106). */
+int cgt_amd_max_pool_pullback_f32(const int *mask, const float *top_diff,
+                                  long N, long C, long H, long W,
+                                  int kh, int kw, int ph, int pw, int sh, int sw,
+                                  long PH, long PW, float *bottom_diff, void *stream);
+
+/* ---------------------------------------------------------------- cross-channel LRN */
+
+/* scale[n,c,h,w] = k + (alpha/size) * sum_{c' in [c-pre, c+post]} x^2 with
+ * pre = (size-1)/2, post = size-pre-1, window clipped to [0,C);
+ * top = x * scale^(-beta).  k = 1 is the reference (it has no k parameter).
+ * Requires 1 <= size <= C, as the reference kernel does.
+ * Replaces LRNFillScale + LRNComputeOutput (include/lrn.cuh:3-52) and
+ * launchker of CrossChannelLRNForward (cgt/nn_ops/cross_channel_lrn.py:27-39). */
+int cgt_amd_lrn_fwd_f32(const float *x, long N, long C, long H, long W,
+                        int size, double alpha, double beta, double k,
+                        float *top, float *scale, void *stream);
+
+/* bottom_diff = top_diff * scale^(-beta)
+ *             - (2*alpha*beta/size) * x * sum_{c' in [c-pre', c+post']} top_diff*top/scale
+ * with pre' = size-(size+1)/2, post' = size-pre'-1.
+ * Replaces LRNComputeDiff (include/lrn.cuh:54-114) and launchker of
+ * CrossChannelLRNBackward (cgt/nn_ops/cross_channel_lrn.py:72-84). */
+int cgt_amd_lrn_bwd_f32(const float *x, const float *top, const float *scale,
+                        const float *top_diff, long N, long C, long H, long W,
+                        int size, double alpha, double beta,
+                        float *bottom_diff, void *stream);
+
+/* ---------------------------------------------------------------- GEMM */
+
+/* Row-major C[M,N] = op(A) . op(B), alpha = 1, beta = 0, true fp32 (MFMA
+ * v_mfma_f32_32x32x2_f32, no reduced-precision inputs).  tA/tB select the
+ * transposed operand; lda/ldb/ldc are the stored row lengths.
+ * Replaces the cblas_sgemm / cublasSgemm_v2 call of the Mul22 op body
+ * (cgt/core.py:2194-2224).  May use a split-K workspace owned by the library
+ * (one per stream); the reduction order is fixed, so results are
+ * deterministic. */
+int cgt_amd_sgemm(int tA, int tB, long M, long N, long K,
+                  const float *A, long lda, const float *B, long ldb,
+                  float *C, long ldc, void *stream);
+
+/* P independent products at A + p*strideA, B + p*strideB, C + p*strideC.
+ * Replaces the cblas_sgemm loop of BatchedMul22 (cgt/core.py:2272-2285);
+ * the reference has no GPU implementation of it. */
+int cgt_amd_sgemm_batched(int tA, int tB, long P, long M, long N, long K,
+                          const float *A, long lda, long strideA,
+                          const float *B, long ldb, long strideB,
+                          float *C, long ldc, long strideC, void *stream);
+
+/* ---------------------------------------------------------------- conv glue */
+
+/* out[i0,i1,i2,i3] = in[...] with out.shape[d] = in.shape[axes[d]].
+ * Replaces the Transpose op's CPU loop (cgt/core.py:1578-1594), which conv2d
+ * applies as {0,3,1,2} after the GEMM and its pullback as {0,2,3,1}. */
+int cgt_amd_transpose4_f32(const float *in, const long *inshape, const int *axes,
+                           float *out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CGT_AMD_H */

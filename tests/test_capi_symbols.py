@@ -1,0 +1,57 @@
+"""The C-ABI library loads and exports every symbol include/cgt_amd.h declares
+(no compute calls: this runs without a GPU)."""
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "cgt_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cgt_amd_\w+)\s*\(", text)))
+
+
+def test_header_declares_the_hot_path():
+    syms = declared_symbols()
+    for need in ["cgt_amd_im2col_f32", "cgt_amd_col2im_f32", "cgt_amd_max_pool_f32",
+                 "cgt_amd_max_pool_pullback_f32", "cgt_amd_lrn_fwd_f32", "cgt_amd_lrn_bwd_f32",
+                 "cgt_amd_sgemm", "cgt_amd_sgemm_batched", "cgt_amd_transpose4_f32",
+                 "cgt_amd_alloc", "cgt_amd_free", "cgt_amd_memcpy"]:
+        assert need in syms
+
+
+def test_library_exports_every_declared_symbol():
+    from cgt_amd import capi
+    if not os.path.exists(capi.libpath()):
+        pytest.fail("libcgt_amd.so is not built: run `python -m cgt_amd.build`")
+    handle = capi.lib()
+    syms = declared_symbols()
+    assert sorted(capi.PROTOTYPES) == syms, "capi.PROTOTYPES and include/cgt_amd.h disagree"
+    for name in syms:
+        assert getattr(handle, name) is not None
+
+
+def test_no_compute_needed_for_host_only_entry_points():
+    from cgt_amd import capi
+    lib = capi.lib()
+    assert lib.cgt_amd_version() >= 100
+    assert lib.cgt_amd_pool_outsize(28, 2, 0, 2) == 13
+    assert lib.cgt_amd_pool_outsize(55, 3, 0, 2) == 26
+    assert lib.cgt_amd_pool_outsize(5, 4, 0, 1) == 1
+    assert lib.cgt_amd_pool_outsize(2, 3, 0, 1) == 0
+    assert capi.device_count() >= 0
+
+
+def test_argument_errors_are_reported_not_fatal():
+    # argument validation happens on the host before any launch
+    from cgt_amd import capi
+    lib = capi.lib()
+    rc = lib.cgt_amd_im2col_f32(None, 1, 1, 4, 4, 0, 3, 0, 0, 1, 1, None, None)
+    assert rc == 1 and "geometry" in capi.last_error()
+    rc = lib.cgt_amd_lrn_fwd_f32(None, 1, 3, 2, 2, 5, 1e-4, 0.75, 1.0, None, None, None)
+    assert rc == 1 and "size" in capi.last_error()
+    rc = lib.cgt_amd_sgemm(0, 0, 4, 4, 4, None, 2, None, 4, None, 4, None)
+    assert rc == 1

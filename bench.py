@@ -1,0 +1,290 @@
+#!/usr/bin/env python3
+"""Benchmark of the CGT CNN hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+
+A step is one forward+backward pass of one configured layer over one batch of
+synthetic input, every buffer resident in HBM before the timed region:
+    conv2d forward  = im2col -> GEMM(NT) -> transpose{0,3,1,2}
+    [cross-channel LRN forward] -> max-pool forward (values + argmax)
+    max-pool pullback -> [LRN backward]
+    conv2d backward = transpose{0,2,3,1} -> GEMM(NN) -> col2im, GEMM(TN)
+Prints ONE JSON line: the headline conv2d fwd+bwd TFLOP/s over the whole
+step, a per-kernel table (HIP-event timed on the launch stream) with GB/s or
+TFLOP/s against the MI355X roofs, the roofline of the dominant kernel (the
+MFMA GEMM) and the CPU path timed on this box's host cores on a bounded
+sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
+
+WORKLOADS = {
+    # BASELINE.json configs[3]: VGG-style mid layer
+    "vgg_mid_conv3x3_128x56x56_b64": dict(
+        x=(64, 128, 56, 56), f=(128, 128, 3, 3), pad=(1, 1), stride=(1, 1),
+        fscale="he", lrn=None, pool=((2, 2), (0, 0), (2, 2))),
+    # BASELINE.json configs[2]: AlexNet conv1 -> LRN -> pool
+    "alexnet_conv1_11x11s4_3x227x227_b128": dict(
+        x=(128, 3, 227, 227), f=(96, 3, 11, 11), pad=(0, 0), stride=(4, 4),
+        fscale=0.01, lrn=(5, 1e-4, 0.75, 1.0), pool=((3, 3), (0, 0), (2, 2))),
+    # BASELINE.json configs[1], second conv of the CIFAR stack (with its pool + LRN input side)
+    "cifar_conv2_5x5_32x15x15_b128": dict(
+        x=(128, 32, 15, 15), f=(64, 32, 5, 5), pad=(2, 2), stride=(1, 1),
+        fscale=0.01, lrn=None, pool=None),
+    # BASELINE.json configs[0]: MNIST conv block (conv + pool)
+    "mnist_conv3x3_1x28x28_b64": dict(
+        x=(64, 1, 28, 28), f=(32, 1, 3, 3), pad=(1, 1), stride=(1, 1),
+        fscale=0.1, lrn=None, pool=((2, 2), (0, 0), (2, 2))),
+}
+DEFAULT_WORKLOAD = "vgg_mid_conv3x3_128x56x56_b64"
+
+
+def make_inputs(cfg, batch=None, seed=0):
+    """Seeded synthetic inputs: legacy RandomState stream, input then weights."""
+    rs = np.random.RandomState(seed)
+    xs = list(cfg["x"])
+    if batch is not None:
+        xs[0] = batch
+    x = rs.randn(*xs).astype(np.float32)
+    f = rs.randn(*cfg["f"])
+    if cfg["fscale"] == "he":
+        f = f * np.sqrt(1.0 / np.prod(cfg["f"][1:]))
+    else:
+        f = f * cfg["fscale"]
+    return x, f.astype(np.float32)
+
+
+class Stage(object):
+    def __init__(self, name, kernel, fn, work, bound):
+        self.name, self.kernel, self.fn, self.work, self.bound = name, kernel, fn, work, bound
+        self.ms = None
+
+
+class LayerOnGpu(object):
+    """One configured layer with every buffer pre-allocated on the device."""
+
+    def __init__(self, cfg, stream=None):
+        from cgt_amd import kernels as K
+        from cgt_amd.gpuarray import empty, to_gpu
+        self.cfg, self.K, self.stream = cfg, K, stream
+        x, f = make_inputs(cfg)
+        B, C, H, W = x.shape
+        L, _, r, c = f.shape
+        pad, stride = cfg["pad"], cfg["stride"]
+        m, n = K.conv_outsize(H, r, pad[0], stride[0]), K.conv_outsize(W, c, pad[1], stride[1])
+        Z = C * r * c
+        Bmn = B * m * n
+        self.dims = dict(B=B, C=C, H=H, W=W, L=L, r=r, c=c, m=m, n=n, Z=Z, Bmn=Bmn)
+        self.x, self.f = to_gpu(x), to_gpu(f)
+        self.f_LZ = self.f.reshape(L, Z)
+        self.col = empty((B, m, n, Z))
+        self.col2 = self.col.reshape(Bmn, Z)
+        self.y_mnL = empty((Bmn, L))
+        self.y = empty((B, L, m, n))
+        act = self.y
+        nelem = lambda a: int(np.prod(a.shape))  # noqa: E731
+        st = []
+        s = stream
+        st.append(Stage("im2col", "im2col_rows_kernel", lambda: K.im2col(self.x, (r, c), pad, stride, out=self.col, stream=s),
+                        4 * (nelem(self.x) + nelem(self.col)), "hbm"))
+        st.append(Stage("gemm_fwd_NT", "sgemm_kernel<1,1>", lambda: K.mul22(self.col2, self.f_LZ, False, True, out=self.y_mnL, stream=s),
+                        2 * Bmn * L * Z, "mfma"))
+        st.append(Stage("transpose_0312", "batched_transpose_kernel",
+                        lambda: K.transpose4(self.y_mnL.reshape(B, m, n, L), (0, 3, 1, 2), out=self.y, stream=s),
+                        2 * 4 * nelem(self.y), "hbm"))
+        if cfg["lrn"]:
+            size, alpha, beta, k = cfg["lrn"]
+            self.top, self.scale = empty(self.y.shape), empty(self.y.shape)
+            st.append(Stage("lrn_fwd", "lrn_fwd_kernel", lambda: K.lrn_fwd(self.y, size, alpha, beta, k, out=(self.top, self.scale), stream=s),
+                            3 * 4 * nelem(self.y), "hbm"))
+            act = self.top
+        if cfg["pool"]:
+            pk, pp, ps = cfg["pool"]
+            PH, PW = K.pool_outsize(m, pk[0], pp[0], ps[0]), K.pool_outsize(n, pk[1], pp[1], ps[1])
+            self.pool, self.mask = empty((B, L, PH, PW)), empty((B, L, PH, PW), np.int32)
+            self.gpool = to_gpu(np.ones((B, L, PH, PW), np.float32))
+            self.gact = empty(self.y.shape)
+            pool_in = act
+            st.append(Stage("max_pool_fwd", "max_pool_fwd_kernel", lambda: K.max_pool(pool_in, pk, pp, ps, out=(self.pool, self.mask), stream=s),
+                            4 * (nelem(self.y) + 2 * nelem(self.pool)), "hbm"))
+            st.append(Stage("max_pool_bwd", "max_pool_bwd_kernel",
+                            lambda: K.max_pool_pullback(self.y.shape, self.mask, self.gpool, pk, pp, ps, out=self.gact, stream=s),
+                            4 * (2 * nelem(self.pool) + nelem(self.y)), "hbm"))
+            gy = self.gact
+        else:
+            gy = to_gpu(np.ones(self.y.shape, np.float32))   # loss = sum of outputs
+        if cfg["lrn"]:
+            self.gy_lrn = empty(self.y.shape)
+            g_in = gy
+            st.append(Stage("lrn_bwd", "lrn_bwd_kernel",
+                            lambda: K.lrn_bwd(self.y, self.top, self.scale, g_in, size, alpha, beta, out=self.gy_lrn, stream=s),
+                            5 * 4 * nelem(self.y), "hbm"))
+            gy = self.gy_lrn
+        self.gy = gy
+        self.gc = empty((B, m, n, L))
+        self.gc2 = self.gc.reshape(Bmn, L)
+        self.gcol = empty((Bmn, Z))
+        self.gx = empty(self.x.shape)
+        self.gf = empty((L, Z))
+        st.append(Stage("transpose_0231", "batched_transpose_kernel", lambda: K.transpose4(self.gy, (0, 2, 3, 1), out=self.gc, stream=s),
+                        2 * 4 * nelem(self.y), "hbm"))
+        st.append(Stage("gemm_dgrad_NN", "sgemm_kernel<1,0>", lambda: K.mul22(self.gc2, self.f_LZ, False, False, out=self.gcol, stream=s),
+                        2 * Bmn * L * Z, "mfma"))
+        st.append(Stage("col2im", "col2im_gather_kernel",
+                        lambda: K.col2im(self.gcol.reshape(B, m, n, Z), self.x.shape, (r, c), pad, stride, out=self.gx, stream=s),
+                        4 * (nelem(self.x) + nelem(self.col)), "hbm"))
+        st.append(Stage("gemm_wgrad_TN", "sgemm_kernel<0,0>", lambda: K.mul22(self.gc2, self.col2, True, False, out=self.gf, stream=s),
+                        2 * Bmn * L * Z, "mfma"))
+        self.stages = st
+        self.conv_flops = 6 * Bmn * L * Z
+
+    def step(self):
+        for st in self.stages:
+            st.fn()
+
+    def time_stages(self, reps):
+        from cgt_amd import capi
+        for st in self.stages:
+            st.fn()
+            e0, e1 = capi.Event(), capi.Event()
+            e0.record(self.stream)
+            for _ in range(reps):
+                st.fn()
+            e1.record(self.stream)
+            st.ms = e0.elapsed_ms(e1) / reps
+
+
+def check_against_oracle(cfg):
+    """Parity gate run with every measurement, on a 2-image slice of the workload."""
+    from cgt_amd import kernels as K
+    from cgt_amd.gpuarray import to_gpu
+    from oracle import oracle as O
+    x, f = make_inputs(cfg, batch=2, seed=1)
+    pad, stride = cfg["pad"], cfg["stride"]
+    r, c = f.shape[2:]
+    col = K.im2col(to_gpu(x), (r, c), pad, stride)
+    ocol = O.im2col(x, (r, c), pad, stride)
+    ok = np.array_equal(col.get().view(np.uint32), ocol.view(np.uint32))
+    y = K.conv2d(to_gpu(x), to_gpu(f), pad, stride).get()
+    y64 = O.conv2d(x.astype(np.float64), f.astype(np.float64), pad, stride)
+    err = float(np.linalg.norm(y - y64) / np.linalg.norm(y64))
+    return {"im2col_bit_exact": bool(ok), "conv2d_rel_fro": err, "ok": bool(ok and err <= 1e-4)}
+
+
+def cpu_baseline(cfg, sample_batch):
+    """The CPU path (oracle stages + OpenBLAS sgemm) on a bounded sample of the workload."""
+    from oracle import cpu_baseline as CB
+    from oracle import oracle as O
+    threads = CB.set_threads(min(CB.host_cores(), 16))
+    x, f = make_inputs(cfg, batch=sample_batch)
+    pad, stride = cfg["pad"], cfg["stride"]
+    L, C, r, c = f.shape
+    m = O.conv_outsize(x.shape[2], r, pad[0], stride[0])
+    n = O.conv_outsize(x.shape[3], c, pad[1], stride[1])
+    gy = np.ones((sample_batch, L, m, n), np.float32)
+
+    def run():
+        y, gx, gf = CB.conv2d_fwd_bwd(x, f, gy, pad, stride)
+        act = y
+        if cfg["lrn"]:
+            size, alpha, beta, k = cfg["lrn"]
+            act, scale = O.lrn_fwd(y, size, alpha, beta, k)
+        if cfg["pool"]:
+            pk, pp, ps = cfg["pool"]
+            pool, mask = O.max_pool(act, pk, pp, ps)
+            g = O.max_pool_pullback(act.shape, mask, np.ones_like(pool))
+            if cfg["lrn"]:
+                O.lrn_bwd(y, act, scale, g, size, alpha, beta)
+
+    best, reps = CB.timed(run, min_seconds=8.0, max_reps=20)
+    flops = 6 * sample_batch * m * n * L * C * r * c
+    return {"value": flops / best / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": "%d of %d images of the workload, best of %d passes (%.2f s each); im2col/col2im/"
+                      "transpose/pool/LRN single-threaded C, GEMM %s with %d threads; host %s, %d cores usable"
+                      % (sample_batch, cfg["x"][0], reps, best, CB.blas_config(), threads, CB.cpu_model(), CB.host_cores())}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
+    ap.add_argument("--stage-reps", type=int, default=20)
+    ap.add_argument("--cpu-sample", type=int, default=4, help="images in the CPU baseline sample")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (the hot path has no "
+                 "multi-GPU part: it would shard the batch axis, see DESIGN.md)" % args.gpus)
+
+    from cgt_amd import capi
+    capi.require_gpu()
+    cfg = WORKLOADS[args.workload]
+    layer = LayerOnGpu(cfg)
+    parity = check_against_oracle(cfg)
+
+    for _ in range(args.warmup):
+        layer.step()
+    capi.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        layer.step()
+    capi.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+
+    layer.time_stages(args.stage_reps)
+    stages = []
+    gemm_flops = gemm_ms = 0.0
+    for st in layer.stages:
+        row = {"stage": st.name, "kernel": st.kernel, "ms": round(st.ms, 4), "bound": st.bound}
+        if st.bound == "hbm":
+            gbs = st.work / (st.ms * 1e-3) / 1e9
+            row.update(bytes=st.work, GBps=round(gbs, 1), frac=round(gbs / HBM_PEAK_GBS, 4))
+        else:
+            tf = st.work / (st.ms * 1e-3) / 1e12
+            row.update(flops=st.work, TFLOPs=round(tf, 2), frac=round(tf / FP32_MFMA_PEAK_TFLOPS, 4))
+            gemm_flops += st.work
+            gemm_ms += st.ms
+        stages.append(row)
+    gemm_tf = gemm_flops / (gemm_ms * 1e-3) / 1e12
+    value = layer.conv_flops / (ms_per_step * 1e-3) / 1e12
+
+    out = {
+        "metric": "conv2d fwd+bwd TFLOP/s (% fp32 MFMA peak); pool/LRN/im2col GB/s (% HBM)",
+        "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": args.workload, "x": list(cfg["x"]), "filters": list(cfg["f"]),
+                   "pad": list(cfg["pad"]), "stride": list(cfg["stride"]),
+                   "value_is": "conv GEMM flops (6*B*m*n*L*Z) / whole step time incl. im2col, col2im, "
+                               "transposes, pool and LRN stages"},
+        "frac_fp32_mfma_peak": round(value / FP32_MFMA_PEAK_TFLOPS, 4),
+        "roofline": {"bound": "mfma", "kernel": "sgemm_kernel (NT + NN + TN launches of one step)",
+                     "achieved": round(gemm_tf, 2), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(gemm_tf / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None},
+        "stages": stages,
+        "parity": parity,
+        "device": capi.device_name(),
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample)
+    print(json.dumps(out))
+    if not parity["ok"]:
+        sys.exit("bench.py: parity gate failed: %r" % (parity,))
+
+
+if __name__ == "__main__":
+    main()

@@ -16,12 +16,15 @@
 //   channel is ascending z -- the order the sequential reference adds them in
 //   -- so no atomics are needed and the result is bit-identical.
 #include "common.h"
+#include <algorithm>
 
 namespace cgt_amd {
 
 // Geometry known at compile time (hot shapes) ...
 template <int KH, int KW, int PH, int PW, int SH, int SW>
 struct StaticGeom {
+    static constexpr bool is_static = true;
+    static constexpr int kKH = KH, kKW = KW, kPH = PH, kPW = PW, kSH = SH, kSW = SW;
     __host__ __device__ constexpr int kh() const { return KH; }
     __host__ __device__ constexpr int kw() const { return KW; }
     __host__ __device__ constexpr int ph() const { return PH; }
@@ -31,6 +34,7 @@ struct StaticGeom {
 };
 // ... or only at run time (anything else).
 struct DynGeom {
+    static constexpr bool is_static = false;
     int kh_, kw_, ph_, pw_, sh_, sw_;
     __host__ __device__ int kh() const { return kh_; }
     __host__ __device__ int kw() const { return kw_; }
@@ -162,6 +166,143 @@ __global__ __launch_bounds__(256) void col2im_gather_kernel(
     }
 }
 
+
+// LDS-staged col2im for compile-time geometry.
+//
+// A workgroup owns (image b, CC channels, TH image rows, 64*WSUB image columns)
+// and keeps that tile's sums in registers: thread (wave, lane) owns the pixel
+// columns q = wave + 4*i (q -> channel q % CC, column block q / CC, column
+// wp0 + 64*block + lane) with TH accumulators each.  The column-buffer rows
+// that feed the tile are streamed through LDS from the highest h to the
+// lowest, one row per step, each as contiguous runs of CC*kh*kw floats
+// (coalesced, every byte of the buffer read once apart from the halo rows
+// between neighbouring tiles).  For a fixed pixel, descending h is ascending
+// kernel row ho and taps inside a row are taken in ascending wo, so the adds
+// happen in ascending z exactly as in the sequential reference loop.
+// All accumulator indices are compile-time after unrolling because tile rows
+// start on multiples of TH and TH % stride == 0.
+template <class G, int CC, int WSUB, int TH>
+__global__ __launch_bounds__(256) void col2im_rows_kernel(
+    G g, const float* __restrict__ col, float* __restrict__ im, int C, int H, int W, int m, int n,
+    int tiles_h, int tiles_w, int nchunks, int vec) {
+    constexpr int KH = G::kKH, KW = G::kKW, PH = G::kPH, PW = G::kPW, SH = G::kSH, SW = G::kSW;
+    constexpr int KK = KH * KW, RUN = CC * KK;
+    constexpr int LD = RUN | 1;                       // odd row stride: conflict-free column reads
+    constexpr int TW = 64 * WSUB;
+    constexpr int NQ = (CC * WSUB + 3) / 4;
+    static_assert(TH % SH == 0, "tile rows must start on a stride multiple");
+    constexpr int H0 = (TH - 1 + PH) / SH;            // highest contributing row = hp0/SH + H0
+    constexpr int NH = (TH - 1 + KH - 1) / SH + 1;    // rows that can touch a tile
+    constexpr int NT = (KW + SW - 1) / SW;            // taps per row and pixel
+    extern __shared__ float stage[];                  // [nw][LD]
+
+    long bid = blockIdx.x;
+    const int wt = (int)(bid % tiles_w);
+    bid /= tiles_w;
+    const int ht = (int)(bid % tiles_h);
+    bid /= tiles_h;
+    const int ck = (int)(bid % nchunks);
+    const long b = bid / nchunks;
+    const int hp0 = ht * TH, wp0 = wt * TW, c0 = ck * CC;
+    const int cc = min(CC, C - c0);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long Z = (long)C * KK;
+
+    const int wl = wp0 + PW - (KW - 1);
+    const int w_lo = wl > 0 ? (wl + SW - 1) / SW : 0;
+    const int w_hi = min(n - 1, (wp0 + TW - 1 + PW) / SW);
+    const int nw = w_hi - w_lo + 1;
+    const int htop = hp0 / SH + H0;
+
+    int cq[NQ], wp[NQ];
+    bool ok[NQ];
+    float acc[NQ][TH];
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) {
+        const int q = wave + 4 * i;
+        cq[i] = q % CC;
+        wp[i] = wp0 + (q / CC) * 64 + lane;
+        ok[i] = (q < CC * WSUB) && (cq[i] < cc) && (wp[i] < W);
+#pragma unroll
+        for (int j = 0; j < TH; ++j) acc[i][j] = 0.0f;
+    }
+
+#pragma unroll
+    for (int hi = 0; hi < NH; ++hi) {
+        const int h = htop - hi;
+        if (h < 0 || h >= m || nw <= 0) continue;     // uniform over the workgroup
+        const float* src = col + ((b * m + h) * (long)n + w_lo) * Z + (long)c0 * KK;
+        if (cc == CC) {
+            if (vec) {
+                for (int idx = threadIdx.x; idx < nw * (RUN / 4); idx += 256) {
+                    const int w = idx / (RUN / 4), z4 = (idx - w * (RUN / 4)) * 4;
+                    const float4 v = *reinterpret_cast<const float4*>(src + (long)w * Z + z4);
+                    float* d = stage + w * LD + z4;
+                    d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+                }
+            } else {
+                for (int idx = threadIdx.x; idx < nw * RUN; idx += 256) {
+                    const int w = idx / RUN, zc = idx - w * RUN;
+                    stage[w * LD + zc] = src[(long)w * Z + zc];
+                }
+            }
+        } else {
+            const int run = cc * KK;
+            for (int idx = threadIdx.x; idx < nw * run; idx += 256) {
+                const int w = idx / run, zc = idx - w * run;
+                stage[w * LD + zc] = src[(long)w * Z + zc];
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            if (!ok[i]) continue;
+            const int wpp = wp[i] + PW;
+            const int r = wpp % SW;
+#pragma unroll
+            for (int ho = 0; ho < KH; ++ho) {
+                const int j = (H0 - hi) * SH - PH + ho;   // compile-time after unrolling
+                if (j < 0 || j >= TH) continue;
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const int wo = r + t * SW;
+                    const int ww = wpp - wo;
+                    const int w = ww / SW;
+                    if (wo < KW && ww >= 0 && w <= w_hi)
+                        acc[i][j] += stage[(w - w_lo) * LD + (cq[i] * KH + ho) * KW + wo];
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) {
+        if (!ok[i]) continue;
+        float* dst = im + ((b * C + c0 + cq[i]) * (long)H) * W + wp[i];
+#pragma unroll
+        for (int j = 0; j < TH; ++j)
+            if (hp0 + j < H) dst[(long)(hp0 + j) * W] = acc[i][j];
+    }
+}
+
+template <class G, int CC, int WSUB, int TH>
+static int launch_col2im_rows(G g, const float* col, long B, int C, int H, int W, int m, int n,
+                              float* im, hipStream_t st) {
+    constexpr int KK = G::kKH * G::kKW, RUN = CC * KK, LD = RUN | 1, TW = 64 * WSUB;
+    const int tiles_h = (int)cdiv(H, TH), tiles_w = (int)cdiv(W, TW), nchunks = (int)cdiv(C, CC);
+    const long nwb = std::min((long)n, (long)(TW + G::kKW - 2) / G::kSW + 1);
+    const size_t lds = (size_t)nwb * LD * sizeof(float);
+    const long blocks = B * nchunks * tiles_h * tiles_w;
+    CGT_ARG_CHECK(blocks < (1L << 31) && lds <= 64 * 1024, "col2im: tile configuration out of range");
+    const long Z = (long)C * KK;
+    const int vec = (RUN % 4 == 0 && Z % 4 == 0 && reinterpret_cast<uintptr_t>(col) % 16 == 0) ? 1 : 0;
+    col2im_rows_kernel<G, CC, WSUB, TH><<<dim3((unsigned)blocks), dim3(256), lds, st>>>(
+        g, col, im, C, H, W, m, n, tiles_h, tiles_w, nchunks, vec);
+    CGT_LAUNCH_CHECK("col2im_rows_kernel");
+    return CGT_AMD_OK;
+}
+
 static int check_geom(const char* what, long B, long C, long H, long W, int kh, int kw, int ph,
                       int pw, int sh, int sw, long* m, long* n) {
     CGT_ARG_CHECK(B >= 0 && C >= 0 && H >= 0 && W >= 0, "%s: negative shape", what);
@@ -220,11 +361,43 @@ static int launch_im2col(G g, const float* im, long B, int C, int H, int W, int 
     return CGT_AMD_OK;
 }
 
+// Tiling of col2im_rows_kernel per compile-time geometry: <channels per chunk,
+// 64-column blocks per tile, image rows per tile>.  Returns -1 when the shape
+// is better served by the plain gather kernel.
+template <class G>
+static int try_col2im_rows(G, const float*, long, int, int, int, int, int, float*, hipStream_t) {
+    return -1;
+}
+static int try_col2im_rows(StaticGeom<3, 3, 1, 1, 1, 1> g, const float* col, long B, int C, int H,
+                           int W, int m, int n, float* im, hipStream_t st) {
+    if (C >= 16 && W >= 24) return launch_col2im_rows<decltype(g), 16, 1, 14>(g, col, B, C, H, W, m, n, im, st);
+    return -1;
+}
+static int try_col2im_rows(StaticGeom<3, 3, 0, 0, 1, 1> g, const float* col, long B, int C, int H,
+                           int W, int m, int n, float* im, hipStream_t st) {
+    if (C >= 16 && W >= 24) return launch_col2im_rows<decltype(g), 16, 1, 14>(g, col, B, C, H, W, m, n, im, st);
+    return -1;
+}
+static int try_col2im_rows(StaticGeom<5, 5, 2, 2, 1, 1> g, const float* col, long B, int C, int H,
+                           int W, int m, int n, float* im, hipStream_t st) {
+    if (C >= 4 && W >= 24) return launch_col2im_rows<decltype(g), 4, 1, 28>(g, col, B, C, H, W, m, n, im, st);
+    return -1;
+}
+static int try_col2im_rows(StaticGeom<11, 11, 0, 0, 4, 4> g, const float* col, long B, int C, int H,
+                           int W, int m, int n, float* im, hipStream_t st) {
+    if (C == 3 && W >= 64) return launch_col2im_rows<decltype(g), 3, 2, 32>(g, col, B, C, H, W, m, n, im, st);
+    return -1;
+}
+
 template <class G>
 static int launch_col2im(G g, const float* col, long B, int C, int H, int W, int m, int n,
                          float* im, hipStream_t st) {
     const long total = B * C * H * W;
     if (total == 0) return CGT_AMD_OK;
+    {
+        const int rc = try_col2im_rows(g, col, B, C, H, W, m, n, im, st);
+        if (rc >= 0) return rc;
+    }
     long blocks = cdiv(total, 256);
     if (blocks > 1 << 20) blocks = 1 << 20;
     col2im_gather_kernel<G><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(g, col, im, total, C, H, W, m, n);

@@ -97,6 +97,10 @@ IM2COL_CASES = [
     ((2, 4, 13, 14), (5, 3), (2, 1), (2, 3)),
     ((1, 1, 3, 20000), (3, 3), (1, 1), (1, 1)),    # row too wide for LDS staging
     ((1, 2, 4, 6), (4, 6), (0, 0), (1, 1)),        # single output pixel
+    ((2, 6, 30, 40), (5, 5), (2, 2), (1, 1)),      # 5x5 row-streamed col2im, partial channel chunk
+    ((1, 20, 17, 70), (3, 3), (0, 0), (1, 1)),     # two column tiles, partial row tile
+    ((1, 16, 56, 56), (3, 3), (1, 1), (1, 1)),
+    ((1, 3, 100, 300), (11, 11), (0, 0), (4, 4)),  # three column tiles at stride 4
 ]
 
 

@@ -47,6 +47,8 @@ WORKLOADS = {
         x=(64, 1, 28, 28), f=(32, 1, 3, 3), pad=(1, 1), stride=(1, 1),
         fscale=0.1, lrn=None, pool=((2, 2), (0, 0), (2, 2))),
 }
+# BASELINE.json configs[4]: raw dense contraction
+GEMM_WORKLOAD = "raw_gemm_4096_and_batched_64x512"
 DEFAULT_WORKLOAD = "vgg_mid_conv3x3_128x56x56_b64"
 
 
@@ -165,6 +167,47 @@ class LayerOnGpu(object):
             st.ms = e0.elapsed_ms(e1) / reps
 
 
+class GemmOnGpu(object):
+    """Mul22 4096^3 in all four transpose variants + BatchedMul22 64 x 512^3, operands ~ U(-1,1)."""
+
+    def __init__(self, stream=None, n=4096, P=64, nb=512):
+        from cgt_amd import kernels as K
+        from cgt_amd.gpuarray import empty, to_gpu
+        rs = np.random.RandomState(0)
+        self.stream = stream
+        self.A = to_gpu(rs.uniform(-1, 1, (n, n)).astype(np.float32))
+        self.B = to_gpu(rs.uniform(-1, 1, (n, n)).astype(np.float32))
+        self.C = empty((n, n))
+        self.bA = to_gpu(rs.uniform(-1, 1, (P, nb, nb)).astype(np.float32))
+        self.bB = to_gpu(rs.uniform(-1, 1, (P, nb, nb)).astype(np.float32))
+        self.bC = empty((P, nb, nb))
+        s = stream
+        st = []
+        for tA, tB, name in [(False, False, "NN"), (False, True, "NT"), (True, False, "TN"), (True, True, "TT")]:
+            st.append(Stage("mul22_%s_%d" % (name, n), "sgemm_kernel<%d,%d>" % (not tA, tB),
+                            (lambda tA=tA, tB=tB: K.mul22(self.A, self.B, tA, tB, out=self.C, stream=s)),
+                            2 * n ** 3, "mfma"))
+        st.append(Stage("batched_mul22_%dx%d" % (P, nb), "sgemm_kernel<1,0>",
+                        lambda: K.batched_mul22(self.bA, self.bB, out=self.bC, stream=s), 2 * P * nb ** 3, "mfma"))
+        self.stages = st
+        self.conv_flops = sum(x.work for x in st)
+
+    step = LayerOnGpu.step
+    time_stages = LayerOnGpu.time_stages
+
+
+def check_gemm_against_oracle():
+    from cgt_amd import kernels as K
+    from cgt_amd.gpuarray import to_gpu
+    rs = np.random.RandomState(1)
+    A = rs.uniform(-1, 1, (300, 1000)).astype(np.float32)
+    B = rs.uniform(-1, 1, (200, 1000)).astype(np.float32)
+    C = K.mul22(to_gpu(A), to_gpu(B), False, True).get()
+    ref = A.astype(np.float64) @ B.astype(np.float64).T
+    err = float(np.linalg.norm(C - ref) / np.linalg.norm(ref))
+    return {"mul22_rel_fro": err, "ok": bool(err <= 1e-4)}
+
+
 def check_against_oracle(cfg):
     """Parity gate run with every measurement, on a 2-image slice of the workload."""
     from cgt_amd import kernels as K
@@ -215,14 +258,26 @@ def cpu_baseline(cfg, sample_batch):
                       % (sample_batch, cfg["x"][0], reps, best, CB.blas_config(), threads, CB.cpu_model(), CB.host_cores())}
 
 
+def cpu_gemm_baseline(n=2048):
+    from oracle import cpu_baseline as CB
+    threads = CB.set_threads(min(CB.host_cores(), 16))
+    rs = np.random.RandomState(0)
+    A = rs.uniform(-1, 1, (n, n)).astype(np.float32)
+    B = rs.uniform(-1, 1, (n, n)).astype(np.float32)
+    best, reps = CB.timed(lambda: CB.sgemm(A, B), min_seconds=8.0, max_reps=200)
+    return {"value": 2 * n ** 3 / best / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": "Mul22 NN %d^3 (1/8 of the 4096^3 work), best of %d; %s with %d threads; host %s"
+                      % (n, reps, CB.blas_config(), threads, CB.cpu_model())}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS) + [GEMM_WORKLOAD])
     ap.add_argument("--stage-reps", type=int, default=20)
-    ap.add_argument("--cpu-sample", type=int, default=4, help="images in the CPU baseline sample")
+    ap.add_argument("--cpu-sample", type=int, default=16, help="images in the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -231,9 +286,15 @@ def main():
 
     from cgt_amd import capi
     capi.require_gpu()
-    cfg = WORKLOADS[args.workload]
-    layer = LayerOnGpu(cfg)
-    parity = check_against_oracle(cfg)
+    is_gemm = args.workload == GEMM_WORKLOAD
+    if is_gemm:
+        cfg = {"x": [4096, 4096], "f": [4096, 4096], "pad": [], "stride": []}
+        layer = GemmOnGpu()
+        parity = check_gemm_against_oracle()
+    else:
+        cfg = WORKLOADS[args.workload]
+        layer = LayerOnGpu(cfg)
+        parity = check_against_oracle(cfg)
 
     for _ in range(args.warmup):
         layer.step()
@@ -279,8 +340,13 @@ def main():
         "parity": parity,
         "device": capi.device_name(),
     }
-    if not args.no_cpu:
+    if is_gemm:
+        out["config"]["value_is"] = "flops of Mul22 4096^3 x {NN,NT,TN,TT} + BatchedMul22 64x512^3 / step time"
+        out["roofline"]["kernel"] = "sgemm_kernel (all launches of one step)"
+    if not args.no_cpu and not is_gemm:
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample)
+    elif not args.no_cpu:
+        out["cpu_baseline"] = cpu_gemm_baseline()
     print(json.dumps(out))
     if not parity["ok"]:
         sys.exit("bench.py: parity gate failed: %r" % (parity,))

@@ -18,6 +18,11 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(LIBDIR, "obj")
 LIBPATH = os.path.join(LIBDIR, "libcgt_amd.so")
+RT_LIBPATH = os.path.join(LIBDIR, "libcgt_rt.so")
+RT_INCLUDE = os.path.join(CSRC, "include")
+CXX = os.environ.get("CXX", "g++")
+# flags of the reference's native-compile step for host code (cgt/compilation.py:688)
+CPP_FLAGS = ["-fvisibility=hidden", "-std=c++11", "-fPIC", "-O3", "-DNDEBUG"]
 INCLUDE = os.path.join(ROOT, "include")
 
 SOURCES = ["runtime.hip", "im2col.hip", "pool.hip", "lrn.hip", "gemm.hip", "glue.hip"]
@@ -63,7 +68,19 @@ def build(verbose=True):
     os.replace(tmp, LIBPATH)
     if verbose:
         print("built", LIBPATH)
+    build_runtime(verbose)
     return LIBPATH
+
+
+def build_runtime(verbose=True):
+    """Host runtime (object model, C API for the host language, interpreter): plain g++."""
+    tmp = RT_LIBPATH + ".tmp"
+    _run([CXX] + CPP_FLAGS + ["-I" + INCLUDE, "-I" + RT_INCLUDE, os.path.join(CSRC, "cgt_runtime.cpp"),
+                              "-shared", "-o", tmp, "-L" + LIBDIR, "-lcgt_amd", "-Wl,-rpath,$ORIGIN"])
+    os.replace(tmp, RT_LIBPATH)
+    if verbose:
+        print("built", RT_LIBPATH)
+    return RT_LIBPATH
 
 
 def main(argv):

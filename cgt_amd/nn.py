@@ -1,0 +1,31 @@
+"""cgt.nn front end of the CNN hot path (reference cgt/nn.py:85-111).
+
+conv2d keeps the reference's CPU-path composition
+    im2col -> reshape -> Mul22(False, True) -> reshape -> transpose{0,3,1,2}
+with every op running on the GPU (the reference's devtype == "gpu" branch
+calls cuDNN instead, which this build replaces).
+"""
+from . import core
+from .nn_ops.cross_channel_lrn import cross_channel_lrn  # noqa: F401
+from .nn_ops.im2col import im2col
+from .nn_ops.max_pool_2d import MaxPool, PoolInfo
+
+
+def conv2d(x_BKRC, f_LKrc, kernelshape, pad=(0, 0), stride=(1, 1)):
+    x_BKRC, f_LKrc = core.as_node(x_BKRC), core.as_node(f_LKrc)
+    L, K, r, c = f_LKrc.shape
+    assert tuple(kernelshape) == (r, c), "kernelshape must match the filter's last two axes"
+    col_BmnZ = im2col(x_BKRC, kernelshape, pad, stride)
+    f_LZ = f_LKrc.reshape([L, K * r * c])
+    B, m, n, Z = col_BmnZ.shape
+    col_Bmn_Z = col_BmnZ.reshape([B * m * n, Z])
+    col_Bmn_L = core.Result(core.Mul22(False, True), [col_Bmn_Z, f_LZ])
+    return col_Bmn_L.reshape([B, m, n, L]).transpose([0, 3, 1, 2])
+
+
+def max_pool_2d(x, kernelshape, pad=(0, 0), stride=(1, 1)):
+    kernel_h, kernel_w = kernelshape
+    pad_h, pad_w = pad
+    stride_h, stride_w = stride
+    info = PoolInfo(kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w)
+    return core.Result(MaxPool(info), [x])[0]

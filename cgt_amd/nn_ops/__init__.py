@@ -1,0 +1,2 @@
+"""The image-processing ops of the CNN hot path (reference cgt/nn_ops/)."""
+from . import cross_channel_lrn, im2col, max_pool_2d  # noqa: F401

@@ -1,0 +1,97 @@
+"""Cross-channel LRN ops (reference cgt/nn_ops/cross_channel_lrn.py).
+
+The closure keeps the reference's fields (localsize, alpha, beta) and adds
+`k`, the additive constant of the scale, which the reference fixes at 1
+(include/lrn.cuh:27); k = 1 is therefore reference behaviour.
+"""
+import ctypes
+from collections import namedtuple
+
+from .. import core
+
+LRNInfo = namedtuple("LRNInfo", ["localsize", "alpha", "beta"])
+
+
+def make_closure(info, k=1.0):
+    return [
+        ("localsize", ctypes.c_int, info.localsize),
+        ("alpha", ctypes.c_double, info.alpha),
+        ("beta", ctypes.c_double, info.beta),
+        ("k", ctypes.c_double, k),
+    ]
+
+
+class CrossChannelLRNForward(core.Op):
+    available_impls = ("native_gpu",)
+
+    def __init__(self, info, k=1.0):
+        assert isinstance(info, LRNInfo)
+        self.info = info
+        self.k = float(k)
+
+    def get_native_compile_info(self, input_types, devtype):
+        assert devtype == "gpu" and input_types[0].dtype == "f4"
+        code = r"""
+            CGT_EXPORT_C void $function($closure* cldata, cgtArray** reads, cgtTuple* write) {
+                cgtArray* X = reads[0];
+                long num_img = X->shape()[0],
+                     channels = X->shape()[1],
+                     height = X->shape()[2],
+                     width = X->shape()[3];
+                cgtArray* top = (cgtArray*)write->getitem(0);
+                cgtArray* scale = (cgtArray*)write->getitem(1);
+                int rc = cgt_amd_lrn_fwd_f32((const float*)X->data(), num_img, channels, height, width,
+                    cldata->localsize, cldata->alpha, cldata->beta, cldata->k,
+                    (float*)top->data(), (float*)scale->data(), cgt_get_stream());
+                cgt_check(rc == CGT_AMD_OK, "CrossChannelLRNForward: %s", cgt_amd_last_error());
+            }"""
+        return core.NativeCompileInfo(code, closure_triples=make_closure(self.info, self.k),
+                                      includes=["cgt_amd.h"], gpu_deref_mask=(True,))
+
+    def shp_apply(self, inputs):
+        return (core.shape(inputs[0]), core.shape(inputs[0]))
+
+    def typ_apply(self, input_types):
+        return core.TupleType(input_types[0], input_types[0])
+
+    def pullback(self, inputs, output, gout):
+        top, scaling = core.unpack(output)
+        gtop, _ = gout
+        return [core.Result(CrossChannelLRNBackward(self.info), [inputs[0], top, scaling, gtop])]
+
+
+class CrossChannelLRNBackward(core.Op):
+    available_impls = ("native_gpu",)
+
+    def __init__(self, info):
+        self.info = info
+
+    def get_native_compile_info(self, input_types, devtype):
+        assert devtype == "gpu" and input_types[0].dtype == "f4"
+        code = r"""
+            CGT_EXPORT_C void $function($closure* cldata, cgtArray** reads, cgtArray* bottom_diff) {
+                cgtArray *X=reads[0], *top=reads[1], *scaling=reads[2], *top_diff=reads[3];
+                long num_img = X->shape()[0],
+                     channels = X->shape()[1],
+                     height = X->shape()[2],
+                     width = X->shape()[3];
+                int rc = cgt_amd_lrn_bwd_f32((const float*)X->data(), (const float*)top->data(),
+                    (const float*)scaling->data(), (const float*)top_diff->data(),
+                    num_img, channels, height, width, cldata->localsize, cldata->alpha, cldata->beta,
+                    (float*)bottom_diff->data(), cgt_get_stream());
+                cgt_check(rc == CGT_AMD_OK, "CrossChannelLRNBackward: %s", cgt_amd_last_error());
+            }"""
+        return core.NativeCompileInfo(code, closure_triples=make_closure(self.info),
+                                      includes=["cgt_amd.h"], gpu_deref_mask=(True, True, True, True))
+
+    def shp_apply(self, inputs):
+        return core.shape(inputs[0])
+
+    def typ_apply(self, _inputs):
+        return core.TensorType(core.floatX, 4)
+
+
+def cross_channel_lrn(X, localsize, alpha, beta, k=1.0):
+    X = core.as_node(X)
+    assert X.ndim == 4
+    return core.Result(CrossChannelLRNForward(LRNInfo(localsize, alpha, beta), k), [X])[0]

@@ -1,0 +1,74 @@
+/*
+ * cgt_rt -- C API of the host runtime (libcgt_rt.so) for a host language that
+ * drives compiled op closures without a C++ binding of its own.
+ *
+ * The objects behind the void* handles are the cgtArray / cgtTuple classes of
+ * cgt_amd/csrc/include/cgt_common.h, i.e. what a compiled closure
+ *     void call_X(closure*, cgtArray** reads, cgtArray* | cgtTuple* write)
+ * receives.  This API replaces, for this path, the Cython bridge of the
+ * reference (src/cycgt.pyx): object construction / conversion
+ * (cycgt.pyx:97-141), apply_byref (cycgt.pyx:439-449) and the interpreter
+ * wrapper (cycgt.pyx:338-434) over the instruction set of
+ * include/execution.h:44-165 / src/execution.cpp:247-292.
+ *
+ * Every function that can fail leaves a status readable with
+ * cgt_rt_status() / cgt_rt_error() (cgtGlobalStatus / cgtGlobalErrorMsg of
+ * the reference, include/cgt_common.h:194-215, which nothing there reads).
+ */
+#ifndef CGT_RT_H
+#define CGT_RT_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* dtype: numpy type numbers (f4 = 11, i4 = 5, i8 = 7); devtype: 0 = host, 1 = GPU */
+
+int cgt_rt_status(void);            /* 0 = ok */
+const char *cgt_rt_error(void);
+void cgt_rt_clear_error(void);
+
+/* stream the op closures launch on (NULL = default stream) */
+void *cgt_get_stream(void);
+void cgt_set_stream(void *stream);
+
+/* objects: every handle returned here carries one reference owned by the caller */
+void *cgt_rt_array_new(int ndim, const long *shape, int dtype, int devtype);
+void *cgt_rt_array_view(int ndim, const long *shape, int dtype, int devtype, void *data);
+void *cgt_rt_tuple_new(int len);
+void cgt_rt_tuple_setitem(void *tup, int i, void *obj);
+void *cgt_rt_tuple_getitem(void *tup, int i);   /* borrowed */
+int cgt_rt_tuple_len(void *tup);
+void cgt_rt_retain(void *obj);
+void cgt_rt_release(void *obj);
+int cgt_rt_kind(void *obj);          /* 1 = array, 2 = tuple */
+int cgt_rt_array_ndim(void *a);
+const long *cgt_rt_array_shape(void *a);
+int cgt_rt_array_dtype(void *a);
+int cgt_rt_array_devtype(void *a);
+void *cgt_rt_array_data(void *a);
+long cgt_rt_array_nbytes(void *a);
+long cgt_rt_array_stride(void *a, int i);
+int cgt_rt_copy_object(void *to, void *from);   /* host <-> device as needed */
+
+/* fire one compiled closure */
+int cgt_rt_apply_byref(void *fptr, void *closure, void **reads, int n_reads, void *write);
+void *cgt_rt_apply_byval(void *fptr, void *closure, void **reads, int n_reads);
+
+/* sequential interpreter over storage slots (LoadArgument / Alloc / BuildTup /
+ * ReturnByRef / ReturnByVal); add_* return the instruction index or -1 */
+void *cgt_rt_interp_new(long n_slots);
+void cgt_rt_interp_free(void *interp);
+int cgt_rt_interp_add_load_argument(void *interp, int arg_index, long widx, int wdev);
+int cgt_rt_interp_add_alloc(void *interp, int dtype, const long *ridx, const int *rdev, int nr, long widx, int wdev);
+int cgt_rt_interp_add_build_tup(void *interp, const long *ridx, const int *rdev, int nr, long widx, int wdev);
+int cgt_rt_interp_add_return_byref(void *interp, void *fptr, void *closure, const long *ridx, const int *rdev, int nr, long widx, int wdev);
+int cgt_rt_interp_add_return_byval(void *interp, void *fptr, void *closure, const long *ridx, const int *rdev, int nr, long widx, int wdev);
+int cgt_rt_interp_set_slot(void *interp, long idx, void *obj);
+void *cgt_rt_interp_get_slot(void *interp, long idx);  /* borrowed */
+int cgt_rt_interp_run(void *interp, void **args, int n_args); /* 0, or 1 + failing instruction */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CGT_RT_H */

@@ -17,6 +17,7 @@
 //   -- so no atomics are needed and the result is bit-identical.
 #include "common.h"
 #include <algorithm>
+#include <cstdlib>
 
 namespace cgt_amd {
 
@@ -47,18 +48,35 @@ struct DynGeom {
 constexpr int kIm2colThreads = 256;
 constexpr int kIm2colWaves = kIm2colThreads / kWave;
 
-// VEC: 4 consecutive z per lane, 16-byte stores (needs Z%4==0, chunk*kh*kw%4==0).
+// Workgroups are handed to the 8 XCDs round-robin by linear id.  Remapping the
+// id so that each XCD owns one contiguous range puts neighbouring tiles (which
+// share halo rows) behind the same L2 and close together in time.
+__device__ __forceinline__ long xcd_remap(long id, long n) {
+    const long q = n / kNumXCD, r = n % kNumXCD;
+    const long xcd = id % kNumXCD, local = id / kNumXCD;
+    return xcd * q + (xcd < r ? xcd : r) + local;
+}
+
+// VEC: units of 4 consecutive z per thread and 16-byte stores (needs Z%4==0
+// and chunk*kh*kw%4==0); otherwise units of one float.
+//
+// A thread owns a fixed unit column (its z values, hence its (channel, kernel
+// row, kernel col) LDS offsets, decoded once) and walks the output pixels w of
+// the row: per step the LDS offsets advance by the stride and the store address
+// by Z floats -- no divisions in the loop.  Lanes hold consecutive unit columns,
+// so each store instruction covers one contiguous run.
 template <class G, bool VEC>
 __global__ __launch_bounds__(kIm2colThreads) void im2col_rows_kernel(
     G g, const float* __restrict__ im, float* __restrict__ col, int C, int H, int W, int m, int n,
     int chunk, int nchunks) {
     extern __shared__ float tile[];  // [cc*kh][Wp], Wp = W + 2*pw
+    constexpr int UW = VEC ? 4 : 1;
 
     const int KH = g.kh(), KW = g.kw();
     const int Wp = W + 2 * g.pw();
-    const long bid = blockIdx.x;
-    const int ck = (int)(bid % nchunks);
-    const int h = (int)((bid / nchunks) % m);
+    const long bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int h = (int)(bid % m);
+    const int ck = (int)((bid / m) % nchunks);
     const long b = bid / ((long)nchunks * m);
     const int c0 = ck * chunk;
     const int cc = min(chunk, C - c0);
@@ -81,31 +99,138 @@ __global__ __launch_bounds__(kIm2colThreads) void im2col_rows_kernel(
     __syncthreads();
 
     const int KK = KH * KW;
-    const int zc_n = cc * KK;                // z's this workgroup writes per output pixel
+    const int units = cc * KK / UW;          // unit columns this workgroup writes per pixel
     const long Z = (long)C * KK;
     float* orow = col + ((b * m + h) * (long)n) * Z + (long)c0 * KK;
-    for (int w = wave; w < n; w += kIm2colWaves) {
-        float* out = orow + (long)w * Z;
-        const int xbase = w * g.sw();
-        if (VEC) {
-            for (int z4 = lane * 4; z4 < zc_n; z4 += kWave * 4) {
-                float v[4];
+    // few unit columns: several threads share a column and interleave over w
+    const int slots = units < kIm2colThreads ? kIm2colThreads / units : 1;
+    const int w0 = units < kIm2colThreads ? (int)threadIdx.x / units : 0;
+    const int u0 = units < kIm2colThreads ? (int)threadIdx.x % units : (int)threadIdx.x;
+    if (w0 >= slots) return;
+    const int sw = g.sw();
+    for (int u = u0; u < units; u += kIm2colThreads) {
+        int off[UW];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int zc = z4 + j;
+        for (int j = 0; j < UW; ++j) {
+            const int zc = u * UW + j;
+            const int c = zc / KK, r = zc - c * KK;
+            const int ho = r / KW, wo = r - ho * KW;
+            off[j] = (c * KH + ho) * Wp + wo + w0 * sw;
+        }
+        float* out = orow + (long)w0 * Z + u * UW;
+        const int dstep = slots * sw;
+        const long ostep = (long)slots * Z;
+        for (int w = w0; w < n; w += slots) {
+            if (VEC) {
+                *reinterpret_cast<float4*>(out) =
+                    make_float4(tile[off[0]], tile[off[UW > 1 ? 1 : 0]], tile[off[UW > 2 ? 2 : 0]], tile[off[UW > 3 ? 3 : 0]]);
+            } else {
+                out[0] = tile[off[0]];
+            }
+#pragma unroll
+            for (int j = 0; j < UW; ++j) off[j] += dstep;
+            out += ostep;
+        }
+    }
+}
+
+// Pipelined variant: a workgroup owns one output row (b, h) -- one contiguous
+// region of the column buffer -- and walks its channel chunks.  While it
+// streams chunk i out of one LDS buffer, the global loads of chunk i+1 are in
+// flight into registers and are parked in the other buffer afterwards; one
+// barrier per chunk.  The staging offsets of a thread are the same for every
+// chunk and are computed once.
+constexpr int kIm2colNI = 12;                            // staged floats per thread and chunk
+constexpr int kIm2colBuf = kIm2colNI * kIm2colThreads;   // floats per LDS buffer (12 KiB)
+
+template <class G, bool VEC>
+__global__ __launch_bounds__(kIm2colThreads) void im2col_pipe_kernel(
+    G g, const float* __restrict__ im, float* __restrict__ col, int C, int H, int W, int m, int n,
+    int chunk, int nchunks) {
+    extern __shared__ float tile[];  // 2 x [chunk*kh][Wp]
+    constexpr int UW = VEC ? 4 : 1;
+    constexpr int NI = kIm2colNI;
+    const int KH = g.kh(), KW = g.kw(), KK = KH * KW;
+    const int Wp = W + 2 * g.pw();
+    const int rowlen = KH * Wp;                  // staged floats per channel
+    const int buflen = chunk * rowlen;           // <= kIm2colBuf
+    const long bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int h = (int)(bid % m);
+    const long b = bid / m;
+    const int hbase = h * g.sh() - g.ph();
+    const long plane = (long)H * W;
+
+    int soff[NI];                                // image offset inside the chunk, or -1 for padding
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int e = threadIdx.x + i * kIm2colThreads;
+        const int c = e / rowlen, rem = e - c * rowlen;
+        const int ho = rem / Wp, x = rem - ho * Wp;
+        const int hp = hbase + ho, wp = x - g.pw();
+        soff[i] = (e < buflen && hp >= 0 && hp < H && wp >= 0 && wp < W) ? (int)(c * plane + hp * W + wp) : -1;
+    }
+    float reg[NI];
+    auto load = [&](int ck) {
+        const int c0 = ck * chunk;
+        const int lim = min(chunk, C - c0) * rowlen;
+        const float* base = im + (b * C + c0) * plane;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int e = threadIdx.x + i * kIm2colThreads;
+            reg[i] = (soff[i] >= 0 && e < lim) ? base[soff[i]] : 0.0f;
+        }
+    };
+    auto stash = [&](float* buf) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int e = threadIdx.x + i * kIm2colThreads;
+            if (e < buflen) buf[e] = reg[i];
+        }
+    };
+
+    const long Z = (long)C * KK;
+    float* orow = col + ((b * m + h) * (long)n) * Z;
+    const int sw = g.sw();
+    load(0);
+    stash(tile);
+    __syncthreads();
+    for (int ck = 0; ck < nchunks; ++ck) {
+        const bool more = ck + 1 < nchunks;
+        if (more) load(ck + 1);
+        const float* cur = tile + (ck & 1) * buflen;
+        const int c0 = ck * chunk;
+        const int units = min(chunk, C - c0) * KK / UW;
+        const int slots = units < kIm2colThreads ? kIm2colThreads / units : 1;
+        const int w0 = units < kIm2colThreads ? (int)threadIdx.x / units : 0;
+        const int u0 = units < kIm2colThreads ? (int)threadIdx.x % units : (int)threadIdx.x;
+        if (w0 < slots) {
+            for (int u = u0; u < units; u += kIm2colThreads) {
+                int off[UW];
+#pragma unroll
+                for (int j = 0; j < UW; ++j) {
+                    const int zc = u * UW + j;
                     const int c = zc / KK, r = zc - c * KK;
                     const int ho = r / KW, wo = r - ho * KW;
-                    v[j] = tile[(c * KH + ho) * Wp + xbase + wo];
+                    off[j] = (c * KH + ho) * Wp + wo + w0 * sw;
                 }
-                *reinterpret_cast<float4*>(out + z4) = make_float4(v[0], v[1], v[2], v[3]);
-            }
-        } else {
-            for (int zc = lane; zc < zc_n; zc += kWave) {
-                const int c = zc / KK, r = zc - c * KK;
-                const int ho = r / KW, wo = r - ho * KW;
-                out[zc] = tile[(c * KH + ho) * Wp + xbase + wo];
+                float* out = orow + (long)w0 * Z + (long)c0 * KK + u * UW;
+                const int dstep = slots * sw;
+                const long ostep = (long)slots * Z;
+                for (int w = w0; w < n; w += slots) {
+                    if (VEC) {
+                        *reinterpret_cast<float4*>(out) =
+                            make_float4(cur[off[0]], cur[off[UW > 1 ? 1 : 0]], cur[off[UW > 2 ? 2 : 0]], cur[off[UW > 3 ? 3 : 0]]);
+                    } else {
+                        out[0] = cur[off[0]];
+                    }
+#pragma unroll
+                    for (int j = 0; j < UW; ++j) off[j] += dstep;
+                    out += ostep;
+                }
             }
         }
+        if (more) stash(tile + ((ck + 1) & 1) * buflen);
+        __syncthreads();
     }
 }
 
@@ -325,24 +450,46 @@ static int launch_im2col(G g, const float* im, long B, int C, int H, int W, int 
     const int KK = g.kh() * g.kw();
     const long Z = (long)C * KK;
     const int Wp = W + 2 * g.pw();
-    const long row_bytes = (long)g.kh() * Wp * sizeof(float);  // LDS per channel
-    const long lds_budget = 32 * 1024;
-    if (row_bytes <= 64 * 1024 && B * m < (1L << 31) / 64) {
-        int chunk = (int)(lds_budget / row_bytes);
-        if (chunk < 1) chunk = 1;
-        if (chunk > C) chunk = C;
-        // 16-byte stores need every chunk's z-run to start and end on a
-        // multiple of 4 floats: Z % 4 == 0 and (chunk*kh*kw) % 4 == 0.
-        bool vec = (Z % 4 == 0) && (reinterpret_cast<uintptr_t>(col) % 16 == 0);
+    const long rowlen = (long)g.kh() * Wp;                // staged floats per channel
+    const bool aligned = (Z % 4 == 0) && (reinterpret_cast<uintptr_t>(col) % 16 == 0);
+    const int step = 4 / gcd4(KK);       // smallest channel count whose z-run is a multiple of 4 floats
+    if (B * m * n * Z == 0) return CGT_AMD_OK;
+
+    // 1. pipelined kernel: a chunk of channels must fit one staging buffer
+    const long cap = kIm2colBuf;
+    if (rowlen <= cap && B * m < (1L << 31) && C * (long)H * W < (1L << 31)) {
+        int chunk = (int)std::min((long)C, cap / rowlen);
+        bool vec = aligned;
         if (vec && chunk < C) {
-            const int step = 4 / gcd4(KK);       // smallest channel count with (step*KK) % 4 == 0
+            if (chunk >= step) chunk = chunk / step * step;
+            else vec = false;
+        }
+        const int nchunks = (int)cdiv(C, chunk);
+        const size_t lds = 2 * (size_t)chunk * rowlen * sizeof(float);
+        const long blocks = B * m;
+        if (vec)
+            im2col_pipe_kernel<G, true><<<dim3((unsigned)blocks), dim3(kIm2colThreads), lds, st>>>(
+                g, im, col, C, H, W, m, n, chunk, nchunks);
+        else
+            im2col_pipe_kernel<G, false><<<dim3((unsigned)blocks), dim3(kIm2colThreads), lds, st>>>(
+                g, im, col, C, H, W, m, n, chunk, nchunks);
+        CGT_LAUNCH_CHECK("im2col_pipe_kernel");
+        return CGT_AMD_OK;
+    }
+
+    // 2. wide rows: one workgroup per (b, h, chunk), rows staged in up to 48 KiB of LDS
+    const long row_bytes = rowlen * (long)sizeof(float);
+    const long lds_budget = 48 * 1024;
+    if (row_bytes <= lds_budget && B * m < (1L << 31) / 64) {
+        int chunk = (int)std::min((long)C, lds_budget / row_bytes);
+        bool vec = aligned;
+        if (vec && chunk < C) {
             if (chunk >= step) chunk = chunk / step * step;
             else vec = false;
         }
         const int nchunks = (int)cdiv(C, chunk);
         const size_t lds = (size_t)chunk * row_bytes;
         const long blocks = B * m * nchunks;
-        if (blocks == 0) return CGT_AMD_OK;
         if (vec)
             im2col_rows_kernel<G, true><<<dim3((unsigned)blocks), dim3(kIm2colThreads), lds, st>>>(
                 g, im, col, C, H, W, m, n, chunk, nchunks);
@@ -352,8 +499,9 @@ static int launch_im2col(G g, const float* im, long B, int C, int H, int W, int 
         CGT_LAUNCH_CHECK("im2col_rows_kernel");
         return CGT_AMD_OK;
     }
+
+    // 3. anything else: one thread per output element
     const long total = B * m * n * Z;
-    if (total == 0) return CGT_AMD_OK;
     long blocks = cdiv(total, 256);
     if (blocks > 1 << 20) blocks = 1 << 20;
     im2col_direct_kernel<G><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(g, im, col, total, C, H, W, m, n);

@@ -101,6 +101,8 @@ IM2COL_CASES = [
     ((1, 20, 17, 70), (3, 3), (0, 0), (1, 1)),     # two column tiles, partial row tile
     ((1, 16, 56, 56), (3, 3), (1, 1), (1, 1)),
     ((1, 3, 100, 300), (11, 11), (0, 0), (4, 4)),  # three column tiles at stride 4
+    ((1, 2, 5, 2000), (3, 3), (1, 1), (1, 1)),     # rows longer than one pipelined staging buffer
+    ((2, 40, 9, 30), (3, 3), (1, 1), (1, 1)),      # several channel chunks, last one partial
 ]
 
 

@@ -1,28 +1,40 @@
 // fp32 GEMM on the gfx950 matrix cores: C[M,N] = op(A) . op(B), row-major.
 //
-// Tiling: a 256-thread workgroup (4 wavefronts, 2x2) owns a 128x128 tile of C;
-// each wavefront owns 64x64 = 2x2 blocks of v_mfma_f32_32x32x2_f32 (true fp32
-// in, fp32 accumulate; 64 accumulator registers per lane).  K is walked in
-// slices of 16 through double-buffered LDS tiles: while the matrix cores work
-// on slice t from LDS buffer t&1, the global loads of slice t+1 are in flight
-// into registers and are written to the other buffer afterwards -- one
-// barrier per slice.
+// Tiling: a 256-thread workgroup (4 wavefronts) owns a BM x BN tile of C; each
+// wavefront owns TM x TN blocks of v_mfma_f32_32x32x2_f32 (true fp32 in, fp32
+// accumulate, 16 accumulator registers per block and lane).  The default is
+// 128x128 with 2x2 wavefronts of 2x2 blocks; narrow outputs (the conv GEMMs
+// have N = 32 / 64 / 96 filters, or M = 96 for the weight gradient) use
+// 128 x {32,64,96} with the wavefronts stacked along M, or 96 x 128 with the
+// wavefronts stacked along N, so no matrix-core work is spent on padding.
 //
-// LDS layouts, chosen so that both the 16-byte global loads and the fragment
-// reads are contiguous:
+// K is walked in slices of 16 through double-buffered LDS tiles: while the
+// matrix cores work on slice t from LDS buffer t&1, the global loads of slice
+// t+1 are in flight into registers and are written to the other buffer
+// afterwards -- one barrier per slice.
+//
+// LDS layouts, chosen so that both the global loads and the fragment reads are
+// contiguous:
 //   operand stored k-contiguous in memory (A not transposed, B transposed):
 //       tile[row][k], row stride 20 floats; a lane reads its four k values of
-//       an 8-wide k group with one 16-byte LDS read, conflict-free;
+//       an 8-wide k group with one 16-byte LDS read;
 //   operand stored row-contiguous (A transposed, B not transposed):
-//       tile[k][row], row stride 132 floats; four 4-byte reads per k group.
+//       tile[k][row], row stride ROWS+4 floats; four 4-byte reads per k group.
 // Inside an 8-wide k group MFMA step i takes k = 4*half + i from lane half
 // `half` (lanes 0-31 / 32-63).  A and B use the same assignment, so the
 // products match; only the summation order inside the group differs from
 // k-ascending.
 //
+// Global loads are 16 bytes per lane when the leading dimension and base
+// address allow it; otherwise a second instantiation reads 4 bytes per lane
+// with consecutive lanes on consecutive addresses (im2col buffers have
+// Z = 363 or 75 floats per row).
+//
 // Skinny outputs (few tiles, long K: the conv weight gradient) are split along
 // K into a workspace of partial tiles, reduced afterwards in a fixed order, so
-// the result is deterministic.
+// the result is deterministic.  The grid is one-dimensional and ordered so
+// that workgroups sharing an operand panel land on the same XCD (same L2) at
+// about the same time.
 #include "common.h"
 #include <algorithm>
 #include <mutex>
@@ -32,12 +44,9 @@ namespace cgt_amd {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 128, BN = 128, KT = 16;
+constexpr int KT = 16;
 constexpr int kGemmThreads = 256;
-constexpr int LDK = KT + 4;    // [128][LDK]
-constexpr int LDM = BM + 4;    // [KT][LDM]
-constexpr int kTileFloats = (BM * LDK > KT * LDM) ? BM * LDK : KT * LDM;
-static_assert(BM == BN, "operand tiles share one layout");
+constexpr int LDK = KT + 4;    // row stride of a k-contiguous tile [ROWS][LDK]
 
 struct GemmArgs {
     const float* A;
@@ -47,63 +56,98 @@ struct GemmArgs {
     long sA, sB, sC;   // batch strides (elements)
     int M, N, K;
     int tiles_m, tiles_n;
+    int batch;
     int splits;        // > 1: partial products go to ws[split][M][N]
     int kchunk;        // K range per split, multiple of KT
     float* ws;
-    int vecA, vecB;    // 16-byte global loads allowed for A / B
 };
 
-// One 128 x KT operand tile, 2 float4 per thread.
+// One ROWS x KT operand tile.
 // KC: element (r, k) lives at p[r*ld + k]; otherwise at p[k*ld + r].
-template <bool KC>
+// VEC: 16-byte global loads (needs ld % 4 == 0 and a 16-byte aligned base).
+template <bool KC, int ROWS, bool VEC>
 struct OperandTile {
-    float4 v[2];
+    static constexpr int LDM = ROWS + 4;
+    static constexpr int kFloats = KC ? ROWS * LDK : KT * LDM;
+    static constexpr int kElems = ROWS * KT;
+    static constexpr int kPerThread = (kElems + kGemmThreads - 1) / kGemmThreads;   // 8 for 128 rows
+    static constexpr int NV = (kPerThread + 3) / 4;
+    float v[NV * 4];
 
     __device__ __forceinline__ void load(const float* __restrict__ p, long ld, int r0, int R,
-                                         int k0, int kend, bool vec) {
+                                         int k0, int kend) {
+        if (VEC) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int idx = threadIdx.x + i * kGemmThreads;
-            if (KC) {
-                const int row = r0 + (idx >> 2), k = k0 + (idx & 3) * 4;
-                const float* src = p + (long)row * ld + k;
-                if (vec && row < R && k + 3 < kend) {
-                    v[i] = *reinterpret_cast<const float4*>(src);
-                } else {
-                    float t[4] = {0.f, 0.f, 0.f, 0.f};
-                    if (row < R) {
+            for (int i = 0; i < NV; ++i) {
+                const int idx = threadIdx.x + i * kGemmThreads;     // float4 index
+                float t[4] = {0.f, 0.f, 0.f, 0.f};
+                if (idx * 4 < kElems) {
+                    if (KC) {
+                        const int row = r0 + (idx >> 2), k = k0 + (idx & 3) * 4;
+                        const float* src = p + (long)row * ld + k;
+                        if (row < R && k + 3 < kend) {
+                            const float4 q = *reinterpret_cast<const float4*>(src);
+                            t[0] = q.x; t[1] = q.y; t[2] = q.z; t[3] = q.w;
+                        } else if (row < R) {
 #pragma unroll
-                        for (int j = 0; j < 4; ++j)
-                            if (k + j < kend) t[j] = src[j];
+                            for (int j = 0; j < 4; ++j)
+                                if (k + j < kend) t[j] = src[j];
+                        }
+                    } else {
+                        const int k = k0 + idx / (ROWS / 4), row = r0 + (idx % (ROWS / 4)) * 4;
+                        const float* src = p + (long)k * ld + row;
+                        if (k < kend && row + 3 < R) {
+                            const float4 q = *reinterpret_cast<const float4*>(src);
+                            t[0] = q.x; t[1] = q.y; t[2] = q.z; t[3] = q.w;
+                        } else if (k < kend) {
+#pragma unroll
+                            for (int j = 0; j < 4; ++j)
+                                if (row + j < R) t[j] = src[j];
+                        }
                     }
-                    v[i] = make_float4(t[0], t[1], t[2], t[3]);
                 }
-            } else {
-                const int k = k0 + (idx >> 5), row = r0 + (idx & 31) * 4;
-                const float* src = p + (long)k * ld + row;
-                if (vec && k < kend && row + 3 < R) {
-                    v[i] = *reinterpret_cast<const float4*>(src);
-                } else {
-                    float t[4] = {0.f, 0.f, 0.f, 0.f};
-                    if (k < kend) {
 #pragma unroll
-                        for (int j = 0; j < 4; ++j)
-                            if (row + j < R) t[j] = src[j];
+                for (int j = 0; j < 4; ++j) v[i * 4 + j] = t[j];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kPerThread; ++i) {
+                const int idx = threadIdx.x + i * kGemmThreads;     // element index
+                float t = 0.f;
+                if (idx < kElems) {
+                    if (KC) {
+                        const int row = r0 + (idx >> 4), k = k0 + (idx & 15);
+                        if (row < R && k < kend) t = p[(long)row * ld + k];
+                    } else {
+                        const int k = k0 + idx / ROWS, row = r0 + idx % ROWS;
+                        if (k < kend && row < R) t = p[(long)k * ld + row];
                     }
-                    v[i] = make_float4(t[0], t[1], t[2], t[3]);
                 }
+                v[i] = t;
             }
         }
     }
 
     __device__ __forceinline__ void store(float* __restrict__ tile) const {
+        if (VEC) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int idx = threadIdx.x + i * kGemmThreads;
-            if (KC)
-                *reinterpret_cast<float4*>(tile + (idx >> 2) * LDK + (idx & 3) * 4) = v[i];
-            else
-                *reinterpret_cast<float4*>(tile + (idx >> 5) * LDM + (idx & 31) * 4) = v[i];
+            for (int i = 0; i < NV; ++i) {
+                const int idx = threadIdx.x + i * kGemmThreads;
+                if (idx * 4 < kElems) {
+                    float* dst = KC ? tile + (idx >> 2) * LDK + (idx & 3) * 4
+                                    : tile + (idx / (ROWS / 4)) * LDM + (idx % (ROWS / 4)) * 4;
+                    *reinterpret_cast<float4*>(dst) = make_float4(v[i * 4], v[i * 4 + 1], v[i * 4 + 2], v[i * 4 + 3]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kPerThread; ++i) {
+                const int idx = threadIdx.x + i * kGemmThreads;
+                if (idx < kElems) {
+                    if (KC) tile[(idx >> 4) * LDK + (idx & 15)] = v[i];
+                    else tile[(idx / ROWS) * LDM + idx % ROWS] = v[i];
+                }
+            }
         }
     }
 
@@ -129,18 +173,37 @@ __device__ __forceinline__ int xcd_remap(int id, int n) {
     return xcd * q + min(xcd, r) + local;
 }
 
-template <bool AKC, bool BKC>
+// WGM x WGN wavefronts, each TM x TN blocks of 32x32.
+template <bool AKC, bool BKC, bool VEC, int WGM, int WGN, int TM, int TN>
 __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
-    __shared__ __attribute__((aligned(16))) float As[2][kTileFloats];
-    __shared__ __attribute__((aligned(16))) float Bs[2][kTileFloats];
+    static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
+    constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
+    typedef OperandTile<AKC, BM, VEC> TileA;
+    typedef OperandTile<BKC, BN, VEC> TileB;
+    __shared__ __attribute__((aligned(16))) float As[2][TileA::kFloats];
+    __shared__ __attribute__((aligned(16))) float Bs[2][TileB::kFloats];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WGN, wn = wave % WGN;
     const int l32 = lane & 31, half = lane >> 5;
 
+    // linear workgroup id -> (batch, split, tile)
+    const int tiles = a.tiles_m * a.tiles_n;
+    int batch = 0, split = 0, lid;
+    if (a.splits > 1) {
+        // groups of 8 splits: the tiles of one split share its K range of both
+        // operands, so give them ids that are equal mod 8 (same XCD)
+        const int per_group = kNumXCD * tiles;
+        const int grp = blockIdx.x / per_group, r = blockIdx.x - grp * per_group;
+        const int in_grp = min(kNumXCD, a.splits - grp * kNumXCD);
+        split = grp * kNumXCD + r % in_grp;
+        lid = r / in_grp;
+    } else {
+        batch = blockIdx.x / tiles;
+        lid = xcd_remap(blockIdx.x - batch * tiles, tiles);
+    }
     // tile order: groups of 8 tile rows, column-major inside a group, so tiles
     // that run together share A row panels and B column panels in L2
-    const int lid = xcd_remap(blockIdx.x, a.tiles_m * a.tiles_n);
     constexpr int GM = 8;
     const int per_group = GM * a.tiles_n;
     const int group = lid / per_group, in_group = lid - group * per_group;
@@ -149,27 +212,25 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
     const int tm = first_m + in_group % gsz, tn = in_group / gsz;
     const int m0 = tm * BM, n0 = tn * BN;
 
-    const int z = blockIdx.y;
-    const int batch = z / a.splits, split = z - batch * a.splits;
     const int kbeg = split * a.kchunk;
     const int kend = min(a.K, kbeg + a.kchunk);
     const float* A = a.A + batch * a.sA;
     const float* B = a.B + batch * a.sB;
 
-    v16f acc[2][2];
+    v16f acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
     const int nk = (kend - kbeg + KT - 1) / KT;
-    OperandTile<AKC> ta;
-    OperandTile<BKC> tb;
+    TileA ta;
+    TileB tb;
     if (nk > 0) {
-        ta.load(A, a.lda, m0, a.M, kbeg, kend, a.vecA);
-        tb.load(B, a.ldb, n0, a.N, kbeg, kend, a.vecB);
+        ta.load(A, a.lda, m0, a.M, kbeg, kend);
+        tb.load(B, a.ldb, n0, a.N, kbeg, kend);
         ta.store(As[0]);
         tb.store(Bs[0]);
     }
@@ -179,25 +240,24 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
         const bool more = kt + 1 < nk;
         if (more) {
             const int k0 = kbeg + (kt + 1) * KT;
-            ta.load(A, a.lda, m0, a.M, k0, kend, a.vecA);
-            tb.load(B, a.ldb, n0, a.N, k0, kend, a.vecB);
+            ta.load(A, a.lda, m0, a.M, k0, kend);
+            tb.load(B, a.ldb, n0, a.N, k0, kend);
         }
         const float* as = As[cur];
         const float* bs = Bs[cur];
 #pragma unroll
         for (int kk = 0; kk < KT / 8; ++kk) {
-            float af[2][4], bf[2][4];
+            float af[TM][4], bf[TN][4];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                OperandTile<AKC>::frag(as, wm * 64 + i * 32 + l32, kk, half, af[i]);
-                OperandTile<BKC>::frag(bs, wn * 64 + i * 32 + l32, kk, half, bf[i]);
-            }
+            for (int i = 0; i < TM; ++i) TileA::frag(as, (wm * TM + i) * 32 + l32, kk, half, af[i]);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) TileB::frag(bs, (wn * TN + j) * 32 + l32, kk, half, bf[j]);
 #pragma unroll
             for (int s = 0; s < 4; ++s)
 #pragma unroll
-                for (int i = 0; i < 2; ++i)
+                for (int i = 0; i < TM; ++i)
 #pragma unroll
-                    for (int j = 0; j < 2; ++j)
+                    for (int j = 0; j < TN; ++j)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][s], bf[j][s],
                                                                          acc[i][j], 0, 0, 0);
         }
@@ -219,14 +279,14 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
         ldo = a.ldc;
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int col = n0 + wn * 64 + j * 32 + l32;
+        for (int j = 0; j < TN; ++j) {
+            const int col = n0 + (wn * TN + j) * 32 + l32;
             if (col >= a.N) continue;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int row = m0 + wm * 64 + i * 32 + 8 * (e / 4) + 4 * half + (e % 4);
+                const int row = m0 + (wm * TM + i) * 32 + 8 * (e / 4) + 4 * half + (e % 4);
                 if (row < a.M) out[(long)row * ldo + col] = acc[i][j][e];
             }
         }
@@ -272,6 +332,33 @@ static float* get_workspace(void* stream, size_t bytes) {
 
 static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
 
+struct TileShape {
+    int bm, bn;
+};
+
+// Tile shapes on offer; the 128x128 default comes first and wins ties.
+static const TileShape kShapes[] = {{128, 128}, {128, 96}, {128, 64}, {128, 32}, {96, 128}};
+
+template <bool AKC, bool BKC, bool VEC>
+static void launch_shape(int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
+    dim3 block(kGemmThreads);
+    switch (shape) {
+        case 0: sgemm_kernel<AKC, BKC, VEC, 2, 2, 2, 2><<<grid, block, 0, st>>>(a); break;
+        case 1: sgemm_kernel<AKC, BKC, VEC, 4, 1, 1, 3><<<grid, block, 0, st>>>(a); break;
+        case 2: sgemm_kernel<AKC, BKC, VEC, 4, 1, 1, 2><<<grid, block, 0, st>>>(a); break;
+        case 3: sgemm_kernel<AKC, BKC, VEC, 4, 1, 1, 1><<<grid, block, 0, st>>>(a); break;
+        default: sgemm_kernel<AKC, BKC, VEC, 1, 4, 3, 1><<<grid, block, 0, st>>>(a); break;
+    }
+}
+
+template <bool VEC>
+static void launch_trans(int tA, int tB, int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
+    if (!tA && !tB) launch_shape<true, false, VEC>(shape, grid, st, a);
+    else if (!tA && tB) launch_shape<true, true, VEC>(shape, grid, st, a);
+    else if (tA && !tB) launch_shape<false, false, VEC>(shape, grid, st, a);
+    else launch_shape<false, true, VEC>(shape, grid, st, a);
+}
+
 static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const float* A, long lda,
                          long sA, const float* B, long ldb, long sB, float* C, long ldc, long sC,
                          void* stream) {
@@ -280,21 +367,31 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     CGT_ARG_CHECK(A || K == 0, "sgemm: null A");
     CGT_ARG_CHECK(B || K == 0, "sgemm: null B");
     CGT_ARG_CHECK(C, "sgemm: null C");
-    CGT_ARG_CHECK(M < (1L << 31) - BM && N < (1L << 31) - BN && K < (1L << 31) - KT && P < 65536,
+    CGT_ARG_CHECK(M < (1L << 31) - 128 && N < (1L << 31) - 128 && K < (1L << 31) - KT && P < 65536,
                   "sgemm: size too large");
     CGT_ARG_CHECK(lda >= (tA ? M : K) && ldb >= (tB ? K : N) && ldc >= N,
                   "sgemm: leading dimension too small (lda=%ld ldb=%ld ldc=%ld)", lda, ldb, ldc);
+    // tile shape: least padded work, ties to the earlier (larger) shape
+    int shape = 0;
+    double best = 0;
+    for (int i = 0; i < (int)(sizeof(kShapes) / sizeof(kShapes[0])); ++i) {
+        const double work = (double)(cdiv(M, kShapes[i].bm) * kShapes[i].bm) *
+                            (double)(cdiv(N, kShapes[i].bn) * kShapes[i].bn);
+        if (i == 0 || work < best * 0.97) {
+            best = work;
+            shape = i;
+        }
+    }
     GemmArgs a;
     a.A = A; a.B = B; a.C = C;
     a.lda = lda; a.ldb = ldb; a.ldc = ldc;
     a.sA = sA; a.sB = sB; a.sC = sC;
     a.M = (int)M; a.N = (int)N; a.K = (int)K;
-    a.tiles_m = (int)cdiv(M, BM);
-    a.tiles_n = (int)cdiv(N, BN);
+    a.tiles_m = (int)cdiv(M, kShapes[shape].bm);
+    a.tiles_n = (int)cdiv(N, kShapes[shape].bn);
+    a.batch = (int)P;
     const long tiles = (long)a.tiles_m * a.tiles_n;
-    CGT_ARG_CHECK(tiles < (1L << 31), "sgemm: too many tiles");
-    a.vecA = (lda % 4 == 0 && sA % 4 == 0 && aligned16(A)) ? 1 : 0;
-    a.vecB = (ldb % 4 == 0 && sB % 4 == 0 && aligned16(B)) ? 1 : 0;
+    const bool vec = lda % 4 == 0 && sA % 4 == 0 && aligned16(A) && ldb % 4 == 0 && sB % 4 == 0 && aligned16(B);
     a.splits = 1;
     a.kchunk = (int)(cdiv(std::max(K, 1L), KT) * KT);
     a.ws = nullptr;
@@ -315,12 +412,12 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
             }
         }
     }
+    const long wgs = tiles * P * a.splits;
+    CGT_ARG_CHECK(wgs < (1L << 31), "sgemm: too many workgroups");
     hipStream_t st = as_stream(stream);
-    dim3 grid((unsigned)tiles, (unsigned)(P * a.splits)), block(kGemmThreads);
-    if (!tA && !tB) sgemm_kernel<true, false><<<grid, block, 0, st>>>(a);
-    else if (!tA && tB) sgemm_kernel<true, true><<<grid, block, 0, st>>>(a);
-    else if (tA && !tB) sgemm_kernel<false, false><<<grid, block, 0, st>>>(a);
-    else sgemm_kernel<false, true><<<grid, block, 0, st>>>(a);
+    dim3 grid((unsigned)wgs);
+    if (vec) launch_trans<true>(tA, tB, shape, grid, st, a);
+    else launch_trans<false>(tA, tB, shape, grid, st, a);
     CGT_LAUNCH_CHECK("sgemm_kernel");
     if (a.splits > 1) {
         const long MN = M * N;

@@ -21,30 +21,6 @@
 
 namespace cgt_amd {
 
-// Geometry known at compile time (hot shapes) ...
-template <int KH, int KW, int PH, int PW, int SH, int SW>
-struct StaticGeom {
-    static constexpr bool is_static = true;
-    static constexpr int kKH = KH, kKW = KW, kPH = PH, kPW = PW, kSH = SH, kSW = SW;
-    __host__ __device__ constexpr int kh() const { return KH; }
-    __host__ __device__ constexpr int kw() const { return KW; }
-    __host__ __device__ constexpr int ph() const { return PH; }
-    __host__ __device__ constexpr int pw() const { return PW; }
-    __host__ __device__ constexpr int sh() const { return SH; }
-    __host__ __device__ constexpr int sw() const { return SW; }
-};
-// ... or only at run time (anything else).
-struct DynGeom {
-    static constexpr bool is_static = false;
-    int kh_, kw_, ph_, pw_, sh_, sw_;
-    __host__ __device__ int kh() const { return kh_; }
-    __host__ __device__ int kw() const { return kw_; }
-    __host__ __device__ int ph() const { return ph_; }
-    __host__ __device__ int pw() const { return pw_; }
-    __host__ __device__ int sh() const { return sh_; }
-    __host__ __device__ int sw() const { return sw_; }
-};
-
 constexpr int kIm2colThreads = 256;
 constexpr int kIm2colWaves = kIm2colThreads / kWave;
 

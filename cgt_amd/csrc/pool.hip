@@ -16,15 +16,17 @@
 
 namespace cgt_amd {
 
-struct PoolGeom {
-    int kh, kw, ph, pw, sh, sw;
-};
-
 constexpr int kPoolThreads = 256;
 
-// planes_per_wg planes per workgroup; LDS holds their inputs.
+// floor(n / d) for 0 <= n < 2^21 with rcp = 1.0f / d: (n + 0.5) / d is at least
+// 0.5/d away from every integer, more than the float rounding error.
+__device__ __forceinline__ int fastdiv(int n, float rcp) { return (int)(((float)n + 0.5f) * rcp); }
+
+// planes_per_wg planes per workgroup; LDS holds their inputs; one thread per
+// pooled cell.
+template <class G>
 __global__ __launch_bounds__(kPoolThreads) void max_pool_fwd_kernel(
-    PoolGeom g, const float* __restrict__ bottom, float* __restrict__ top, int* __restrict__ mask,
+    G g, const float* __restrict__ bottom, float* __restrict__ top, int* __restrict__ mask,
     long nplanes, int H, int W, int PH, int PW, int planes_per_wg) {
     extern __shared__ float tile[];
     const long p0 = (long)blockIdx.x * planes_per_wg;
@@ -36,14 +38,15 @@ __global__ __launch_bounds__(kPoolThreads) void max_pool_fwd_kernel(
     for (int i = threadIdx.x; i < nin; i += kPoolThreads) tile[i] = src[i];
     __syncthreads();
 
-    const int nout = np * PP;
     float* tdst = top + p0 * PP;
     int* mdst = mask + p0 * PP;
+    const int nout = np * PP;
+    const float rPP = 1.0f / PP, rPW = 1.0f / PW;
     for (int o = threadIdx.x; o < nout; o += kPoolThreads) {
-        const int pl = o / PP, r = o - pl * PP;
-        const int y = r / PW, x = r - y * PW;
-        int hs = y * g.sh - g.ph, ws = x * g.sw - g.pw;
-        const int he = min(hs + g.kh, H), we = min(ws + g.kw, W);
+        const int pl = fastdiv(o, rPP), r = o - pl * PP;
+        const int y = fastdiv(r, rPW), x = r - y * PW;
+        int hs = y * g.sh() - g.ph(), ws = x * g.sw() - g.pw();
+        const int he = min(hs + g.kh(), H), we = min(ws + g.kw(), W);
         hs = max(hs, 0);
         ws = max(ws, 0);
         const float* pt = tile + pl * HW;
@@ -63,8 +66,9 @@ __global__ __launch_bounds__(kPoolThreads) void max_pool_fwd_kernel(
 }
 
 // Plane too large for LDS: read through the cache hierarchy.
+template <class G>
 __global__ __launch_bounds__(kPoolThreads) void max_pool_fwd_direct_kernel(
-    PoolGeom g, const float* __restrict__ bottom, float* __restrict__ top, int* __restrict__ mask,
+    G g, const float* __restrict__ bottom, float* __restrict__ top, int* __restrict__ mask,
     long total, int H, int W, int PH, int PW) {
     const long PP = (long)PH * PW;
     for (long o = (long)blockIdx.x * blockDim.x + threadIdx.x; o < total;
@@ -72,8 +76,8 @@ __global__ __launch_bounds__(kPoolThreads) void max_pool_fwd_direct_kernel(
         const long pl = o / PP;
         const int r = (int)(o - pl * PP);
         const int y = r / PW, x = r - y * PW;
-        int hs = y * g.sh - g.ph, ws = x * g.sw - g.pw;
-        const int he = min(hs + g.kh, H), we = min(ws + g.kw, W);
+        int hs = y * g.sh() - g.ph(), ws = x * g.sw() - g.pw();
+        const int he = min(hs + g.kh(), H), we = min(ws + g.kw(), W);
         hs = max(hs, 0);
         ws = max(ws, 0);
         const float* pt = bottom + pl * H * W;
@@ -97,9 +101,10 @@ __device__ __forceinline__ int floordiv(int a, int b) {  // b > 0
     return (a % b != 0 && a < 0) ? q - 1 : q;
 }
 
-// LDS holds mask and top_diff of the workgroup's planes.
+// LDS holds mask and top_diff of the workgroup's planes; one thread per input cell.
+template <class G>
 __global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_kernel(
-    PoolGeom g, const int* __restrict__ mask, const float* __restrict__ top_diff,
+    G g, const int* __restrict__ mask, const float* __restrict__ top_diff,
     float* __restrict__ bottom_diff, long nplanes, int H, int W, int PH, int PW,
     int planes_per_wg) {
     extern __shared__ float tile[];
@@ -116,26 +121,30 @@ __global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_kernel(
     }
     __syncthreads();
 
-    const int nin = np * HW;
     float* dst = bottom_diff + p0 * HW;
+    const int nin = np * HW;
+    const float rHW = 1.0f / HW, rW = 1.0f / W;
     for (int i = threadIdx.x; i < nin; i += kPoolThreads) {
-        const int pl = i / HW, cell = i - pl * HW;
-        const int h = cell / W, w = cell - h * W;
+        const int pl = fastdiv(i, rHW), cell = i - pl * HW;
+        const int h = fastdiv(cell, rW), w = cell - h * W;
         // windows covering (h, w): ph*sh - pad <= h < ph*sh - pad + kh
-        const int y0 = max(0, floordiv(h + g.ph - g.kh, g.sh) + 1), y1 = min(PH - 1, (h + g.ph) / g.sh);
-        const int x0 = max(0, floordiv(w + g.pw - g.kw, g.sw) + 1), x1 = min(PW - 1, (w + g.pw) / g.sw);
+        const int y0 = max(0, floordiv(h + g.ph() - g.kh(), g.sh()) + 1), y1 = min(PH - 1, (h + g.ph()) / g.sh());
+        const int x0 = max(0, floordiv(w + g.pw() - g.kw(), g.sw()) + 1), x1 = min(PW - 1, (w + g.pw()) / g.sw());
+        const float* tdp = td + pl * PP;
+        const int* mkp = mk + pl * PP;
         float acc = 0.0f;
         for (int y = y0; y <= y1; ++y)
             for (int x = x0; x <= x1; ++x) {
-                const int o = pl * PP + y * PW + x;
-                if (mk[o] == cell) acc += td[o];
+                const int o = y * PW + x;
+                if (mkp[o] == cell) acc += tdp[o];
             }
         dst[i] = acc;
     }
 }
 
+template <class G>
 __global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_direct_kernel(
-    PoolGeom g, const int* __restrict__ mask, const float* __restrict__ top_diff,
+    G g, const int* __restrict__ mask, const float* __restrict__ top_diff,
     float* __restrict__ bottom_diff, long total, int H, int W, int PH, int PW) {
     const long HW = (long)H * W, PP = (long)PH * PW;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
@@ -143,8 +152,8 @@ __global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_direct_kernel(
         const long pl = i / HW;
         const int cell = (int)(i - pl * HW);
         const int h = cell / W, w = cell - h * W;
-        const int y0 = max(0, floordiv(h + g.ph - g.kh, g.sh) + 1), y1 = min(PH - 1, (h + g.ph) / g.sh);
-        const int x0 = max(0, floordiv(w + g.pw - g.kw, g.sw) + 1), x1 = min(PW - 1, (w + g.pw) / g.sw);
+        const int y0 = max(0, floordiv(h + g.ph() - g.kh(), g.sh()) + 1), y1 = min(PH - 1, (h + g.ph()) / g.sh());
+        const int x0 = max(0, floordiv(w + g.pw() - g.kw(), g.sw()) + 1), x1 = min(PW - 1, (w + g.pw()) / g.sw());
         float acc = 0.0f;
         for (int y = y0; y <= y1; ++y)
             for (int x = x0; x <= x1; ++x) {
@@ -178,6 +187,56 @@ CGT_API long cgt_amd_pool_outsize(long H, int k, int pad, int stride) {
     return (num + stride - 1) / stride;
 }
 
+// Pool geometries compiled with constant index math: (kh, kw, ph, pw, sh, sw).
+#define CGT_STATIC_POOLS(X) \
+    X(2, 2, 0, 0, 2, 2)     \
+    X(3, 3, 0, 0, 2, 2)     \
+    X(3, 3, 1, 1, 2, 2)
+
+namespace cgt_amd {
+
+template <class G>
+static int launch_pool_fwd(G g, const float* bottom, long nplanes, long H, long W, long PH, long PW,
+                           float* top, int* mask, hipStream_t st) {
+    const long plane_bytes = H * W * (long)sizeof(float);
+    if (plane_bytes <= 48 * 1024) {
+        int ppw = (int)std::max(1L, (16 * 1024) / std::max(1L, plane_bytes));
+        const long blocks = cdiv(nplanes, ppw);
+        max_pool_fwd_kernel<G><<<dim3((unsigned)blocks), dim3(kPoolThreads), (size_t)ppw * plane_bytes, st>>>(
+            g, bottom, top, mask, nplanes, (int)H, (int)W, (int)PH, (int)PW, ppw);
+        CGT_LAUNCH_CHECK("max_pool_fwd_kernel");
+    } else {
+        const long total = nplanes * PH * PW;
+        long blocks = std::min(cdiv(total, (long)kPoolThreads), 1L << 20);
+        max_pool_fwd_direct_kernel<G><<<dim3((unsigned)blocks), dim3(kPoolThreads), 0, st>>>(
+            g, bottom, top, mask, total, (int)H, (int)W, (int)PH, (int)PW);
+        CGT_LAUNCH_CHECK("max_pool_fwd_direct_kernel");
+    }
+    return CGT_AMD_OK;
+}
+
+template <class G>
+static int launch_pool_bwd(G g, const int* mask, const float* top_diff, long nplanes, long H, long W,
+                           long PH, long PW, float* bottom_diff, hipStream_t st) {
+    const long out_bytes = PH * PW * 2 * (long)sizeof(float);  // top_diff + mask per plane
+    if (out_bytes <= 48 * 1024) {
+        int ppw = (int)std::max(1L, (16 * 1024) / out_bytes);
+        const long blocks = cdiv(nplanes, ppw);
+        max_pool_bwd_kernel<G><<<dim3((unsigned)blocks), dim3(kPoolThreads), (size_t)ppw * out_bytes, st>>>(
+            g, mask, top_diff, bottom_diff, nplanes, (int)H, (int)W, (int)PH, (int)PW, ppw);
+        CGT_LAUNCH_CHECK("max_pool_bwd_kernel");
+    } else {
+        const long total = nplanes * H * W;
+        long blocks = std::min(cdiv(total, (long)kPoolThreads), 1L << 20);
+        max_pool_bwd_direct_kernel<G><<<dim3((unsigned)blocks), dim3(kPoolThreads), 0, st>>>(
+            g, mask, top_diff, bottom_diff, total, (int)H, (int)W, (int)PH, (int)PW);
+        CGT_LAUNCH_CHECK("max_pool_bwd_direct_kernel");
+    }
+    return CGT_AMD_OK;
+}
+
+}  // namespace cgt_amd
+
 CGT_API int cgt_amd_max_pool_f32(const float* bottom, long N, long C, long H, long W, int kh,
                                  int kw, int ph, int pw, int sh, int sw, long PH, long PW,
                                  float* top, int* mask, void* stream) {
@@ -186,23 +245,13 @@ CGT_API int cgt_amd_max_pool_f32(const float* bottom, long N, long C, long H, lo
     const long nplanes = N * C;
     if (nplanes * PH * PW == 0) return CGT_AMD_OK;
     CGT_ARG_CHECK(bottom && top && mask, "max_pool: null pointer");
-    PoolGeom g{kh, kw, ph, pw, sh, sw};
     hipStream_t st = as_stream(stream);
-    const long plane_bytes = H * W * (long)sizeof(float);
-    if (plane_bytes <= 48 * 1024) {
-        int ppw = (int)std::max(1L, (16 * 1024) / std::max(1L, plane_bytes));
-        const long blocks = cdiv(nplanes, ppw);
-        max_pool_fwd_kernel<<<dim3((unsigned)blocks), dim3(kPoolThreads), (size_t)ppw * plane_bytes, st>>>(
-            g, bottom, top, mask, nplanes, (int)H, (int)W, (int)PH, (int)PW, ppw);
-        CGT_LAUNCH_CHECK("max_pool_fwd_kernel");
-    } else {
-        const long total = nplanes * PH * PW;
-        long blocks = std::min(cdiv(total, (long)kPoolThreads), 1L << 20);
-        max_pool_fwd_direct_kernel<<<dim3((unsigned)blocks), dim3(kPoolThreads), 0, st>>>(
-            g, bottom, top, mask, total, (int)H, (int)W, (int)PH, (int)PW);
-        CGT_LAUNCH_CHECK("max_pool_fwd_direct_kernel");
-    }
-    return CGT_AMD_OK;
+#define X(KH, KW, PH_, PW_, SH, SW)                                                     \
+    if (kh == KH && kw == KW && ph == PH_ && pw == PW_ && sh == SH && sw == SW)         \
+        return launch_pool_fwd(StaticGeom<KH, KW, PH_, PW_, SH, SW>(), bottom, nplanes, H, W, PH, PW, top, mask, st);
+    CGT_STATIC_POOLS(X)
+#undef X
+    return launch_pool_fwd(DynGeom{kh, kw, ph, pw, sh, sw}, bottom, nplanes, H, W, PH, PW, top, mask, st);
 }
 
 CGT_API int cgt_amd_max_pool_pullback_f32(const int* mask, const float* top_diff, long N, long C,
@@ -217,20 +266,10 @@ CGT_API int cgt_amd_max_pool_pullback_f32(const int* mask, const float* top_diff
     hipStream_t st = as_stream(stream);
     if (PH * PW == 0) return cgt_amd_fill_u32(bottom_diff, 0u, nplanes * H * W, stream);
     CGT_ARG_CHECK(mask && top_diff, "max_pool_pullback: null pointer");
-    PoolGeom g{kh, kw, ph, pw, sh, sw};
-    const long out_bytes = PH * PW * 2 * (long)sizeof(float);  // top_diff + mask per plane
-    if (out_bytes <= 48 * 1024) {
-        int ppw = (int)std::max(1L, (16 * 1024) / out_bytes);
-        const long blocks = cdiv(nplanes, ppw);
-        max_pool_bwd_kernel<<<dim3((unsigned)blocks), dim3(kPoolThreads), (size_t)ppw * out_bytes, st>>>(
-            g, mask, top_diff, bottom_diff, nplanes, (int)H, (int)W, (int)PH, (int)PW, ppw);
-        CGT_LAUNCH_CHECK("max_pool_bwd_kernel");
-    } else {
-        const long total = nplanes * H * W;
-        long blocks = std::min(cdiv(total, (long)kPoolThreads), 1L << 20);
-        max_pool_bwd_direct_kernel<<<dim3((unsigned)blocks), dim3(kPoolThreads), 0, st>>>(
-            g, mask, top_diff, bottom_diff, total, (int)H, (int)W, (int)PH, (int)PW);
-        CGT_LAUNCH_CHECK("max_pool_bwd_direct_kernel");
-    }
-    return CGT_AMD_OK;
+#define X(KH, KW, PH_, PW_, SH, SW)                                                     \
+    if (kh == KH && kw == KW && ph == PH_ && pw == PW_ && sh == SH && sw == SW)         \
+        return launch_pool_bwd(StaticGeom<KH, KW, PH_, PW_, SH, SW>(), mask, top_diff, nplanes, H, W, PH, PW, bottom_diff, st);
+    CGT_STATIC_POOLS(X)
+#undef X
+    return launch_pool_bwd(DynGeom{kh, kw, ph, pw, sh, sw}, mask, top_diff, nplanes, H, W, PH, PW, bottom_diff, st);
 }

@@ -98,7 +98,7 @@ class LayerOnGpu(object):
         nelem = lambda a: int(np.prod(a.shape))  # noqa: E731
         st = []
         s = stream
-        st.append(Stage("im2col", "im2col_rows_kernel", lambda: K.im2col(self.x, (r, c), pad, stride, out=self.col, stream=s),
+        st.append(Stage("im2col", "im2col_pipe_kernel", lambda: K.im2col(self.x, (r, c), pad, stride, out=self.col, stream=s),
                         4 * (nelem(self.x) + nelem(self.col)), "hbm"))
         st.append(Stage("gemm_fwd_NT", "sgemm_kernel<1,1>", lambda: K.mul22(self.col2, self.f_LZ, False, True, out=self.y_mnL, stream=s),
                         2 * Bmn * L * Z, "mfma"))
@@ -143,7 +143,7 @@ class LayerOnGpu(object):
                         2 * 4 * nelem(self.y), "hbm"))
         st.append(Stage("gemm_dgrad_NN", "sgemm_kernel<1,0>", lambda: K.mul22(self.gc2, self.f_LZ, False, False, out=self.gcol, stream=s),
                         2 * Bmn * L * Z, "mfma"))
-        st.append(Stage("col2im", "col2im_gather_kernel",
+        st.append(Stage("col2im", "col2im_stream_kernel",
                         lambda: K.col2im(self.gcol.reshape(B, m, n, Z), self.x.shape, (r, c), pad, stride, out=self.gx, stream=s),
                         4 * (nelem(self.x) + nelem(self.col)), "hbm"))
         st.append(Stage("gemm_wgrad_TN", "sgemm_kernel<0,0>", lambda: K.mul22(self.gc2, self.col2, True, False, out=self.gf, stream=s),

@@ -18,6 +18,7 @@
 #include "common.h"
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 
 namespace cgt_amd {
 
@@ -268,43 +269,49 @@ __global__ __launch_bounds__(256) void col2im_gather_kernel(
 }
 
 
-// LDS-staged col2im for compile-time geometry.
+// Streaming col2im for compile-time geometry (stride <= kernel).
 //
-// A workgroup owns (image b, CC channels, TH image rows, 64*WSUB image columns)
-// and keeps that tile's sums in registers: thread (wave, lane) owns the pixel
-// columns q = wave + 4*i (q -> channel q % CC, column block q / CC, column
-// wp0 + 64*block + lane) with TH accumulators each.  The column-buffer rows
-// that feed the tile are streamed through LDS from the highest h to the
-// lowest, one row per step, each as contiguous runs of CC*kh*kw floats
-// (coalesced, every byte of the buffer read once apart from the halo rows
-// between neighbouring tiles).  For a fixed pixel, descending h is ascending
-// kernel row ho and taps inside a row are taken in ascending wo, so the adds
-// happen in ascending z exactly as in the sequential reference loop.
-// All accumulator indices are compile-time after unrolling because tile rows
-// start on multiples of TH and TH % stride == 0.
-template <class G, int CC, int WSUB, int TH>
-__global__ __launch_bounds__(256) void col2im_rows_kernel(
+// A workgroup owns (image b, CC channels, a band of image rows, 64*WSUB image
+// columns).  Thread (wave, lane) owns the pixel columns q = wave + 4*i
+// (q -> channel q % CC, column block q / CC, column wp0 + 64*block + lane).
+// The column-buffer rows h that feed the band are streamed from the highest to
+// the lowest: row h adds into image rows h*sh - ph + ho, ho = 0..kh-1, so a
+// thread keeps a sliding window of kh accumulators per pixel column, indexed
+// by ho (compile-time after unrolling).  After row h the top sh rows of the
+// window can receive nothing more: they are written out and the window slides
+// down by sh.  For a fixed pixel, descending h is ascending ho and taps inside
+// a row are taken in ascending wo, so the adds happen in ascending z exactly
+// as in the sequential reference loop -- bit-identical, no atomics.
+//
+// Each row is staged through LDS as contiguous runs of CC*kh*kw floats
+// (coalesced; the buffer is read once apart from kh-sh halo rows per band and
+// the kw-sw halo columns per tile).  The global loads of row h-1 are issued
+// into registers before row h is consumed, so their latency is hidden.
+template <class G, int CC, int WSUB, bool VEC>
+__global__ __launch_bounds__(256) void col2im_stream_kernel(
     G g, const float* __restrict__ col, float* __restrict__ im, int C, int H, int W, int m, int n,
-    int tiles_h, int tiles_w, int nchunks, int vec) {
+    int band, int bands, int tiles_w, int nchunks) {
     constexpr int KH = G::kKH, KW = G::kKW, PH = G::kPH, PW = G::kPW, SH = G::kSH, SW = G::kSW;
+    static_assert(SH <= KH && SW <= KW, "streaming col2im needs stride <= kernel");
     constexpr int KK = KH * KW, RUN = CC * KK;
     constexpr int LD = RUN | 1;                       // odd row stride: conflict-free column reads
     constexpr int TW = 64 * WSUB;
     constexpr int NQ = (CC * WSUB + 3) / 4;
-    static_assert(TH % SH == 0, "tile rows must start on a stride multiple");
-    constexpr int H0 = (TH - 1 + PH) / SH;            // highest contributing row = hp0/SH + H0
-    constexpr int NH = (TH - 1 + KH - 1) / SH + 1;    // rows that can touch a tile
     constexpr int NT = (KW + SW - 1) / SW;            // taps per row and pixel
+    constexpr int NWB = (TW + KW - 2) / SW + 1;       // staged pixels per row, upper bound
+    // staged values per thread: float4 units of full runs (VEC) or single floats
+    constexpr int NP = VEC ? (NWB * (RUN / 4) + 255) / 256 : (NWB * RUN + 255) / 256;
     extern __shared__ float stage[];                  // [nw][LD]
 
-    long bid = blockIdx.x;
+    long bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int bd = (int)(bid % bands);                // bands of one image/chunk are neighbours
+    bid /= bands;
     const int wt = (int)(bid % tiles_w);
     bid /= tiles_w;
-    const int ht = (int)(bid % tiles_h);
-    bid /= tiles_h;
     const int ck = (int)(bid % nchunks);
     const long b = bid / nchunks;
-    const int hp0 = ht * TH, wp0 = wt * TW, c0 = ck * CC;
+    const int hp0 = bd * band, hp1 = min(H, hp0 + band);
+    const int wp0 = wt * TW, c0 = ck * CC;
     const int cc = min(CC, C - c0);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const long Z = (long)C * KK;
@@ -313,11 +320,13 @@ __global__ __launch_bounds__(256) void col2im_rows_kernel(
     const int w_lo = wl > 0 ? (wl + SW - 1) / SW : 0;
     const int w_hi = min(n - 1, (wp0 + TW - 1 + PW) / SW);
     const int nw = w_hi - w_lo + 1;
-    const int htop = hp0 / SH + H0;
+    const bool full = (cc == CC);                     // VEC is only launched when C % CC == 0
+    const int run = cc * KK;
+    const int total = VEC ? nw * (RUN / 4) : nw * run;
 
     int cq[NQ], wp[NQ];
     bool ok[NQ];
-    float acc[NQ][TH];
+    float acc[NQ][KH];
 #pragma unroll
     for (int i = 0; i < NQ; ++i) {
         const int q = wave + 4 * i;
@@ -325,82 +334,134 @@ __global__ __launch_bounds__(256) void col2im_rows_kernel(
         wp[i] = wp0 + (q / CC) * 64 + lane;
         ok[i] = (q < CC * WSUB) && (cq[i] < cc) && (wp[i] < W);
 #pragma unroll
-        for (int j = 0; j < TH; ++j) acc[i][j] = 0.0f;
+        for (int j = 0; j < KH; ++j) acc[i][j] = 0.0f;
     }
 
-#pragma unroll
-    for (int hi = 0; hi < NH; ++hi) {
-        const int h = htop - hi;
-        if (h < 0 || h >= m || nw <= 0) continue;     // uniform over the workgroup
+    // rows h_top .. h_bot cover every image row of the band; rows outside
+    // [0, m) contribute nothing but still slide the window
+    const int h_top = (hp1 - 1 + PH) / SH;
+    const int t_bot = hp0 + PH - (KH - 1);
+    const int h_bot = t_bot >= 0 ? (t_bot + SH - 1) / SH : -((-t_bot) / SH);
+
+    typename std::conditional<VEC, float4, float>::type pre[NP];
+    auto prefetch = [&](int h) {
+        if (h < 0 || h >= m || nw <= 0) return;
         const float* src = col + ((b * m + h) * (long)n + w_lo) * Z + (long)c0 * KK;
-        if (cc == CC) {
-            if (vec) {
-                for (int idx = threadIdx.x; idx < nw * (RUN / 4); idx += 256) {
-                    const int w = idx / (RUN / 4), z4 = (idx - w * (RUN / 4)) * 4;
-                    const float4 v = *reinterpret_cast<const float4*>(src + (long)w * Z + z4);
+#pragma unroll
+        for (int u = 0; u < NP; ++u) {
+            const int idx = threadIdx.x + u * 256;
+            if constexpr (VEC) {
+                const int w = idx / (RUN / 4), z4 = (idx - w * (RUN / 4)) * 4;
+                if (idx < total) pre[u] = *reinterpret_cast<const float4*>(src + (long)w * Z + z4);
+            } else {
+                const int w = full ? idx / RUN : idx / run;
+                const int zc = idx - w * run;
+                if (idx < total) pre[u] = src[(long)w * Z + zc];
+            }
+        }
+    };
+    auto park = [&]() {
+#pragma unroll
+        for (int u = 0; u < NP; ++u) {
+            const int idx = threadIdx.x + u * 256;
+            if constexpr (VEC) {
+                const int w = idx / (RUN / 4), z4 = (idx - w * (RUN / 4)) * 4;
+                if (idx < total) {
                     float* d = stage + w * LD + z4;
-                    d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+                    d[0] = pre[u].x; d[1] = pre[u].y; d[2] = pre[u].z; d[3] = pre[u].w;
                 }
             } else {
-                for (int idx = threadIdx.x; idx < nw * RUN; idx += 256) {
-                    const int w = idx / RUN, zc = idx - w * RUN;
-                    stage[w * LD + zc] = src[(long)w * Z + zc];
-                }
-            }
-        } else {
-            const int run = cc * KK;
-            for (int idx = threadIdx.x; idx < nw * run; idx += 256) {
-                const int w = idx / run, zc = idx - w * run;
-                stage[w * LD + zc] = src[(long)w * Z + zc];
+                const int w = full ? idx / RUN : idx / run;
+                const int zc = idx - w * run;
+                if (idx < total) stage[w * LD + zc] = pre[u];
             }
         }
-        __syncthreads();
+    };
+
+    prefetch(h_top);
+    for (int h = h_top; h >= h_bot; --h) {
+        const bool live = h >= 0 && h < m && nw > 0;      // uniform over the workgroup
+        if (live) {
+            park();
+            __syncthreads();
+        }
+        if (h > h_bot) prefetch(h - 1);
+        if (live) {
+#pragma unroll
+            for (int i = 0; i < NQ; ++i) {
+                if (!ok[i]) continue;
+                const int wpp = wp[i] + PW;
+                const int r = wpp % SW;
+#pragma unroll
+                for (int ho = 0; ho < KH; ++ho) {
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        const int wo = r + t * SW;
+                        const int ww = wpp - wo;
+                        const int w = ww / SW;
+                        if (wo < KW && ww >= 0 && w <= w_hi)
+                            acc[i][ho] += stage[(w - w_lo) * LD + (cq[i] * KH + ho) * KW + wo];
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        // image rows h*SH - PH + ho, ho >= KH - SH, are complete: write and slide
+        const int base = h * SH - PH;
 #pragma unroll
         for (int i = 0; i < NQ; ++i) {
-            if (!ok[i]) continue;
-            const int wpp = wp[i] + PW;
-            const int r = wpp % SW;
+            if (ok[i]) {
+                float* dst = im + ((b * C + c0 + cq[i]) * (long)H) * W + wp[i];
 #pragma unroll
-            for (int ho = 0; ho < KH; ++ho) {
-                const int j = (H0 - hi) * SH - PH + ho;   // compile-time after unrolling
-                if (j < 0 || j >= TH) continue;
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    const int wo = r + t * SW;
-                    const int ww = wpp - wo;
-                    const int w = ww / SW;
-                    if (wo < KW && ww >= 0 && w <= w_hi)
-                        acc[i][j] += stage[(w - w_lo) * LD + (cq[i] * KH + ho) * KW + wo];
+                for (int ho = KH - SH; ho < KH; ++ho) {
+                    const int hp = base + ho;
+                    if (hp >= hp0 && hp < hp1) dst[(long)hp * W] = acc[i][ho];
                 }
             }
+#pragma unroll
+            for (int ho = KH - 1; ho >= SH; --ho) acc[i][ho] = acc[i][ho - SH];
+#pragma unroll
+            for (int ho = 0; ho < SH; ++ho) acc[i][ho] = 0.0f;
         }
-        __syncthreads();
     }
-
+    // rows of the band below the lowest window (still open in the window)
+    const int base = (h_bot - 1) * SH - PH;
 #pragma unroll
     for (int i = 0; i < NQ; ++i) {
         if (!ok[i]) continue;
         float* dst = im + ((b * C + c0 + cq[i]) * (long)H) * W + wp[i];
 #pragma unroll
-        for (int j = 0; j < TH; ++j)
-            if (hp0 + j < H) dst[(long)(hp0 + j) * W] = acc[i][j];
+        for (int ho = SH; ho < KH; ++ho) {
+            const int hp = base + ho;
+            if (hp >= hp0 && hp < hp1) dst[(long)hp * W] = acc[i][ho];
+        }
     }
 }
 
-template <class G, int CC, int WSUB, int TH>
-static int launch_col2im_rows(G g, const float* col, long B, int C, int H, int W, int m, int n,
-                              float* im, hipStream_t st) {
+template <class G, int CC, int WSUB>
+static int launch_col2im_stream(G g, const float* col, long B, int C, int H, int W, int m, int n,
+                                float* im, hipStream_t st) {
     constexpr int KK = G::kKH * G::kKW, RUN = CC * KK, LD = RUN | 1, TW = 64 * WSUB;
-    const int tiles_h = (int)cdiv(H, TH), tiles_w = (int)cdiv(W, TW), nchunks = (int)cdiv(C, CC);
+    const int tiles_w = (int)cdiv(W, TW), nchunks = (int)cdiv(C, CC);
+    // bands: at least two workgroups per CU, but tall enough that the kh - sh
+    // halo rows stay a small fraction (measured: fewer, taller bands win)
+    const long per_band = B * nchunks * tiles_w;
+    long bands = std::max(1L, std::min(cdiv(512, per_band), (long)H / (4 * G::kKH)));
+    int band = (int)cdiv(cdiv(H, bands), G::kSH) * G::kSH;       // bands start on stride multiples
+    bands = cdiv(H, band);
     const long nwb = std::min((long)n, (long)(TW + G::kKW - 2) / G::kSW + 1);
     const size_t lds = (size_t)nwb * LD * sizeof(float);
-    const long blocks = B * nchunks * tiles_h * tiles_w;
+    const long blocks = per_band * bands;
     CGT_ARG_CHECK(blocks < (1L << 31) && lds <= 64 * 1024, "col2im: tile configuration out of range");
     const long Z = (long)C * KK;
-    const int vec = (RUN % 4 == 0 && Z % 4 == 0 && reinterpret_cast<uintptr_t>(col) % 16 == 0) ? 1 : 0;
-    col2im_rows_kernel<G, CC, WSUB, TH><<<dim3((unsigned)blocks), dim3(256), lds, st>>>(
-        g, col, im, C, H, W, m, n, tiles_h, tiles_w, nchunks, vec);
-    CGT_LAUNCH_CHECK("col2im_rows_kernel");
+    const bool vec = RUN % 4 == 0 && C % CC == 0 && reinterpret_cast<uintptr_t>(col) % 16 == 0;
+    if (vec)
+        col2im_stream_kernel<G, CC, WSUB, (RUN % 4 == 0)><<<dim3((unsigned)blocks), dim3(256), lds, st>>>(
+            g, col, im, C, H, W, m, n, band, (int)bands, tiles_w, nchunks);
+    else
+        col2im_stream_kernel<G, CC, WSUB, false><<<dim3((unsigned)blocks), dim3(256), lds, st>>>(
+            g, col, im, C, H, W, m, n, band, (int)bands, tiles_w, nchunks);
+    CGT_LAUNCH_CHECK("col2im_stream_kernel");
     return CGT_AMD_OK;
 }
 
@@ -485,31 +546,31 @@ static int launch_im2col(G g, const float* im, long B, int C, int H, int W, int 
     return CGT_AMD_OK;
 }
 
-// Tiling of col2im_rows_kernel per compile-time geometry: <channels per chunk,
-// 64-column blocks per tile, image rows per tile>.  Returns -1 when the shape
+// Tiling of col2im_stream_kernel per compile-time geometry: <channels per chunk,
+// 64-column blocks per tile>.  Returns -1 when the shape
 // is better served by the plain gather kernel.
 template <class G>
-static int try_col2im_rows(G, const float*, long, int, int, int, int, int, float*, hipStream_t) {
+static int try_col2im_stream(G, const float*, long, int, int, int, int, int, float*, hipStream_t) {
     return -1;
 }
-static int try_col2im_rows(StaticGeom<3, 3, 1, 1, 1, 1> g, const float* col, long B, int C, int H,
+static int try_col2im_stream(StaticGeom<3, 3, 1, 1, 1, 1> g, const float* col, long B, int C, int H,
                            int W, int m, int n, float* im, hipStream_t st) {
-    if (C >= 16 && W >= 24) return launch_col2im_rows<decltype(g), 16, 1, 14>(g, col, B, C, H, W, m, n, im, st);
+    if (C >= 8 && W >= 24) return launch_col2im_stream<decltype(g), 8, 1>(g, col, B, C, H, W, m, n, im, st);
     return -1;
 }
-static int try_col2im_rows(StaticGeom<3, 3, 0, 0, 1, 1> g, const float* col, long B, int C, int H,
+static int try_col2im_stream(StaticGeom<3, 3, 0, 0, 1, 1> g, const float* col, long B, int C, int H,
                            int W, int m, int n, float* im, hipStream_t st) {
-    if (C >= 16 && W >= 24) return launch_col2im_rows<decltype(g), 16, 1, 14>(g, col, B, C, H, W, m, n, im, st);
+    if (C >= 8 && W >= 24) return launch_col2im_stream<decltype(g), 8, 1>(g, col, B, C, H, W, m, n, im, st);
     return -1;
 }
-static int try_col2im_rows(StaticGeom<5, 5, 2, 2, 1, 1> g, const float* col, long B, int C, int H,
+static int try_col2im_stream(StaticGeom<5, 5, 2, 2, 1, 1> g, const float* col, long B, int C, int H,
                            int W, int m, int n, float* im, hipStream_t st) {
-    if (C >= 4 && W >= 24) return launch_col2im_rows<decltype(g), 4, 1, 28>(g, col, B, C, H, W, m, n, im, st);
+    if (C >= 4 && W >= 24) return launch_col2im_stream<decltype(g), 4, 1>(g, col, B, C, H, W, m, n, im, st);
     return -1;
 }
-static int try_col2im_rows(StaticGeom<11, 11, 0, 0, 4, 4> g, const float* col, long B, int C, int H,
+static int try_col2im_stream(StaticGeom<11, 11, 0, 0, 4, 4> g, const float* col, long B, int C, int H,
                            int W, int m, int n, float* im, hipStream_t st) {
-    if (C == 3 && W >= 64) return launch_col2im_rows<decltype(g), 3, 2, 32>(g, col, B, C, H, W, m, n, im, st);
+    if (C == 3 && W >= 64) return launch_col2im_stream<decltype(g), 3, 2>(g, col, B, C, H, W, m, n, im, st);
     return -1;
 }
 
@@ -519,7 +580,7 @@ static int launch_col2im(G g, const float* col, long B, int C, int H, int W, int
     const long total = B * C * H * W;
     if (total == 0) return CGT_AMD_OK;
     {
-        const int rc = try_col2im_rows(g, col, B, C, H, W, m, n, im, st);
+        const int rc = try_col2im_stream(g, col, B, C, H, W, m, n, im, st);
         if (rc >= 0) return rc;
     }
     long blocks = cdiv(total, 256);

@@ -35,7 +35,15 @@ __global__ __launch_bounds__(kPoolThreads) void max_pool_fwd_kernel(
     const int HW = H * W, PP = PH * PW;
     const float* src = bottom + p0 * HW;
     const int nin = np * HW;
-    for (int i = threadIdx.x; i < nin; i += kPoolThreads) tile[i] = src[i];
+    for (int base = threadIdx.x; base < nin; base += kPoolThreads * 8) {   // 8 loads in flight per thread
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (base + u * kPoolThreads < nin) v[u] = src[base + u * kPoolThreads];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (base + u * kPoolThreads < nin) tile[base + u * kPoolThreads] = v[u];
+    }
     __syncthreads();
 
     float* tdst = top + p0 * PP;
@@ -115,9 +123,21 @@ __global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_kernel(
     const int nout = np * PP;
     float* td = tile;
     int* mk = reinterpret_cast<int*>(tile + planes_per_wg * PP);
-    for (int i = threadIdx.x; i < nout; i += kPoolThreads) {
-        td[i] = top_diff[p0 * PP + i];
-        mk[i] = mask[p0 * PP + i];
+    for (int base = threadIdx.x; base < nout; base += kPoolThreads * 4) {  // 8 loads in flight per thread
+        float v[4];
+        int k[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (base + u * kPoolThreads < nout) {
+                v[u] = top_diff[p0 * PP + base + u * kPoolThreads];
+                k[u] = mask[p0 * PP + base + u * kPoolThreads];
+            }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (base + u * kPoolThreads < nout) {
+                td[base + u * kPoolThreads] = v[u];
+                mk[base + u * kPoolThreads] = k[u];
+            }
     }
     __syncthreads();
 

@@ -9,7 +9,8 @@ import numpy as np
 
 from . import capi
 
-_DTYPES = (np.dtype(np.float32), np.dtype(np.int32), np.dtype(np.int64))
+# float64 buffers exist only so tests can hand double data to checker kernels
+_DTYPES = (np.dtype(np.float32), np.dtype(np.int32), np.dtype(np.int64), np.dtype(np.float64))
 
 
 class _Buffer(object):

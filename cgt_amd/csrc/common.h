@@ -17,6 +17,7 @@ inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 
 constexpr int kWave = 64;    // CDNA wavefront width
 constexpr int kNumXCD = 8;   // MI355X: 8 accelerator dies, each with its own L2
+constexpr int kNumCU = 256;  // MI355X compute units
 
 inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 

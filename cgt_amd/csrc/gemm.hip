@@ -60,6 +60,11 @@ struct GemmArgs {
     int splits;        // > 1: partial products go to ws[split][M][N]
     int kchunk;        // K range per split, multiple of KT
     float* ws;
+    // tail split: workgroups [0, main_wgs) own whole tiles; the remaining
+    // tail_tiles tiles are cut into tail_splits K ranges each so that every CU
+    // gets an equal share of the last, partial round.  Pieces go to ws as
+    // [piece][BM][BN]; tail_reduce_kernel adds them up in order.
+    int main_wgs, tail_splits, tail_kchunk;
 };
 
 // One ROWS x KT operand tile.
@@ -189,7 +194,8 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
 
     // linear workgroup id -> (batch, split, tile)
     const int tiles = a.tiles_m * a.tiles_n;
-    int batch = 0, split = 0, lid;
+    int batch = 0, split = 0, lid, tail_piece = -1;
+    int kchunk = a.kchunk;
     if (a.splits > 1) {
         // groups of 8 splits: the tiles of one split share its K range of both
         // operands, so give them ids that are equal mod 8 (same XCD)
@@ -198,9 +204,15 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
         const int in_grp = min(kNumXCD, a.splits - grp * kNumXCD);
         split = grp * kNumXCD + r % in_grp;
         lid = r / in_grp;
+    } else if ((int)blockIdx.x < a.main_wgs) {
+        const int per_batch = a.main_wgs / a.batch;        // == tiles unless there is a tail (batch 1)
+        batch = blockIdx.x / per_batch;
+        lid = xcd_remap(blockIdx.x - batch * per_batch, per_batch);
     } else {
-        batch = blockIdx.x / tiles;
-        lid = xcd_remap(blockIdx.x - batch * tiles, tiles);
+        tail_piece = blockIdx.x - a.main_wgs;
+        lid = a.main_wgs + tail_piece / a.tail_splits;
+        split = tail_piece % a.tail_splits;
+        kchunk = a.tail_kchunk;
     }
     // tile order: groups of 8 tile rows, column-major inside a group, so tiles
     // that run together share A row panels and B column panels in L2
@@ -212,8 +224,8 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
     const int tm = first_m + in_group % gsz, tn = in_group / gsz;
     const int m0 = tm * BM, n0 = tn * BN;
 
-    const int kbeg = split * a.kchunk;
-    const int kend = min(a.K, kbeg + a.kchunk);
+    const int kbeg = split * kchunk;
+    const int kend = min(a.K, kbeg + kchunk);
     const float* A = a.A + batch * a.sA;
     const float* B = a.B + batch * a.sB;
 
@@ -245,6 +257,8 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
         }
         const float* as = As[cur];
         const float* bs = Bs[cur];
+        // a wavefront inside its MFMA burst goes ahead of wavefronts issuing loads
+        __builtin_amdgcn_s_setprio(3);
 #pragma unroll
         for (int kk = 0; kk < KT / 8; ++kk) {
             float af[TM][4], bf[TN][4];
@@ -261,6 +275,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][s], bf[j][s],
                                                                          acc[i][j], 0, 0, 0);
         }
+        __builtin_amdgcn_s_setprio(0);
         if (more) {
             ta.store(As[cur ^ 1]);
             tb.store(Bs[cur ^ 1]);
@@ -269,6 +284,18 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
     }
 
     // accumulator element e of a 32x32 block: row 8*(e/4) + 4*half + e%4, column l32
+    if (tail_piece >= 0) {
+        // tile-local [BM][BN] piece, no bounds: the reduction clips
+        float* out = a.ws + (long)tail_piece * (BM * BN);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    out[((wm * TM + i) * 32 + 8 * (e / 4) + 4 * half + (e % 4)) * BN + (wn * TN + j) * 32 + l32] = acc[i][j][e];
+        return;
+    }
     float* out;
     long ldo;
     if (a.splits > 1) {
@@ -290,6 +317,44 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
                 if (row < a.M) out[(long)row * ldo + col] = acc[i][j][e];
             }
         }
+}
+
+// Tail tiles: C tile = sum over its K pieces, in order.  blockIdx.y = tail tile,
+// one thread per 4 consecutive tile elements; all pieces are loaded before the
+// adds so the loads overlap.
+constexpr int kMaxTailSplits = 16;
+__global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restrict__ ws,
+                                                          float* __restrict__ C, GemmArgs a, int bm,
+                                                          int bn) {
+    const int lid = a.main_wgs + blockIdx.y;
+    // same tile order as sgemm_kernel
+    constexpr int GM = 8;
+    const int per_group = GM * a.tiles_n;
+    const int group = lid / per_group, in_group = lid - group * per_group;
+    const int first_m = group * GM;
+    const int gsz = min(a.tiles_m - first_m, GM);
+    const int tm = first_m + in_group % gsz, tn = in_group / gsz;
+    const int m0 = tm * bm, n0 = tn * bn;
+    const int i = (blockIdx.x * 256 + threadIdx.x) * 4;      // bn % 4 == 0: the 4 elements share a row
+    if (i >= bm * bn) return;
+    const float* src = ws + (long)blockIdx.y * a.tail_splits * (bm * bn) + i;
+    float4 v[kMaxTailSplits];
+#pragma unroll
+    for (int k = 0; k < kMaxTailSplits; ++k)
+        if (k < a.tail_splits) v[k] = *reinterpret_cast<const float4*>(src + (long)k * (bm * bn));
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int k = 0; k < kMaxTailSplits; ++k)
+        if (k < a.tail_splits) {
+            s.x += v[k].x; s.y += v[k].y; s.z += v[k].z; s.w += v[k].w;
+        }
+    const int r = i / bn, c = i - r * bn;
+    if (m0 + r >= a.M) return;
+    float* dst = C + (long)(m0 + r) * a.ldc + n0 + c;
+    const float o[4] = {s.x, s.y, s.z, s.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        if (n0 + c + j < a.N) dst[j] = o[j];
 }
 
 // C[r][c] = sum_s ws[s][r][c], s ascending.
@@ -412,7 +477,37 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
             }
         }
     }
-    const long wgs = tiles * P * a.splits;
+    // tail split (single product, no split-K): tiles beyond the last full
+    // round of the chip are cut along K so the partial round is balanced
+    a.main_wgs = (int)(tiles * P);
+    a.tail_splits = 1;
+    a.tail_kchunk = a.kchunk;
+    long tail_tiles = 0;
+    const long nk = cdiv(K, KT);
+    if (P == 1 && a.splits == 1 && tiles >= kNumCU && tiles < 24L * kNumCU && tiles % kNumCU != 0 && nk >= 16) {
+        const long r = tiles % kNumCU;
+        long best_s = 1;
+        double best_t = (double)cdiv(r, kNumCU);             // tail time in units of one whole tile
+        for (long sp = 2; sp <= std::min((long)kMaxTailSplits, nk / 4); ++sp) {
+            const double t = (double)cdiv(r * sp, kNumCU) / sp + 0.02 * sp;   // small charge per extra piece
+            if (t < best_t) {
+                best_t = t;
+                best_s = sp;
+            }
+        }
+        if (best_s > 1) {
+            tail_tiles = r;
+            a.main_wgs = (int)(tiles - r);
+            a.tail_kchunk = (int)(cdiv(cdiv(K, best_s), KT) * KT);
+            a.tail_splits = (int)cdiv(K, a.tail_kchunk);
+            a.ws = get_workspace(stream, (size_t)tail_tiles * a.tail_splits * kShapes[shape].bm * kShapes[shape].bn * sizeof(float));
+            if (!a.ws) {
+                set_error("sgemm: cannot allocate tail workspace");
+                return CGT_AMD_ERR_NOMEM;
+            }
+        }
+    }
+    const long wgs = a.splits > 1 ? tiles * a.splits : a.main_wgs + tail_tiles * a.tail_splits;
     CGT_ARG_CHECK(wgs < (1L << 31), "sgemm: too many workgroups");
     hipStream_t st = as_stream(stream);
     dim3 grid((unsigned)wgs);
@@ -424,6 +519,10 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
         long blocks = std::min(cdiv(MN, 256L), 1L << 16);
         splitk_reduce_kernel<<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a.ws, C, MN, (int)N, ldc, a.splits);
         CGT_LAUNCH_CHECK("splitk_reduce_kernel");
+    } else if (tail_tiles > 0) {
+        tail_reduce_kernel<<<dim3((unsigned)cdiv(kShapes[shape].bm * kShapes[shape].bn, 1024), (unsigned)tail_tiles), dim3(256), 0, st>>>(
+            a.ws, C, a, kShapes[shape].bm, kShapes[shape].bn);
+        CGT_LAUNCH_CHECK("tail_reduce_kernel");
     }
     return CGT_AMD_OK;
 }

@@ -235,6 +235,8 @@ GEMM_SHAPES = [
     (2048, 32, 9),                                             # MNIST conv skew
     (200, 64, 800), (96, 363, 3000),                           # split-K range
     (128, 1152, 4100),                                         # VGG weight gradient in miniature
+    (38400, 128, 512),                                         # 300 tiles: whole round + K-split tail
+    (33000, 96, 363),                                          # 258 tiles of 128x96, unaligned K, clipped tail tile
 ]
 
 

@@ -240,47 +240,107 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
     const int nk = (kend - kbeg + KT - 1) / KT;
     TileA ta;
     TileB tb;
-    if (nk > 0) {
-        ta.load(A, a.lda, m0, a.M, kbeg, kend);
-        tb.load(B, a.ldb, n0, a.N, kbeg, kend);
-        ta.store(As[0]);
-        tb.store(Bs[0]);
-    }
-    __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        const int cur = kt & 1;
-        const bool more = kt + 1 < nk;
-        if (more) {
-            const int k0 = kbeg + (kt + 1) * KT;
-            ta.load(A, a.lda, m0, a.M, k0, kend);
-            tb.load(B, a.ldb, n0, a.N, k0, kend);
+
+    // Software pipeline, per wavefront (K slice t lives in LDS buffer t&1):
+    //   top of iteration t   : registers hold slice t+1 (loaded one iteration
+    //                          ago) -> parked in the other LDS buffer; global
+    //                          loads of slice t+2 issued; fragment set 1
+    //                          (k group 1 of slice t) requested from LDS
+    //   first half           : MFMAs on fragment set 0 (k group 0 of slice t,
+    //                          requested during the previous iteration)
+    //   barrier (LDS only)   : slice t+1 is visible; it sits in the middle of
+    //                          the MFMA stream and does not wait for the global
+    //                          loads in flight
+    //   second half          : fragment set 0 of slice t+1 requested, MFMAs on
+    //                          fragment set 1 (already in registers)
+    // so LDS and HBM latencies sit under this wavefront's own MFMAs.  Reads of
+    // a buffer are all issued before the barrier of the iteration that precedes
+    // its next overwrite, and LDS serves requests in order, so two buffers do.
+    float af[2][TM][4], bf[2][TN][4];
+    auto read_frags = [&](int set, const float* as, const float* bs, int kk) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) TileA::frag(as, (wm * TM + i) * 32 + l32, kk, half, af[set][i]);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) TileB::frag(bs, (wn * TN + j) * 32 + l32, kk, half, bf[set][j]);
+    };
+    auto mfma_steps = [&](int set, int s0, int s1) {
+#pragma unroll
+        for (int s = s0; s < s1; ++s)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[set][i][s], bf[set][j][s],
+                                                                     acc[i][j], 0, 0, 0);
+    };
+    // wait for this wavefront's LDS traffic only, then workgroup barrier
+    auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+    // The pipelined schedule pays off when both operands are k-contiguous
+    // (16-byte fragment reads); the other layouts measure faster with the
+    // plain double-buffered loop (one full barrier per slice).
+    constexpr bool kPipelined = AKC && BKC;
+    if constexpr (kPipelined) {
+        if (nk > 0) {
+            ta.load(A, a.lda, m0, a.M, kbeg, kend);
+            tb.load(B, a.ldb, n0, a.N, kbeg, kend);
+            ta.store(As[0]);
+            tb.store(Bs[0]);
+            if (nk > 1) {
+                ta.load(A, a.lda, m0, a.M, kbeg + KT, kend);
+                tb.load(B, a.ldb, n0, a.N, kbeg + KT, kend);
+            }
+            lds_barrier();
+            read_frags(0, As[0], Bs[0], 0);
         }
-        const float* as = As[cur];
-        const float* bs = Bs[cur];
-        // a wavefront inside its MFMA burst goes ahead of wavefronts issuing loads
-        __builtin_amdgcn_s_setprio(3);
-#pragma unroll
-        for (int kk = 0; kk < KT / 8; ++kk) {
-            float af[TM][4], bf[TN][4];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) TileA::frag(as, (wm * TM + i) * 32 + l32, kk, half, af[i]);
-#pragma unroll
-            for (int j = 0; j < TN; ++j) TileB::frag(bs, (wn * TN + j) * 32 + l32, kk, half, bf[j]);
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][s], bf[j][s],
-                                                                         acc[i][j], 0, 0, 0);
+        for (int kt = 0; kt < nk; ++kt) {
+            const int cur = kt & 1;
+            if (kt + 1 < nk) {
+                ta.store(As[cur ^ 1]);       // slice kt+1 (waits for its global loads, issued an iteration ago)
+                tb.store(Bs[cur ^ 1]);
+            }
+            if (kt + 2 < nk) {
+                const int k0 = kbeg + (kt + 2) * KT;
+                ta.load(A, a.lda, m0, a.M, k0, kend);
+                tb.load(B, a.ldb, n0, a.N, k0, kend);
+            }
+            read_frags(1, As[cur], Bs[cur], 1);
+            __builtin_amdgcn_s_setprio(3);   // inside the MFMA stream: ahead of wavefronts issuing loads
+            mfma_steps(0, 0, 4);
+            lds_barrier();
+            if (kt + 1 < nk) read_frags(0, As[cur ^ 1], Bs[cur ^ 1], 0);
+            mfma_steps(1, 0, 4);
+            __builtin_amdgcn_s_setprio(0);
         }
-        __builtin_amdgcn_s_setprio(0);
-        if (more) {
-            ta.store(As[cur ^ 1]);
-            tb.store(Bs[cur ^ 1]);
+    } else {
+        if (nk > 0) {
+            ta.load(A, a.lda, m0, a.M, kbeg, kend);
+            tb.load(B, a.ldb, n0, a.N, kbeg, kend);
+            ta.store(As[0]);
+            tb.store(Bs[0]);
         }
         __syncthreads();
+        for (int kt = 0; kt < nk; ++kt) {
+            const int cur = kt & 1;
+            const bool more = kt + 1 < nk;
+            if (more) {
+                const int k0 = kbeg + (kt + 1) * KT;
+                ta.load(A, a.lda, m0, a.M, k0, kend);
+                tb.load(B, a.ldb, n0, a.N, k0, kend);
+            }
+            __builtin_amdgcn_s_setprio(3);
+#pragma unroll
+            for (int kk = 0; kk < KT / 8; ++kk) {
+                read_frags(0, As[cur], Bs[cur], kk);
+                mfma_steps(0, 0, 4);
+            }
+            __builtin_amdgcn_s_setprio(0);
+            if (more) {
+                ta.store(As[cur ^ 1]);
+                tb.store(Bs[cur ^ 1]);
+            }
+            __syncthreads();
+        }
     }
 
     // accumulator element e of a 32x32 block: row 8*(e/4) + 4*half + e%4, column l32

@@ -107,7 +107,7 @@ class LayerOnGpu(object):
         s = stream
         st.append(Stage("im2col", "im2col_pipe_kernel", lambda: K.im2col(self.x, (r, c), pad, stride, out=self.col, stream=s),
                         4 * (nelem(self.x) + nelem(self.col)), "hbm"))
-        st.append(Stage("gemm_fwd_NT", "sgemm_kernel<true, true, true, 2, 2, 2, 2>", lambda: K.mul22(self.col2, self.f_LZ, False, True, out=self.y_mnL, stream=s),
+        st.append(Stage("gemm_fwd_NT", "sgemm_kernel", lambda: K.mul22(self.col2, self.f_LZ, False, True, out=self.y_mnL, stream=s),
                         2 * Bmn * L * Z, "mfma"))
         st.append(Stage("transpose_0312", "batched_transpose_kernel",
                         lambda: K.transpose4(self.y_mnL.reshape(B, m, n, L), (0, 3, 1, 2), out=self.y, stream=s),
@@ -148,12 +148,12 @@ class LayerOnGpu(object):
         self.gf = empty((L, Z))
         st.append(Stage("transpose_0231", "batched_transpose_kernel", lambda: K.transpose4(self.gy, (0, 2, 3, 1), out=self.gc, stream=s),
                         2 * 4 * nelem(self.y), "hbm"))
-        st.append(Stage("gemm_dgrad_NN", "sgemm_kernel<true, false, true, 2, 2, 2, 2>", lambda: K.mul22(self.gc2, self.f_LZ, False, False, out=self.gcol, stream=s),
+        st.append(Stage("gemm_dgrad_NN", "sgemm_kernel", lambda: K.mul22(self.gc2, self.f_LZ, False, False, out=self.gcol, stream=s),
                         2 * Bmn * L * Z, "mfma"))
         st.append(Stage("col2im", "col2im_stream_kernel",
                         lambda: K.col2im(self.gcol.reshape(B, m, n, Z), self.x.shape, (r, c), pad, stride, out=self.gx, stream=s),
                         4 * (nelem(self.x) + nelem(self.col)), "hbm"))
-        st.append(Stage("gemm_wgrad_TN", "sgemm_kernel<false, false, true, 2, 2, 2, 2>", lambda: K.mul22(self.gc2, self.col2, True, False, out=self.gf, stream=s),
+        st.append(Stage("gemm_wgrad_TN", "sgemm_kernel", lambda: K.mul22(self.gc2, self.col2, True, False, out=self.gf, stream=s),
                         2 * Bmn * L * Z, "mfma"))
         self.stages = st
         self.conv_flops = 6 * Bmn * L * Z
@@ -191,10 +191,10 @@ class GemmOnGpu(object):
         s = stream
         st = []
         for tA, tB, name in [(False, False, "NN"), (False, True, "NT"), (True, False, "TN"), (True, True, "TT")]:
-            st.append(Stage("mul22_%s_%d" % (name, n), "sgemm_kernel<%s, %s, true, 2, 2, 2, 2>" % (str(not tA).lower(), str(tB).lower()),
+            st.append(Stage("mul22_%s_%d" % (name, n), "sgemm_kernel",
                             (lambda tA=tA, tB=tB: K.mul22(self.A, self.B, tA, tB, out=self.C, stream=s)),
                             2 * n ** 3, "mfma"))
-        st.append(Stage("batched_mul22_%dx%d" % (P, nb), "sgemm_kernel<true, false, true, 2, 2, 2, 2>",
+        st.append(Stage("batched_mul22_%dx%d" % (P, nb), "sgemm_kernel",
                         lambda: K.batched_mul22(self.bA, self.bB, out=self.bC, stream=s), 2 * P * nb ** 3, "mfma"))
         self.stages = st
         self.conv_flops = sum(x.work for x in st)

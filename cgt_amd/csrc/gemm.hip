@@ -179,12 +179,12 @@ __device__ __forceinline__ int xcd_remap(int id, int n) {
 }
 
 // WGM x WGN wavefronts, each TM x TN blocks of 32x32.
-template <bool AKC, bool BKC, bool VEC, int WGM, int WGN, int TM, int TN>
+template <bool AKC, bool BKC, bool VECA, bool VECB, int WGM, int WGN, int TM, int TN>
 __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
     static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
-    typedef OperandTile<AKC, BM, VEC> TileA;
-    typedef OperandTile<BKC, BN, VEC> TileB;
+    typedef OperandTile<AKC, BM, VECA> TileA;
+    typedef OperandTile<BKC, BN, VECB> TileB;
     __shared__ __attribute__((aligned(16))) float As[2][TileA::kFloats];
     __shared__ __attribute__((aligned(16))) float Bs[2][TileB::kFloats];
 
@@ -464,24 +464,32 @@ struct TileShape {
 // Tile shapes on offer; the 128x128 default comes first and wins ties.
 static const TileShape kShapes[] = {{128, 128}, {128, 96}, {128, 64}, {128, 32}, {96, 128}};
 
-template <bool AKC, bool BKC, bool VEC>
+template <bool AKC, bool BKC, bool VECA, bool VECB>
 static void launch_shape(int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
     dim3 block(kGemmThreads);
     switch (shape) {
-        case 0: sgemm_kernel<AKC, BKC, VEC, 2, 2, 2, 2><<<grid, block, 0, st>>>(a); break;
-        case 1: sgemm_kernel<AKC, BKC, VEC, 4, 1, 1, 3><<<grid, block, 0, st>>>(a); break;
-        case 2: sgemm_kernel<AKC, BKC, VEC, 4, 1, 1, 2><<<grid, block, 0, st>>>(a); break;
-        case 3: sgemm_kernel<AKC, BKC, VEC, 4, 1, 1, 1><<<grid, block, 0, st>>>(a); break;
-        default: sgemm_kernel<AKC, BKC, VEC, 1, 4, 3, 1><<<grid, block, 0, st>>>(a); break;
+        case 0: sgemm_kernel<AKC, BKC, VECA, VECB, 2, 2, 2, 2><<<grid, block, 0, st>>>(a); break;
+        case 1: sgemm_kernel<AKC, BKC, VECA, VECB, 4, 1, 1, 3><<<grid, block, 0, st>>>(a); break;
+        case 2: sgemm_kernel<AKC, BKC, VECA, VECB, 4, 1, 1, 2><<<grid, block, 0, st>>>(a); break;
+        case 3: sgemm_kernel<AKC, BKC, VECA, VECB, 4, 1, 1, 1><<<grid, block, 0, st>>>(a); break;
+        default: sgemm_kernel<AKC, BKC, VECA, VECB, 1, 4, 3, 1><<<grid, block, 0, st>>>(a); break;
     }
 }
 
-template <bool VEC>
-static void launch_trans(int tA, int tB, int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
-    if (!tA && !tB) launch_shape<true, false, VEC>(shape, grid, st, a);
-    else if (!tA && tB) launch_shape<true, true, VEC>(shape, grid, st, a);
-    else if (tA && !tB) launch_shape<false, false, VEC>(shape, grid, st, a);
-    else launch_shape<false, true, VEC>(shape, grid, st, a);
+template <bool AKC, bool BKC>
+static void launch_vec(bool vecA, bool vecB, int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
+    if (vecA && vecB) launch_shape<AKC, BKC, true, true>(shape, grid, st, a);
+    else if (vecA) launch_shape<AKC, BKC, true, false>(shape, grid, st, a);
+    else if (vecB) launch_shape<AKC, BKC, false, true>(shape, grid, st, a);
+    else launch_shape<AKC, BKC, false, false>(shape, grid, st, a);
+}
+
+static void launch_trans(int tA, int tB, bool vecA, bool vecB, int shape, dim3 grid, hipStream_t st,
+                         const GemmArgs& a) {
+    if (!tA && !tB) launch_vec<true, false>(vecA, vecB, shape, grid, st, a);
+    else if (!tA && tB) launch_vec<true, true>(vecA, vecB, shape, grid, st, a);
+    else if (tA && !tB) launch_vec<false, false>(vecA, vecB, shape, grid, st, a);
+    else launch_vec<false, true>(vecA, vecB, shape, grid, st, a);
 }
 
 static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const float* A, long lda,
@@ -516,7 +524,8 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     a.tiles_n = (int)cdiv(N, kShapes[shape].bn);
     a.batch = (int)P;
     const long tiles = (long)a.tiles_m * a.tiles_n;
-    const bool vec = lda % 4 == 0 && sA % 4 == 0 && aligned16(A) && ldb % 4 == 0 && sB % 4 == 0 && aligned16(B);
+    const bool vecA = lda % 4 == 0 && sA % 4 == 0 && aligned16(A);
+    const bool vecB = ldb % 4 == 0 && sB % 4 == 0 && aligned16(B);
     a.splits = 1;
     a.kchunk = (int)(cdiv(std::max(K, 1L), KT) * KT);
     a.ws = nullptr;
@@ -571,8 +580,7 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     CGT_ARG_CHECK(wgs < (1L << 31), "sgemm: too many workgroups");
     hipStream_t st = as_stream(stream);
     dim3 grid((unsigned)wgs);
-    if (vec) launch_trans<true>(tA, tB, shape, grid, st, a);
-    else launch_trans<false>(tA, tB, shape, grid, st, a);
+    launch_trans(tA, tB, vecA, vecB, shape, grid, st, a);
     CGT_LAUNCH_CHECK("sgemm_kernel");
     if (a.splits > 1) {
         const long MN = M * N;

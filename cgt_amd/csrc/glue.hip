@@ -32,6 +32,87 @@ __global__ __launch_bounds__(256) void batched_transpose_kernel(
     }
 }
 
+
+// Thin case: one of the two transposed extents (L) is small, as in the conv
+// glue where L is the filter count.  A workgroup takes kThinRows positions of
+// the long axis and ALL of L, so the side whose rows are L long is one
+// contiguous block of kThinRows*L floats (16-byte accesses when L % 4 == 0),
+// and the other side is L runs of kThinRows floats.
+//   L_INNER_IN:  in [B, R, L] -> out [B, L, R]
+//   otherwise:   in [B, L, R] -> out [B, R, L]
+constexpr int kThinRows = 64;
+constexpr int kThinMaxL = 128;
+
+__device__ __forceinline__ int div_small(int n, int d, float rd) {
+    // exact for 0 <= n < 2^21: the float quotient is off by at most one
+    int q = (int)((float)n * rd);
+    const int r = n - q * d;
+    q += (r >= d) - (r < 0);
+    return q;
+}
+
+template <bool L_INNER_IN, bool VEC>
+__global__ __launch_bounds__(256) void thin_transpose_kernel(const float* __restrict__ in,
+                                                             float* __restrict__ out, int R, int L,
+                                                             int tiles_r) {
+    extern __shared__ float tile[];          // [kThinRows][LD]
+    const int LD = L | 1;
+    const int tr = blockIdx.x % tiles_r;
+    const long b = blockIdx.x / tiles_r;
+    const int r0 = tr * kThinRows;
+    const int rows = min(kThinRows, R - r0);
+    const float rL = 1.0f / (float)L;
+    const float* src = in + b * (long)R * L;
+    float* dst = out + b * (long)R * L;
+    // the side with rows of length L: block of rows*L contiguous floats
+    const float* blk_in = src + (long)r0 * L;
+    float* blk_out = dst + (long)r0 * L;
+    const int n = rows * L;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (L_INNER_IN) {
+        if (VEC) {
+            for (int i = threadIdx.x * 4; i < n; i += 1024) {
+                const float4 v = *reinterpret_cast<const float4*>(blk_in + i);
+                const int r = div_small(i, L, rL), c = i - r * L;
+                float* t = tile + r * LD + c;
+                t[0] = v.x; t[1] = v.y; t[2] = v.z; t[3] = v.w;
+            }
+        } else {
+            for (int i = threadIdx.x; i < n; i += 256) {
+                const int r = div_small(i, L, rL), c = i - r * L;
+                tile[r * LD + c] = blk_in[i];
+            }
+        }
+        __syncthreads();
+        if (lane < rows)
+            for (int c = wave; c < L; c += 4) dst[(long)c * R + r0 + lane] = tile[lane * LD + c];
+    } else {
+        // eight runs in flight per wavefront before the first LDS store
+        if (lane < rows)
+            for (int c = wave; c < L; c += 32) {
+                float v[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) v[k] = c + 4 * k < L ? src[(long)(c + 4 * k) * R + r0 + lane] : 0.f;
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    if (c + 4 * k < L) tile[lane * LD + c + 4 * k] = v[k];
+            }
+        __syncthreads();
+        if (VEC) {
+            for (int i = threadIdx.x * 4; i < n; i += 1024) {
+                const int r = div_small(i, L, rL), c = i - r * L;
+                const float* t = tile + r * LD + c;
+                *reinterpret_cast<float4*>(blk_out + i) = make_float4(t[0], t[1], t[2], t[3]);
+            }
+        } else {
+            for (int i = threadIdx.x; i < n; i += 256) {
+                const int r = div_small(i, L, rL), c = i - r * L;
+                blk_out[i] = tile[r * LD + c];
+            }
+        }
+    }
+}
+
 struct Perm4 {
     long oshape[4];
     long istride[4];  // input stride of the axis feeding output axis d
@@ -53,11 +134,36 @@ __global__ __launch_bounds__(256) void transpose4_generic_kernel(const float* __
     }
 }
 
+static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
+// in [B, R, Cn] -> out [B, Cn, R]
 static int launch_batched_transpose(const float* in, float* out, long B, long R, long Cn,
                                     hipStream_t st) {
+    CGT_ARG_CHECK(R < (1L << 31) && Cn < (1L << 31), "transpose: too large");
+    // thin paths: the short extent is not a multiple of the square tile (which
+    // would idle lanes) or the long one is odd (unaligned rows either way)
+    const bool thin_in = Cn <= kThinMaxL && R >= 4 * kThinRows && (Cn % kTile != 0 || R % 4 != 0);
+    const bool thin_out = R <= kThinMaxL && Cn >= 4 * kThinRows && (R % kTile != 0 || Cn % 4 != 0);
+    if (thin_in || thin_out) {
+        const long L = thin_in ? Cn : R, longdim = thin_in ? R : Cn;
+        const long tiles = cdiv(longdim, kThinRows);
+        CGT_ARG_CHECK(B * tiles < (1L << 31), "transpose: too large");
+        const bool vec = L % 4 == 0 && aligned16(in) && aligned16(out);
+        const size_t lds = (size_t)kThinRows * (L | 1) * sizeof(float);
+        dim3 grid((unsigned)(B * tiles)), block(256);
+        if (thin_in) {
+            if (vec) thin_transpose_kernel<true, true><<<grid, block, lds, st>>>(in, out, (int)longdim, (int)L, (int)tiles);
+            else thin_transpose_kernel<true, false><<<grid, block, lds, st>>>(in, out, (int)longdim, (int)L, (int)tiles);
+        } else {
+            if (vec) thin_transpose_kernel<false, true><<<grid, block, lds, st>>>(in, out, (int)longdim, (int)L, (int)tiles);
+            else thin_transpose_kernel<false, false><<<grid, block, lds, st>>>(in, out, (int)longdim, (int)L, (int)tiles);
+        }
+        CGT_LAUNCH_CHECK("thin_transpose_kernel");
+        return CGT_AMD_OK;
+    }
     const long tr = cdiv(R, kTile), tc = cdiv(Cn, kTile);
     const long blocks = B * tr * tc;
-    CGT_ARG_CHECK(blocks < (1L << 31) && R < (1L << 31) && Cn < (1L << 31), "transpose: too large");
+    CGT_ARG_CHECK(blocks < (1L << 31), "transpose: too large");
     batched_transpose_kernel<<<dim3((unsigned)blocks), dim3(256), 0, st>>>(in, out, (int)R, (int)Cn,
                                                                            (int)tr, (int)tc);
     CGT_LAUNCH_CHECK("batched_transpose_kernel");

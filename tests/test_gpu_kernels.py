@@ -295,6 +295,19 @@ def test_transpose4(K, axes):
     assert bits_equal(K.transpose4(gpu(x), axes).get(), np.ascontiguousarray(x.transpose(axes)))
 
 
+# conv-glue shapes where the filter count is the short extent: thin-tile path
+# (vector and scalar variants, ragged last tile, long extent odd)
+@pytest.mark.parametrize("shape", [(2, 55, 55, 96), (3, 19, 17, 75), (2, 16, 16, 128), (1, 23, 13, 4),
+                                   (2, 31, 9, 1), (2, 20, 20, 100)])
+@pytest.mark.parametrize("axes", [(0, 3, 1, 2), (0, 2, 3, 1)])
+def test_transpose4_conv_glue(K, shape, axes):
+    rs = np.random.RandomState(8)
+    if axes == (0, 2, 3, 1):
+        shape = (shape[0], shape[3], shape[1], shape[2])      # [B, L, m, n]
+    x = rs.randn(*shape).astype(np.float32)
+    assert bits_equal(K.transpose4(gpu(x), axes).get(), np.ascontiguousarray(x.transpose(axes)))
+
+
 def test_conv2d_reference_known_answer(K):
     # cgt/tests/test_conv.py:14-33 (single precision tolerance atol 1e-3)
     import scipy.signal

@@ -17,44 +17,78 @@ namespace cgt_amd {
 
 constexpr int kLrnThreads = 256;
 
+// One-dimensional grid over (image, channel run, pixel block), pixel blocks
+// fastest.  Workgroups go to the 8 XCDs round-robin by id; the remap gives each
+// XCD a contiguous range, so the two workgroups that share a cache line at a
+// pixel-block boundary (H*W need not be a multiple of anything) meet in one L2.
+struct LrnBlock {
+    int px, run, n;
+};
+__device__ __forceinline__ LrnBlock lrn_block(int HW, int C, int crun) {
+    const int total = gridDim.x;
+    const int q = total / kNumXCD, r = total % kNumXCD;
+    const int xcd = blockIdx.x % kNumXCD, local = blockIdx.x / kNumXCD;
+    int id = xcd * q + min(xcd, r) + local;
+    const int pb = (HW + kLrnThreads - 1) / kLrnThreads, runs = (C + crun - 1) / crun;
+    LrnBlock b;
+    b.px = id % pb;
+    id /= pb;
+    b.run = id % runs;
+    b.n = id / runs;
+    return b;
+}
+
 __device__ __forceinline__ float pow_neg_beta(float s, float nbeta) {
     // s >= k > 0.  exp2(nbeta*log2(s)) on the hardware transcendental units:
     // relative error ~1e-6 for the scale range LRN produces.
     return __builtin_amdgcn_exp2f(nbeta * __builtin_amdgcn_logf(s));
 }
 
-// SIZE > 0: window length known at compile time (ring in registers).
+// SIZE > 0: window length known at compile time.  Channels are walked in
+// chunks of U: the U new loads of a chunk are all issued before the first use,
+// so every lane keeps U runs in flight (one pixel per lane gives only 4-byte
+// loads -- H*W is odd in the AlexNet layer -- so depth has to come from here).
+constexpr int kLrnChunk = 8;
+
 template <int SIZE>
 __global__ __launch_bounds__(kLrnThreads) void lrn_fwd_kernel(
     const float* __restrict__ x, float* __restrict__ top, float* __restrict__ scale, int C,
     int HW, int crun, float aos, float nbeta, float kconst) {
-    constexpr int PRE = (SIZE - 1) / 2, POST = SIZE - PRE - 1;
-    const int p = blockIdx.x * kLrnThreads + threadIdx.x;
+    constexpr int PRE = (SIZE - 1) / 2, POST = SIZE - PRE - 1, U = kLrnChunk;
+    const LrnBlock blk = lrn_block(HW, C, crun);
+    const int p = blk.px * kLrnThreads + threadIdx.x;
     if (p >= HW) return;
-    const long n = blockIdx.z;
-    const int cs = blockIdx.y * crun, ce = min(C, cs + crun);
+    const long n = blk.n;
+    const int cs = blk.run * crun, ce = min(C, cs + crun);
     const float* xp = x + n * C * (long)HW + p;
     float* tp = top + n * C * (long)HW + p;
     float* sp = scale + n * C * (long)HW + p;
 
-    float ring[SIZE];  // ring[j] = x[c - PRE + j]
+    float win[U + SIZE - 1];  // win[j] = x[c0 - PRE + j]
 #pragma unroll
-    for (int j = 1; j < SIZE; ++j) {
-        const int c = cs - PRE + j - 1;
-        ring[j] = (c >= 0 && c < C) ? xp[(long)c * HW] : 0.0f;
+    for (int j = 0; j < SIZE - 1; ++j) {
+        const int c = cs - PRE + j;
+        win[j] = (c >= 0 && c < C) ? xp[(long)c * HW] : 0.0f;
     }
-#pragma unroll 4
-    for (int c = cs; c < ce; ++c) {
+    for (int c0 = cs; c0 < ce; c0 += U) {
 #pragma unroll
-        for (int j = 0; j < SIZE - 1; ++j) ring[j] = ring[j + 1];
-        const int ch = c + POST;
-        ring[SIZE - 1] = (ch < C) ? xp[(long)ch * HW] : 0.0f;
-        float acc = 0.0f;
+        for (int u = 0; u < U; ++u) {
+            const int ch = c0 + POST + u;
+            win[SIZE - 1 + u] = (ch < C) ? xp[(long)ch * HW] : 0.0f;
+        }
 #pragma unroll
-        for (int j = 0; j < SIZE; ++j) acc += ring[j] * ring[j];
-        const float s = kconst + acc * aos;
-        sp[(long)c * HW] = s;
-        tp[(long)c * HW] = ring[PRE] * pow_neg_beta(s, nbeta);
+        for (int u = 0; u < U; ++u) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int j = 0; j < SIZE; ++j) acc += win[u + j] * win[u + j];
+            const float s = kconst + acc * aos;
+            if (c0 + u < ce) {
+                sp[(long)(c0 + u) * HW] = s;
+                tp[(long)(c0 + u) * HW] = win[u + PRE] * pow_neg_beta(s, nbeta);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < SIZE - 1; ++j) win[j] = win[U + j];
     }
 }
 
@@ -63,10 +97,11 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_fwd_generic_kernel(
     const float* __restrict__ x, float* __restrict__ top, float* __restrict__ scale, int C,
     int HW, int crun, int size, float aos, float nbeta, float kconst) {
     const int pre = (size - 1) / 2, post = size - pre - 1;
-    const int p = blockIdx.x * kLrnThreads + threadIdx.x;
+    const LrnBlock blk = lrn_block(HW, C, crun);
+    const int p = blk.px * kLrnThreads + threadIdx.x;
     if (p >= HW) return;
-    const long n = blockIdx.z;
-    const int cs = blockIdx.y * crun, ce = min(C, cs + crun);
+    const long n = blk.n;
+    const int cs = blk.run * crun, ce = min(C, cs + crun);
     const long base = n * C * (long)HW + p;
     for (int c = cs; c < ce; ++c) {
         float acc = 0.0f;
@@ -87,11 +122,12 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_bwd_kernel(
     const float* __restrict__ top_diff, float* __restrict__ bottom_diff, int C, int HW, int crun,
     float nbeta, float ratio) {
     // transposed window: [c - PRE, c + POST]
-    constexpr int PRE = SIZE - (SIZE + 1) / 2, POST = SIZE - PRE - 1;
-    const int p = blockIdx.x * kLrnThreads + threadIdx.x;
+    constexpr int PRE = SIZE - (SIZE + 1) / 2, POST = SIZE - PRE - 1, U = kLrnChunk;
+    const LrnBlock blk = lrn_block(HW, C, crun);
+    const int p = blk.px * kLrnThreads + threadIdx.x;
     if (p >= HW) return;
-    const long n = blockIdx.z;
-    const int cs = blockIdx.y * crun, ce = min(C, cs + crun);
+    const long n = blk.n;
+    const int cs = blk.run * crun, ce = min(C, cs + crun);
     const long base = n * C * (long)HW + p;
     const float* xp = x + base;
     const float* tp = top + base;
@@ -99,47 +135,57 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_bwd_kernel(
     const float* dp = top_diff + base;
     float* bp = bottom_diff + base;
 
-    float tr[SIZE];       // tr[j] = (td*top/scale)[c - PRE + j]
-    float dr[POST + 1];   // dr[j] = td[c + j]
-    float sr[POST + 1];   // sr[j] = scale[c + j]
+    float tr[U + SIZE - 1];   // tr[j] = (td*top/scale)[c0 - PRE + j]
+    float dr[U + POST];       // dr[j] = td[c0 + j]
+    float sr[U + POST];       // sr[j] = scale[c0 + j]
 #pragma unroll
-    for (int j = 1; j < SIZE; ++j) {
-        const int c = cs - PRE + j - 1;
-        float d = 0.0f, s = 1.0f, t = 0.0f;
+    for (int j = 0; j < SIZE - 1; ++j) {
+        const int c = cs - PRE + j;
+        float d = 0.0f, sc = 1.0f, t = 0.0f;
         if (c >= 0 && c < C) {
             d = dp[(long)c * HW];
-            s = sp[(long)c * HW];
+            sc = sp[(long)c * HW];
             t = tp[(long)c * HW];
         }
-        tr[j] = d * t / s;
-        if (j - 1 >= PRE) {       // channel >= cs: also feeds the centre rings
+        tr[j] = d * t / sc;
+        if (j >= PRE) {           // channel >= cs: also a centre later on
             dr[j - PRE] = d;
-            sr[j - PRE] = s;
+            sr[j - PRE] = sc;
         }
     }
-#pragma unroll 4
-    for (int c = cs; c < ce; ++c) {
+    for (int c0 = cs; c0 < ce; c0 += U) {
+        float xc[U], tn[U];
 #pragma unroll
-        for (int j = 0; j < SIZE - 1; ++j) tr[j] = tr[j + 1];
+        for (int u = 0; u < U; ++u) {
+            const int ch = c0 + POST + u;
+            float d = 0.0f, sc = 1.0f, t = 0.0f;
+            if (ch < C) {
+                d = dp[(long)ch * HW];
+                sc = sp[(long)ch * HW];
+                t = tp[(long)ch * HW];
+            }
+            dr[POST + u] = d;
+            sr[POST + u] = sc;
+            tn[u] = t;
+            xc[u] = (c0 + u < ce) ? xp[(long)(c0 + u) * HW] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) tr[SIZE - 1 + u] = dr[POST + u] * tn[u] / sr[POST + u];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int j = 0; j < SIZE; ++j) acc += tr[u + j];
+            if (c0 + u < ce)
+                bp[(long)(c0 + u) * HW] = dr[u] * pow_neg_beta(sr[u], nbeta) - ratio * xc[u] * acc;
+        }
+#pragma unroll
+        for (int j = 0; j < SIZE - 1; ++j) tr[j] = tr[U + j];
 #pragma unroll
         for (int j = 0; j < POST; ++j) {
-            dr[j] = dr[j + 1];
-            sr[j] = sr[j + 1];
+            dr[j] = dr[U + j];
+            sr[j] = sr[U + j];
         }
-        const int ch = c + POST;
-        float d = 0.0f, s = 1.0f, t = 0.0f;
-        if (ch < C) {
-            d = dp[(long)ch * HW];
-            s = sp[(long)ch * HW];
-            t = tp[(long)ch * HW];
-        }
-        tr[SIZE - 1] = d * t / s;
-        dr[POST] = d;
-        sr[POST] = s;
-        float acc = 0.0f;
-#pragma unroll
-        for (int j = 0; j < SIZE; ++j) acc += tr[j];
-        bp[(long)c * HW] = dr[0] * pow_neg_beta(sr[0], nbeta) - ratio * xp[(long)c * HW] * acc;
     }
 }
 
@@ -148,10 +194,11 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_bwd_generic_kernel(
     const float* __restrict__ top_diff, float* __restrict__ bottom_diff, int C, int HW, int crun,
     int size, float nbeta, float ratio) {
     const int pre = size - (size + 1) / 2, post = size - pre - 1;
-    const int p = blockIdx.x * kLrnThreads + threadIdx.x;
+    const LrnBlock blk = lrn_block(HW, C, crun);
+    const int p = blk.px * kLrnThreads + threadIdx.x;
     if (p >= HW) return;
-    const long n = blockIdx.z;
-    const int cs = blockIdx.y * crun, ce = min(C, cs + crun);
+    const long n = blk.n;
+    const int cs = blk.run * crun, ce = min(C, cs + crun);
     const long base = n * C * (long)HW + p;
     for (int c = cs; c < ce; ++c) {
         float acc = 0.0f;
@@ -168,18 +215,23 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_bwd_generic_kernel(
 static int check_lrn(const char* what, long N, long C, long H, long W, int size) {
     CGT_ARG_CHECK(N >= 0 && C >= 0 && H >= 0 && W >= 0, "%s: negative shape", what);
     CGT_ARG_CHECK(size >= 1 && size <= C, "%s: need 1 <= size <= C, got size=%d C=%ld", what, size, C);
-    CGT_ARG_CHECK(H * W < (1L << 31) && C < (1L << 31) && N < 65536, "%s: shape too large", what);
+    CGT_ARG_CHECK(H * W < (1L << 31) && C < (1L << 31) && cdiv(H * W, kLrnThreads) * C * N < (1L << 31), "%s: shape too large", what);
     return CGT_AMD_OK;
 }
 
-// channels per thread run: short enough to fill the chip, long enough that the
-// halo re-read (size-1 channels per run) stays small.
+// Channels per thread run.  Short runs win on this chip even though each run
+// re-reads a halo of size-1 channels: more, shorter workgroups balance better
+// (measured on the AlexNet and VGG shapes: 16 beats 32, 48 and 96).  Small
+// problems go shorter still so that every CU gets work.
 static int pick_crun(long N, int C, int HW, int size) {
     const long pix_blocks = cdiv(HW, kLrnThreads) * N;
     int crun = C;
-    const int min_run = std::max(8 * size, 16);
-    while (crun > min_run && pix_blocks * cdiv(C, crun) < 2048) crun = (crun + 1) / 2;
-    return crun;
+    const int min_run = std::max(3 * size, 16);
+    while (crun > min_run && pix_blocks * cdiv(C, crun) < 8192) crun = (crun + 1) / 2;
+    crun = std::min(C, std::max(crun, min_run));
+    const int floor_run = std::max(size, 8);
+    while (crun > floor_run && pix_blocks * cdiv(C, crun) < 1024) crun = (crun + 1) / 2;
+    return std::min(C, std::max(crun, floor_run));
 }
 
 }  // namespace cgt_amd
@@ -196,7 +248,7 @@ CGT_API int cgt_amd_lrn_fwd_f32(const float* x, long N, long C, long H, long W, 
     CGT_ARG_CHECK(k > 0, "lrn_fwd: k must be positive");
     const int HW = (int)(H * W);
     const int crun = pick_crun(N, (int)C, HW, size);
-    dim3 grid((unsigned)cdiv(HW, kLrnThreads), (unsigned)cdiv(C, crun), (unsigned)N), block(kLrnThreads);
+    dim3 grid((unsigned)(cdiv(HW, kLrnThreads) * cdiv(C, crun) * N)), block(kLrnThreads);
     hipStream_t st = as_stream(stream);
     const float aos = (float)(alpha / size), nbeta = (float)(-beta), kc = (float)k;
 #define LRN_FWD_CASE(S)                                                                           \
@@ -223,7 +275,7 @@ CGT_API int cgt_amd_lrn_bwd_f32(const float* x, const float* top, const float* s
     CGT_ARG_CHECK(x && top && scale && top_diff && bottom_diff, "lrn_bwd: null pointer");
     const int HW = (int)(H * W);
     const int crun = pick_crun(N, (int)C, HW, size);
-    dim3 grid((unsigned)cdiv(HW, kLrnThreads), (unsigned)cdiv(C, crun), (unsigned)N), block(kLrnThreads);
+    dim3 grid((unsigned)(cdiv(HW, kLrnThreads) * cdiv(C, crun) * N)), block(kLrnThreads);
     hipStream_t st = as_stream(stream);
     const float nbeta = (float)(-beta), ratio = (float)(2. * alpha * beta / size);
 #define LRN_BWD_CASE(S)                                                                      \

@@ -162,6 +162,81 @@ __global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_kernel(
     }
 }
 
+constexpr int cfloordiv(int a, int b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }   // b > 0
+constexpr int cceildiv(int a, int b) { return -cfloordiv(-a, b); }
+
+// Pullback for geometries known at compile time.  A thread owns one stride-sized
+// block of input cells (rows by*SH.., columns bx*SW..).  Relative to (by, bx) the
+// windows that can cover a cell of the block sit at offsets fixed by the
+// geometry, so the thread loads that small neighbourhood of (mask, top_diff)
+// once, straight from global memory (consecutive threads read consecutive
+// pooled cells), and every cell adds the windows that name it, in ascending
+// (ph, pw) as the reference's sequential scatter does.  No division per cell,
+// no LDS, no barrier.
+template <class G>
+__global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_block_kernel(
+    G, const int* __restrict__ mask, const float* __restrict__ top_diff,
+    float* __restrict__ bottom_diff, long nplanes, int H, int W, int PH, int PW, int BH, int BW,
+    int planes_per_wg, int vec2) {
+    constexpr int KH = G::kKH, KW = G::kKW, PDH = G::kPH, PDW = G::kPW, SH = G::kSH, SW = G::kSW;
+    constexpr int DY0 = cceildiv(PDH - KH + 1, SH), DY1 = cfloordiv(SH - 1 + PDH, SH);
+    constexpr int DX0 = cceildiv(PDW - KW + 1, SW), DX1 = cfloordiv(SW - 1 + PDW, SW);
+    constexpr int NY = DY1 - DY0 + 1, NX = DX1 - DX0 + 1;
+    const long p0 = (long)blockIdx.x * planes_per_wg;
+    const long left = nplanes - p0;
+    const int np = left < planes_per_wg ? (int)left : planes_per_wg;
+    const int HW = H * W, PP = PH * PW, per_plane = BH * BW;
+    const int n = np * per_plane;
+    const float rPer = 1.0f / per_plane, rBW = 1.0f / BW;
+    for (int j = threadIdx.x; j < n; j += kPoolThreads) {
+        const int pl = fastdiv(j, rPer), r = j - pl * per_plane;
+        const int by = fastdiv(r, rBW), bx = r - by * BW;
+        const int* mk = mask + (p0 + pl) * PP;
+        const float* td = top_diff + (p0 + pl) * PP;
+        int mv[NY][NX];
+        float tv[NY][NX];
+#pragma unroll
+        for (int dy = 0; dy < NY; ++dy)
+#pragma unroll
+            for (int dx = 0; dx < NX; ++dx) {
+                const int y = by + DY0 + dy, x = bx + DX0 + dx;
+                const bool ok = y >= 0 && y < PH && x >= 0 && x < PW;
+                mv[dy][dx] = ok ? mk[y * PW + x] : -1;
+                tv[dy][dx] = ok ? td[y * PW + x] : 0.0f;
+            }
+        float* dst = bottom_diff + (p0 + pl) * HW;
+#pragma unroll
+        for (int i = 0; i < SH; ++i) {
+            const int h = by * SH + i;
+            if (h >= H) break;
+            float out[SW];
+#pragma unroll
+            for (int jj = 0; jj < SW; ++jj) {
+                const int cell = h * W + bx * SW + jj;
+                float acc = 0.0f;
+#pragma unroll
+                for (int dy = 0; dy < NY; ++dy)
+#pragma unroll
+                    for (int dx = 0; dx < NX; ++dx) {
+                        // does window offset (dy, dx) cover cell (i, jj) of the block?
+                        const bool covers = DY0 + dy >= cceildiv(i + PDH - KH + 1, SH) && DY0 + dy <= cfloordiv(i + PDH, SH) &&
+                                            DX0 + dx >= cceildiv(jj + PDW - KW + 1, SW) && DX0 + dx <= cfloordiv(jj + PDW, SW);
+                        if (covers) acc = (mv[dy][dx] == cell) ? acc + tv[dy][dx] : acc;
+                    }
+                out[jj] = acc;
+            }
+            float* row = dst + h * W + bx * SW;
+            if (SW == 2 && vec2) {
+                *reinterpret_cast<float2*>(row) = make_float2(out[0], out[SW - 1]);
+            } else {
+#pragma unroll
+                for (int jj = 0; jj < SW; ++jj)
+                    if (bx * SW + jj < W) row[jj] = out[jj];
+            }
+        }
+    }
+}
+
 template <class G>
 __global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_direct_kernel(
     G g, const int* __restrict__ mask, const float* __restrict__ top_diff,
@@ -238,6 +313,20 @@ static int launch_pool_fwd(G g, const float* bottom, long nplanes, long H, long 
 template <class G>
 static int launch_pool_bwd(G g, const int* mask, const float* top_diff, long nplanes, long H, long W,
                            long PH, long PW, float* bottom_diff, hipStream_t st) {
+    if constexpr (G::is_static) {
+        const long BH = cdiv(H, (long)G::kSH), BW = cdiv(W, (long)G::kSW);
+        if (BH * BW <= (1L << 18) && H * W < (1L << 30)) {
+            // a few thousand blocks per workgroup, at least one plane
+            const int ppw = (int)std::max(1L, std::min(2048 / (BH * BW), cdiv(nplanes, 4096L)));
+            const long blocks = cdiv(nplanes, ppw);
+            const int vec2 = W % 2 == 0 && reinterpret_cast<uintptr_t>(bottom_diff) % 8 == 0;
+            max_pool_bwd_block_kernel<G><<<dim3((unsigned)blocks), dim3(kPoolThreads), 0, st>>>(
+                g, mask, top_diff, bottom_diff, nplanes, (int)H, (int)W, (int)PH, (int)PW, (int)BH,
+                (int)BW, ppw, vec2);
+            CGT_LAUNCH_CHECK("max_pool_bwd_block_kernel");
+            return CGT_AMD_OK;
+        }
+    }
     const long out_bytes = PH * PW * 2 * (long)sizeof(float);  // top_diff + mask per plane
     if (out_bytes <= 48 * 1024) {
         int ppw = (int)std::max(1L, (16 * 1024) / out_bytes);

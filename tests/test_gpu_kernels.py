@@ -146,6 +146,9 @@ POOL_CASES = [
     ((3, 2, 9, 13), (2, 3), (0, 1), (2, 1)),
     ((1, 2, 130, 120), (3, 3), (0, 0), (2, 2)),    # plane too large for LDS staging
     ((1, 1, 3, 3), (2, 2), (0, 0), (2, 2)),        # one output
+    ((2, 3, 11, 13), (3, 3), (1, 1), (2, 2)),      # compiled-in geometry, odd extents, padding
+    ((3, 4, 7, 9), (2, 2), (0, 0), (2, 2)),        # odd width: no paired stores in the pullback
+    ((600, 9, 6, 6), (2, 2), (0, 0), (2, 2)),      # many small planes per workgroup
 ]
 
 

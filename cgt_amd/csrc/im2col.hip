@@ -284,10 +284,20 @@ __global__ __launch_bounds__(256) void col2im_gather_kernel(
 // (coalesced; the buffer is read once apart from kh-sh halo rows per band and
 // the kw-sw halo columns per tile).  The global loads of row h-1 are issued
 // into registers before row h is consumed, so their latency is hidden.
-template <class G, int CC, int WSUB, bool VEC>
+//
+// Staging modes: kStageScalar (4-byte loads), kStageRuns (16-byte loads inside
+// each run; needs CC*kh*kw % 4 == 0 and C % CC == 0), kStageLinear (CC == C, so
+// the runs of neighbouring pixels are adjacent in memory and a row's staged
+// pixels are ONE contiguous block: it is copied with 16-byte loads from the
+// 16-byte boundary below its first float, whatever its alignment, and lands in
+// LDS at the same offset from that boundary, with no index arithmetic at all).
+constexpr int kStageScalar = 0, kStageRuns = 1, kStageLinear = 2;
+
+template <class G, int CC, int WSUB, int MODE>
 __global__ __launch_bounds__(256) void col2im_stream_kernel(
     G g, const float* __restrict__ col, float* __restrict__ im, int C, int H, int W, int m, int n,
-    int band, int bands, int tiles_w, int nchunks) {
+    int band, int bands, int tiles_w, int nchunks, long col_floats) {
+    constexpr bool VEC = MODE == kStageRuns, LIN = MODE == kStageLinear;
     constexpr int KH = G::kKH, KW = G::kKW, PH = G::kPH, PW = G::kPW, SH = G::kSH, SW = G::kSW;
     static_assert(SH <= KH && SW <= KW, "streaming col2im needs stride <= kernel");
     constexpr int KK = KH * KW, RUN = CC * KK;
@@ -297,8 +307,10 @@ __global__ __launch_bounds__(256) void col2im_stream_kernel(
     constexpr int NT = (KW + SW - 1) / SW;            // taps per row and pixel
     constexpr int NWB = (TW + KW - 2) / SW + 1;       // staged pixels per row, upper bound
     // staged values per thread: float4 units of full runs (VEC) or single floats
-    constexpr int NP = VEC ? (NWB * (RUN / 4) + 255) / 256 : (NWB * RUN + 255) / 256;
-    extern __shared__ float stage[];                  // [nw][LD]
+    constexpr int NP = LIN ? ((NWB * RUN + 6) / 4 + 255) / 256
+                     : VEC ? (NWB * (RUN / 4) + 255) / 256 : (NWB * RUN + 255) / 256;
+    static_assert(!LIN || LD == RUN, "linear staging keeps the memory layout: the run length must be odd");
+    extern __shared__ __attribute__((aligned(16))) float stage[];   // [nw][LD] (+ up to 3 floats of lead-in)
 
     long bid = xcd_remap(blockIdx.x, gridDim.x);
     const int bd = (int)(bid % bands);                // bands of one image/chunk are neighbours
@@ -340,24 +352,57 @@ __global__ __launch_bounds__(256) void col2im_stream_kernel(
     const int t_bot = hp0 + PH - (KH - 1);
     const int h_bot = t_bot >= 0 ? (t_bot + SH - 1) / SH : -((-t_bot) / SH);
 
-    typename std::conditional<VEC, float4, float>::type pre[NP];
-    auto prefetch = [&](int h) {
+    typedef typename std::conditional<VEC || LIN, float4, float>::type PreT;
+    PreT pre0[NP], pre1[NP];        // two rows in flight
+    int lead = 0, lead0 = 0, lead1 = 0;   // LIN: floats between the 16-byte boundary and the row's first float
+    auto prefetch = [&](PreT (&pre)[NP], int& lead_next, int h) {
         if (h < 0 || h >= m || nw <= 0) return;
         const float* src = col + ((b * m + h) * (long)n + w_lo) * Z + (long)c0 * KK;
+        if constexpr (LIN) {
+            lead_next = (int)((reinterpret_cast<uintptr_t>(src) >> 2) & 3);
+            const float* al = src - lead_next;           // col is 16-byte aligned: never below it
+            const long off = al - col;
+            const int n4 = (nw * RUN + lead_next + 3) >> 2;
+#pragma unroll
+            for (int u = 0; u < NP; ++u) {
+                const int idx = threadIdx.x + u * 256;
+                if (idx < n4) {
+                    if (off + 4L * idx + 3 < col_floats) {
+                        pre[u] = reinterpret_cast<const float4*>(al)[idx];
+                    } else {                             // last floats of the whole buffer
+                        float t[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) t[j] = off + 4L * idx + j < col_floats ? al[4 * idx + j] : 0.0f;
+                        pre[u] = make_float4(t[0], t[1], t[2], t[3]);
+                    }
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int u = 0; u < NP; ++u) {
             const int idx = threadIdx.x + u * 256;
             if constexpr (VEC) {
                 const int w = idx / (RUN / 4), z4 = (idx - w * (RUN / 4)) * 4;
                 if (idx < total) pre[u] = *reinterpret_cast<const float4*>(src + (long)w * Z + z4);
-            } else {
+            } else if constexpr (!LIN) {
                 const int w = full ? idx / RUN : idx / run;
                 const int zc = idx - w * run;
                 if (idx < total) pre[u] = src[(long)w * Z + zc];
             }
         }
     };
-    auto park = [&]() {
+    auto park = [&](const PreT (&pre)[NP], int lead_next) {
+        if constexpr (LIN) {
+            lead = lead_next;
+            const int n4 = (nw * RUN + lead + 3) >> 2;
+#pragma unroll
+            for (int u = 0; u < NP; ++u) {
+                const int idx = threadIdx.x + u * 256;
+                if (idx < n4) reinterpret_cast<float4*>(stage)[idx] = pre[u];
+            }
+            return;
+        }
 #pragma unroll
         for (int u = 0; u < NP; ++u) {
             const int idx = threadIdx.x + u * 256;
@@ -367,7 +412,7 @@ __global__ __launch_bounds__(256) void col2im_stream_kernel(
                     float* d = stage + w * LD + z4;
                     d[0] = pre[u].x; d[1] = pre[u].y; d[2] = pre[u].z; d[3] = pre[u].w;
                 }
-            } else {
+            } else if constexpr (!LIN) {
                 const int w = full ? idx / RUN : idx / run;
                 const int zc = idx - w * run;
                 if (idx < total) stage[w * LD + zc] = pre[u];
@@ -375,29 +420,31 @@ __global__ __launch_bounds__(256) void col2im_stream_kernel(
         }
     };
 
-    prefetch(h_top);
-    for (int h = h_top; h >= h_bot; --h) {
+    // one column-buffer row: park it (its loads were issued two rows ago), refill
+    // the same registers with the row two below, then consume it from LDS
+    auto row_step = [&](PreT (&pre)[NP], int& lead_slot, int h) {
         const bool live = h >= 0 && h < m && nw > 0;      // uniform over the workgroup
         if (live) {
-            park();
+            park(pre, lead_slot);
             __syncthreads();
         }
-        if (h > h_bot) prefetch(h - 1);
+        if (h - 2 >= h_bot) prefetch(pre, lead_slot, h - 2);
         if (live) {
 #pragma unroll
             for (int i = 0; i < NQ; ++i) {
                 if (!ok[i]) continue;
+                // tap t of pixel column wp: wo = r + t*SW from staged pixel wq - t;
+                // for one accumulator the taps come in ascending wo
                 const int wpp = wp[i] + PW;
-                const int r = wpp % SW;
+                const int r = wpp % SW, wq = wpp / SW;
+                const float* sp = stage + lead + (wq - w_lo) * LD + cq[i] * KK + r;
 #pragma unroll
-                for (int ho = 0; ho < KH; ++ho) {
+                for (int t = 0; t < NT; ++t) {
+                    const int wo = r + t * SW, w = wq - t;
+                    if (wo < KW && w >= 0 && w <= w_hi) {
+                        const float* st = sp + t * (SW - LD);
 #pragma unroll
-                    for (int t = 0; t < NT; ++t) {
-                        const int wo = r + t * SW;
-                        const int ww = wpp - wo;
-                        const int w = ww / SW;
-                        if (wo < KW && ww >= 0 && w <= w_hi)
-                            acc[i][ho] += stage[(w - w_lo) * LD + (cq[i] * KH + ho) * KW + wo];
+                        for (int ho = 0; ho < KH; ++ho) acc[i][ho] += st[ho * KW];
                     }
                 }
             }
@@ -420,6 +467,12 @@ __global__ __launch_bounds__(256) void col2im_stream_kernel(
 #pragma unroll
             for (int ho = 0; ho < SH; ++ho) acc[i][ho] = 0.0f;
         }
+    };
+    prefetch(pre0, lead0, h_top);
+    if (h_top - 1 >= h_bot) prefetch(pre1, lead1, h_top - 1);
+    for (int h = h_top; h >= h_bot; h -= 2) {
+        row_step(pre0, lead0, h);
+        if (h - 1 >= h_bot) row_step(pre1, lead1, h - 1);
     }
     // rows of the band below the lowest window (still open in the window)
     const int base = (h_bot - 1) * SH - PH;
@@ -440,24 +493,34 @@ static int launch_col2im_stream(G g, const float* col, long B, int C, int H, int
                                 float* im, hipStream_t st) {
     constexpr int KK = G::kKH * G::kKW, RUN = CC * KK, LD = RUN | 1, TW = 64 * WSUB;
     const int tiles_w = (int)cdiv(W, TW), nchunks = (int)cdiv(C, CC);
-    // bands: at least two workgroups per CU, but tall enough that the kh - sh
-    // halo rows stay a small fraction (measured: fewer, taller bands win)
-    const long per_band = B * nchunks * tiles_w;
-    long bands = std::max(1L, std::min(cdiv(512, per_band), (long)H / (4 * G::kKH)));
-    int band = (int)cdiv(cdiv(H, bands), G::kSH) * G::kSH;       // bands start on stride multiples
-    bands = cdiv(H, band);
     const long nwb = std::min((long)n, (long)(TW + G::kKW - 2) / G::kSW + 1);
-    const size_t lds = (size_t)nwb * LD * sizeof(float);
-    const long blocks = per_band * bands;
-    CGT_ARG_CHECK(blocks < (1L << 31) && lds <= 64 * 1024, "col2im: tile configuration out of range");
+    const size_t lds = ((size_t)nwb * LD + 8) * sizeof(float);
+    CGT_ARG_CHECK(lds <= 64 * 1024, "col2im: tile configuration out of range");
     const long Z = (long)C * KK;
-    const bool vec = RUN % 4 == 0 && C % CC == 0 && reinterpret_cast<uintptr_t>(col) % 16 == 0;
-    if (vec)
-        col2im_stream_kernel<G, CC, WSUB, (RUN % 4 == 0)><<<dim3((unsigned)blocks), dim3(256), lds, st>>>(
-            g, col, im, C, H, W, m, n, band, (int)bands, tiles_w, nchunks);
-    else
-        col2im_stream_kernel<G, CC, WSUB, false><<<dim3((unsigned)blocks), dim3(256), lds, st>>>(
-            g, col, im, C, H, W, m, n, band, (int)bands, tiles_w, nchunks);
+    const long col_floats = B * m * (long)n * Z;
+    const bool al16 = reinterpret_cast<uintptr_t>(col) % 16 == 0;
+    const int mode = (LD == RUN && C == CC && al16) ? kStageLinear
+                     : (RUN % 4 == 0 && C % CC == 0 && al16) ? kStageRuns : kStageScalar;
+    auto kernel = mode == kStageLinear ? col2im_stream_kernel<G, CC, WSUB, (LD == RUN ? kStageLinear : kStageScalar)>
+                  : mode == kStageRuns ? col2im_stream_kernel<G, CC, WSUB, (RUN % 4 == 0 ? kStageRuns : kStageScalar)>
+                                       : col2im_stream_kernel<G, CC, WSUB, kStageScalar>;
+    // Bands of image rows: as many workgroups as the chip holds at once, and
+    // no more.  The kernel is bound by the loads each wavefront can keep in
+    // flight, so resident wavefronts are what counts; a second, partial round
+    // of workgroups costs more than it gains (measured on the AlexNet layer:
+    // 2 bands 0.17 ms, 3 bands 0.21 ms), and each band re-reads kh - sh halo
+    // rows, so bands stay at least 4 kernel heights tall.
+    int wg_per_cu = 0;
+    CGT_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&wg_per_cu, kernel, 256, lds));
+    const long resident = (long)std::max(wg_per_cu, 1) * kNumCU;
+    const long per_band = B * nchunks * tiles_w;
+    long bands = std::max(1L, std::min(resident / per_band, (long)H / (4 * G::kKH)));
+    const int band = (int)cdiv(cdiv(H, bands), G::kSH) * G::kSH;   // bands start on stride multiples
+    bands = cdiv(H, band);
+    const long blocks = per_band * bands;
+    CGT_ARG_CHECK(blocks < (1L << 31), "col2im: too many workgroups");
+    kernel<<<dim3((unsigned)blocks), dim3(256), lds, st>>>(g, col, im, C, H, W, m, n, band, (int)bands,
+                                                           tiles_w, nchunks, col_floats);
     CGT_LAUNCH_CHECK("col2im_stream_kernel");
     return CGT_AMD_OK;
 }
@@ -582,7 +645,7 @@ static int try_col2im_stream(StaticGeom<5, 5, 2, 2, 1, 1> g, const float* col, l
 }
 static int try_col2im_stream(StaticGeom<11, 11, 0, 0, 4, 4> g, const float* col, long B, int C, int H,
                            int W, int m, int n, float* im, hipStream_t st) {
-    if (C == 3 && W >= 64) return launch_col2im_stream<decltype(g), 3, 2>(g, col, B, C, H, W, m, n, im, st);
+    if (C == 3 && W >= 64) return launch_col2im_stream<decltype(g), 3, 1>(g, col, B, C, H, W, m, n, im, st);
     return -1;
 }
 

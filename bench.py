@@ -83,9 +83,17 @@ class Stage(object):
 class LayerOnGpu(object):
     """One configured layer with every buffer pre-allocated on the device."""
 
-    def __init__(self, cfg, stream=None):
-        from cgt_amd import kernels as K
+    def __init__(self, cfg, overlap=True):
+        from cgt_amd import capi, kernels as K
         from cgt_amd.gpuarray import empty, to_gpu
+        # two streams (default priority): the weight-gradient GEMM depends only on
+        # the transposed output gradient and the column buffer, so step() runs
+        # it beside the data-gradient GEMM + col2im
+        self._main, self._side = capi.Stream(), capi.Stream()
+        self._fork, self._join = capi.Event(), capi.Event()
+        self.overlap = overlap
+        stream = self._main.handle
+        self._wgrad_stream = stream
         self.cfg, self.K, self.stream = cfg, K, stream
         x, f = make_inputs(cfg)
         B, C, H, W = x.shape
@@ -153,14 +161,32 @@ class LayerOnGpu(object):
         st.append(Stage("col2im", "col2im_stream_kernel",
                         lambda: K.col2im(self.gcol.reshape(B, m, n, Z), self.x.shape, (r, c), pad, stride, out=self.gx, stream=s),
                         4 * (nelem(self.x) + nelem(self.col)), "hbm"))
-        st.append(Stage("gemm_wgrad_TN", "sgemm_kernel", lambda: K.mul22(self.gc2, self.col2, True, False, out=self.gf, stream=s),
+        st.append(Stage("gemm_wgrad_TN", "sgemm_kernel", lambda: K.mul22(self.gc2, self.col2, True, False, out=self.gf, stream=self._wgrad_stream),
                         2 * Bmn * L * Z, "mfma"))
         self.stages = st
         self.conv_flops = 6 * Bmn * L * Z
 
     def step(self):
+        from cgt_amd import capi
+        if not self.overlap:
+            for st in self.stages:
+                st.fn()
+            return
+        main, side = self._main.handle, self._side.handle
         for st in self.stages:
+            if st.name == "gemm_wgrad_TN":       # join: the next step overwrites its operands
+                capi.stream_wait_event(main, self._join)
+                continue
             st.fn()
+            if st.name == "gemm_dgrad_NN":
+                # fork after the data-gradient GEMM: the weight-gradient GEMM (matrix
+                # cores) then shares the chip with col2im (HBM), not with another GEMM
+                self._fork.record(main)
+                capi.stream_wait_event(side, self._fork)
+                self._wgrad_stream = side
+                self.stages[-1].fn()
+                self._wgrad_stream = main
+                self._join.record(side)
 
     def time_stages(self, reps):
         from cgt_amd import capi
@@ -286,6 +312,8 @@ def main():
     ap.add_argument("--stage-reps", type=int, default=20)
     ap.add_argument("--cpu-sample", type=int, default=16, help="images in the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="issue every stage on one stream (default: weight-gradient GEMM on a second stream)")
     ap.add_argument("--no-check", action="store_true",
                     help="skip the parity gate (profiling runs: keeps its small launches out of the kernel statistics)")
     args = ap.parse_args()
@@ -302,7 +330,7 @@ def main():
         parity = {"ok": True, "skipped": True} if args.no_check else check_gemm_against_oracle()
     else:
         cfg = WORKLOADS[args.workload]
-        layer = LayerOnGpu(cfg)
+        layer = LayerOnGpu(cfg, overlap=not args.no_overlap)
         parity = {"ok": True, "skipped": True} if args.no_check else check_against_oracle(cfg)
 
     for _ in range(args.warmup):
@@ -341,7 +369,9 @@ def main():
         "config": {"workload": args.workload, "x": list(cfg["x"]), "filters": list(cfg["f"]),
                    "pad": list(cfg["pad"]), "stride": list(cfg["stride"]),
                    "value_is": "conv GEMM flops (6*B*m*n*L*Z) / whole step time incl. im2col, col2im, "
-                               "transposes, pool and LRN stages"},
+                               "transposes, pool and LRN stages",
+                   "schedule": ("one stream" if is_gemm or args.no_overlap else
+                                "weight-gradient GEMM on a second stream beside col2im")},
         "frac_fp32_mfma_peak": round(value / FP32_MFMA_PEAK_TFLOPS, 4),
         # the dominant kernel: the slowest MFMA GEMM launch of a step
         "roofline": {"bound": "mfma", "kernel": dominant.kernel, "stage": dominant.name,

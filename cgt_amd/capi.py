@@ -33,6 +33,7 @@ PROTOTYPES = {
     "cgt_amd_event_create": (c_int, [ctypes.POINTER(c_void_p)]),
     "cgt_amd_event_destroy": (c_int, [c_void_p]),
     "cgt_amd_event_record": (c_int, [c_void_p, c_void_p]),
+    "cgt_amd_stream_wait_event": (c_int, [c_void_p, c_void_p]),
     "cgt_amd_event_elapsed_ms": (c_int, [c_void_p, c_void_p, ctypes.POINTER(ctypes.c_float)]),
     "cgt_amd_im2col_f32": (c_int, [c_void_p] + [c_long] * 4 + [c_int] * 6 + [c_void_p, c_void_p]),
     "cgt_amd_col2im_f32": (c_int, [c_void_p] + [c_long] * 4 + [c_int] * 6 + [c_void_p, c_void_p]),
@@ -108,6 +109,11 @@ def device_name():
 
 def synchronize(stream=None):
     check(lib().cgt_amd_synchronize(stream))
+
+
+def stream_wait_event(stream, event):
+    """Later work on `stream` waits for the work recorded in `event`."""
+    check(lib().cgt_amd_stream_wait_event(stream, event.handle))
 
 
 class Stream(object):

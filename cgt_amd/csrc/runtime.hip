@@ -142,6 +142,12 @@ CGT_API int cgt_amd_event_record(void* event, void* stream) {
     return CGT_AMD_OK;
 }
 
+CGT_API int cgt_amd_stream_wait_event(void* stream, void* event) {
+    CGT_ARG_CHECK(event, "stream_wait_event: null event");
+    CGT_HIP_TRY(hipStreamWaitEvent(as_stream(stream), static_cast<hipEvent_t>(event), 0));
+    return CGT_AMD_OK;
+}
+
 CGT_API int cgt_amd_event_elapsed_ms(void* start, void* stop, float* ms) {
     CGT_ARG_CHECK(start && stop && ms, "event_elapsed: null");
     CGT_HIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(stop)));

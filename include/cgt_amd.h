@@ -76,6 +76,10 @@ int cgt_amd_stream_destroy(void *stream);
 int cgt_amd_event_create(void **event);
 int cgt_amd_event_destroy(void *event);
 int cgt_amd_event_record(void *event, void *stream);
+/* Work issued to `stream` after this call starts only once the work recorded
+ * in `event` is done: lets a host run independent branches of the backward
+ * graph (weight gradient | data gradient + col2im) on two streams. */
+int cgt_amd_stream_wait_event(void *stream, void *event);
 int cgt_amd_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for stop */
 
 /* ---------------------------------------------------------------- im2col / col2im */

@@ -55,7 +55,9 @@ DEFAULT_WORKLOAD = "vgg_mid_conv3x3_128x56x56_b64"
 # WRITE_SIZE runs of this script (summaries and calibration in profiles/):
 # (workload, stage) -> bytes.  None where no counter run has been made.
 TRAFFIC = {
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_fwd_NT"): 1050000000,   # 2.0 * 473.6 MB fetched + 102.8 MB written
+    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_fwd_NT"): 1060500000,    # 2.0 * 472.6 MB fetched + 115.3 MB written
+    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_dgrad_NN"): 1136000000,  # 2.0 * 105.6 MB fetched + 924.8 MB written
+    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_wgrad_TN"): 1125500000,  # 2.0 * 529.7 MB fetched + 66.1 MB written (partials incl.)
 }
 
 
@@ -117,7 +119,7 @@ class LayerOnGpu(object):
                         4 * (nelem(self.x) + nelem(self.col)), "hbm"))
         st.append(Stage("gemm_fwd_NT", "sgemm_kernel", lambda: K.mul22(self.col2, self.f_LZ, False, True, out=self.y_mnL, stream=s),
                         2 * Bmn * L * Z, "mfma"))
-        st.append(Stage("transpose_0312", "batched_transpose_kernel",
+        st.append(Stage("transpose_0312", "thin_transpose_kernel or batched_transpose_kernel",
                         lambda: K.transpose4(self.y_mnL.reshape(B, m, n, L), (0, 3, 1, 2), out=self.y, stream=s),
                         2 * 4 * nelem(self.y), "hbm"))
         if cfg["lrn"]:
@@ -135,7 +137,7 @@ class LayerOnGpu(object):
             pool_in = act
             st.append(Stage("max_pool_fwd", "max_pool_fwd_kernel", lambda: K.max_pool(pool_in, pk, pp, ps, out=(self.pool, self.mask), stream=s),
                             4 * (nelem(self.y) + 2 * nelem(self.pool)), "hbm"))
-            st.append(Stage("max_pool_bwd", "max_pool_bwd_kernel",
+            st.append(Stage("max_pool_bwd", "max_pool_bwd_block_kernel",
                             lambda: K.max_pool_pullback(self.y.shape, self.mask, self.gpool, pk, pp, ps, out=self.gact, stream=s),
                             4 * (2 * nelem(self.pool) + nelem(self.y)), "hbm"))
             gy = self.gact
@@ -154,7 +156,7 @@ class LayerOnGpu(object):
         self.gcol = empty((Bmn, Z))
         self.gx = empty(self.x.shape)
         self.gf = empty((L, Z))
-        st.append(Stage("transpose_0231", "batched_transpose_kernel", lambda: K.transpose4(self.gy, (0, 2, 3, 1), out=self.gc, stream=s),
+        st.append(Stage("transpose_0231", "thin_transpose_kernel or batched_transpose_kernel", lambda: K.transpose4(self.gy, (0, 2, 3, 1), out=self.gc, stream=s),
                         2 * 4 * nelem(self.y), "hbm"))
         st.append(Stage("gemm_dgrad_NN", "sgemm_kernel", lambda: K.mul22(self.gc2, self.f_LZ, False, False, out=self.gcol, stream=s),
                         2 * Bmn * L * Z, "mfma"))
@@ -223,6 +225,7 @@ class GemmOnGpu(object):
         st.append(Stage("batched_mul22_%dx%d" % (P, nb), "sgemm_kernel",
                         lambda: K.batched_mul22(self.bA, self.bB, out=self.bC, stream=s), 2 * P * nb ** 3, "mfma"))
         self.stages = st
+        self.overlap = False
         self.conv_flops = sum(x.work for x in st)
 
     step = LayerOnGpu.step

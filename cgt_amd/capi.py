@@ -51,6 +51,11 @@ PROTOTYPES = {
     "cgt_amd_sgemm_batched": (c_int, [c_int, c_int, c_long, c_long, c_long, c_long,
                                       c_void_p, c_long, c_long, c_void_p, c_long, c_long,
                                       c_void_p, c_long, c_long, c_void_p]),
+    "cgt_amd_elwise_unary_f32": (c_int, [c_int, c_long, c_void_p, c_void_p, c_void_p]),
+    "cgt_amd_elwise_binary": (c_int, [c_int, c_int, c_int, c_long, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p]),
+    "cgt_amd_repeat": (c_int, [c_void_p, c_int, c_int, ctypes.POINTER(c_long), ctypes.POINTER(c_int), c_void_p, c_void_p]),
+    "cgt_amd_sum_f32": (c_int, [c_void_p, c_int, ctypes.POINTER(c_long), ctypes.POINTER(c_int), c_void_p, c_void_p]),
+    "cgt_amd_fill_f32": (c_int, [c_void_p, ctypes.c_float, c_long, c_void_p]),
     "cgt_amd_transpose4_f32": (c_int, [c_void_p, ctypes.POINTER(c_long), ctypes.POINTER(c_int),
                                        c_void_p, c_void_p]),
 }

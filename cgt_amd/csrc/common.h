@@ -19,7 +19,7 @@ constexpr int kWave = 64;    // CDNA wavefront width
 constexpr int kNumXCD = 8;   // MI355X: 8 accelerator dies, each with its own L2
 constexpr int kNumCU = 256;  // MI355X compute units
 
-inline long cdiv(long a, long b) { return (a + b - 1) / b; }
+__host__ __device__ inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 
 // Geometry known at compile time (hot shapes) ...
 template <int KH, int KW, int PH, int PW, int SH, int SW>

@@ -9,8 +9,9 @@ import numpy as np
 
 from . import capi
 
-# float64 buffers exist only so tests can hand double data to checker kernels
-_DTYPES = (np.dtype(np.float32), np.dtype(np.int32), np.dtype(np.int64), np.dtype(np.float64))
+# int8 is the reference's "i1" (what comparisons produce); float64 buffers exist
+# only so tests can hand double data to checker kernels
+_DTYPES = (np.dtype(np.float32), np.dtype(np.int32), np.dtype(np.int64), np.dtype(np.float64), np.dtype(np.int8))
 
 
 class _Buffer(object):
@@ -62,7 +63,7 @@ class GpuArray(object):
         return GpuArray(shape, self.dtype, _buffer=self._buffer, _offset=self._offset)
 
     def set(self, host):
-        host = np.ascontiguousarray(host, dtype=self.dtype)
+        host = _contiguous(host, self.dtype)
         if host.shape != self.shape:
             raise ValueError("shape mismatch %s vs %s" % (host.shape, self.shape))
         capi.check(capi.lib().cgt_amd_memcpy(capi.GPU, capi.CPU, self.ptr, host.ctypes.data, self.nbytes))
@@ -85,6 +86,12 @@ def empty(shape, dtype=np.float32):
     return GpuArray(shape, dtype)
 
 
+def _contiguous(host, dtype=None):
+    """C-contiguous copy/view that keeps 0-d arrays 0-d (np.ascontiguousarray makes them 1-d)."""
+    host = np.asarray(host, dtype=dtype)
+    return host if host.ndim == 0 else np.ascontiguousarray(host)
+
+
 def to_gpu(host, dtype=None):
-    host = np.ascontiguousarray(host, dtype=dtype)
+    host = _contiguous(host, dtype)
     return GpuArray(host.shape, host.dtype).set(host)

@@ -168,6 +168,82 @@ def transpose4(x, axes, out=None, stream=None):
     return res
 
 
+# ---------------------------------------------------------------- conv-layer glue
+
+UNARY_OPS = ["abs", "cos", "exp", "log", "neg", "sign", "sin", "square", "sqrt", "tanh", "sigmoid"]
+BINARY_OPS = ["*", "+", "-", "/", "<", ">", "<=", ">=", "**", "==", "!="]
+_DTYPE_CODE = {np.dtype(np.float32): 11, np.dtype(np.int8): 1}    # cgtDtype / numpy type numbers
+
+
+def binary_out_dtype(opname, xdtype, ydtype):
+    """typ_apply of ElwiseBinary (reference cgt/core.py:1319-1333): comparisons
+    give i1, "/" gives floatX, everything else the promoted operand type."""
+    if opname in ("<", ">", "<=", ">=", "==", "!="):
+        return np.dtype(np.int8)
+    if opname == "/":
+        return np.dtype(np.float32)
+    return np.dtype(np.float32) if np.dtype(np.float32) in (np.dtype(xdtype), np.dtype(ydtype)) else np.dtype(np.int8)
+
+
+def elwise_unary(opname, x, out=None, stream=None):
+    """ElwiseUnary (reference cgt/core.py:1160-1241), float32."""
+    _f32(x)
+    y = _out(out, x.shape)
+    capi.check(capi.lib().cgt_amd_elwise_unary_f32(UNARY_OPS.index(opname), x.size, x.ptr, y.ptr, stream))
+    return y
+
+
+def elwise_binary(opname, x, y, out=None, stream=None):
+    """ElwiseBinary (reference cgt/core.py:1243-1378).  A 0-d operand is the
+    scalar side; otherwise shapes must agree (no implicit broadcasting)."""
+    sx, sy = x.ndim == 0, y.ndim == 0
+    if not sx and not sy and x.shape != y.shape:
+        raise ValueError("mismatched shapes %s %s: implicit broadcasting is not allowed, use broadcast(...)"
+                         % (x.shape, y.shape))
+    if x.dtype not in _DTYPE_CODE or y.dtype not in _DTYPE_CODE:
+        raise TypeError("elementwise ops take float32 / int8 device arrays, got %s, %s" % (x.dtype, y.dtype))
+    shape = y.shape if sx else x.shape
+    z = _out(out, shape, binary_out_dtype(opname, x.dtype, y.dtype))
+    capi.check(capi.lib().cgt_amd_elwise_binary(BINARY_OPS.index(opname), _DTYPE_CODE[x.dtype], _DTYPE_CODE[y.dtype],
+                                                z.size, x.ptr, int(sx), y.ptr, int(sy), z.ptr, stream))
+    return z
+
+
+def repeat(x, axes, reps, out=None, stream=None):
+    """Repeat(axes) (reference cgt/core.py:1511-1557): x has extent 1 on `axes`."""
+    oshape = list(x.shape)
+    flags = [0] * x.ndim
+    for ax, rep in zip(axes, reps):
+        if x.shape[ax] != 1:
+            raise ValueError("Repeat: axis %d has extent %d, not 1" % (ax, x.shape[ax]))
+        oshape[ax] = int(rep)
+        flags[ax] = 1
+    res = _out(out, tuple(oshape), x.dtype)
+    nd = max(x.ndim, 1)
+    capi.check(capi.lib().cgt_amd_repeat(x.ptr, x.dtype.itemsize, x.ndim, (ctypes.c_long * nd)(*oshape),
+                                         (ctypes.c_int * nd)(*flags), res.ptr, stream))
+    return res
+
+
+def sum_keepdims(x, axes, out=None, stream=None):
+    """Sum(axes), keepdims (reference cgt/core.py:1687-1709)."""
+    _f32(x)
+    flags = [1 if a in axes else 0 for a in range(x.ndim)]
+    oshape = tuple(1 if f else s for s, f in zip(x.shape, flags))
+    res = _out(out, oshape)
+    nd = max(x.ndim, 1)
+    capi.check(capi.lib().cgt_amd_sum_f32(x.ptr, x.ndim, (ctypes.c_long * nd)(*x.shape), (ctypes.c_int * nd)(*flags),
+                                          res.ptr, stream))
+    return res
+
+
+def fill(value, shape, out=None, stream=None):
+    """Fill(value) (reference cgt/core.py:966-1007), float32."""
+    res = _out(out, tuple(int(s) for s in shape))
+    capi.check(capi.lib().cgt_amd_fill_f32(res.ptr, float(value), res.size, stream))
+    return res
+
+
 def conv2d(x, f, pad=(0, 0), stride=(1, 1), stream=None, keep=None):
     """conv2d forward as the reference composes it on its CPU path
     (cgt/nn.py:95-100): im2col -> [B*m*n, Z] -> Mul22(False, True) with the

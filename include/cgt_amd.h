@@ -82,6 +82,73 @@ int cgt_amd_event_record(void *event, void *stream);
 int cgt_amd_stream_wait_event(void *stream, void *event);
 int cgt_amd_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for stop */
 
+/* ---------------------------------------------------------------- conv-layer glue
+ *
+ * The ops either side of the GEMM path in a SpatialConvolution training step:
+ * bias add (broadcast "+"), ReLU = x * (x >= 0), their gradients, the scalar
+ * loss and the bias gradient.  In the reference these are code-generated per
+ * op from expression tables; here one entry point per op family takes the op
+ * code. */
+
+/* Element types, numbered like cgtDtype / numpy type numbers
+ * (include/cgt_common.h:21-35): int8 "i1" and float32 "f4". */
+#define CGT_AMD_I8 1
+#define CGT_AMD_F32 11
+
+/* Unary ops, y[i] = f(x[i]), fp32.  Replaces the generated kernel of
+ * ElwiseUnary (cgt/core.py:1160-1241; expressions UNARY_INFO 1118-1134).
+ * SIGN is 2*(x>0)-1 as in the reference's native template (sign(0) = -1). */
+#define CGT_AMD_UN_ABS 0
+#define CGT_AMD_UN_COS 1
+#define CGT_AMD_UN_EXP 2
+#define CGT_AMD_UN_LOG 3
+#define CGT_AMD_UN_NEG 4
+#define CGT_AMD_UN_SIGN 5
+#define CGT_AMD_UN_SIN 6
+#define CGT_AMD_UN_SQUARE 7
+#define CGT_AMD_UN_SQRT 8
+#define CGT_AMD_UN_TANH 9
+#define CGT_AMD_UN_SIGMOID 10
+int cgt_amd_elwise_unary_f32(int op, long n, const float *x, float *y, void *stream);
+
+/* Binary ops, z[i] = f(x[i or 0], y[i or 0]).  Replaces the generated kernel
+ * of ElwiseBinary (cgt/core.py:1243-1378; expressions BINARY_INFO 1139-1152).
+ * Operand types are CGT_AMD_F32 or CGT_AMD_I8; a scalar operand is a
+ * one-element device array (`*_is_scalar` != 0), as under the reference's
+ * scalar_mask.  Output type, as typ_apply gives it: comparisons -> i1,
+ * DIV -> f4, otherwise f4 if either operand is f4, else i1.  `n` is the
+ * element count of the non-scalar operand(s) and of z. */
+#define CGT_AMD_BIN_MUL 0
+#define CGT_AMD_BIN_ADD 1
+#define CGT_AMD_BIN_SUB 2
+#define CGT_AMD_BIN_DIV 3
+#define CGT_AMD_BIN_LT 4
+#define CGT_AMD_BIN_GT 5
+#define CGT_AMD_BIN_LE 6
+#define CGT_AMD_BIN_GE 7
+#define CGT_AMD_BIN_POW 8
+#define CGT_AMD_BIN_EQ 9
+#define CGT_AMD_BIN_NE 10
+int cgt_amd_elwise_binary(int op, int xdtype, int ydtype, long n, const void *x, int x_is_scalar,
+                          const void *y, int y_is_scalar, void *z, void *stream);
+
+/* Repeat: `out` (shape outshape[ndim]) = x broadcast along the axes with
+ * repeated[a] != 0, where x has extent 1.  Replaces the nested at<>() loops of
+ * Repeat (cgt/core.py:1511-1557, cpu-only there).  itemsize 4 or 1, ndim <= 8. */
+int cgt_amd_repeat(const void *x, int itemsize, int ndim, const long *outshape, const int *repeated,
+                   void *out, void *stream);
+
+/* Sum over the axes with reduced[a] != 0, keepdims: out has extent 1 there.
+ * Replaces the reduction loop of Sum (cgt/core.py:1663-1709, cpu-only there).
+ * The summation order differs from the reference's single running sum (lanes,
+ * then a fixed tree, then partials in order) but is fixed: same input, same
+ * bits.  ndim <= 8. */
+int cgt_amd_sum_f32(const float *x, int ndim, const long *shape, const int *reduced, float *out,
+                    void *stream);
+
+/* Fill with an fp32 value (Fill op, cgt/core.py:966-1007, cpu-only there). */
+int cgt_amd_fill_f32(float *dst, float value, long count, void *stream);
+
 /* ---------------------------------------------------------------- im2col / col2im */
 
 /* Patch extraction.  im [B,C,H,W] -> col [B,m,n,Z], Z = C*kh*kw ordered

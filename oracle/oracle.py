@@ -208,3 +208,72 @@ def conv2d_pullback(x, f, gy, pad=(0, 0), stride=(1, 1)):
     gx = col2im(gcol.reshape(B, m, n, Z), x.shape, (r, c), pad, stride)
     gf = mul22(gc, col.reshape(B * m * n, Z), True, False).reshape(f.shape)
     return gx, gf
+
+
+# ---------------------------------------------------------------- conv-layer glue
+
+UNARY_OPS = ["abs", "cos", "exp", "log", "neg", "sign", "sin", "square", "sqrt", "tanh", "sigmoid"]
+BINARY_OPS = ["*", "+", "-", "/", "<", ">", "<=", ">=", "**", "==", "!="]
+
+
+def elwise_unary(opname, x):
+    """ElwiseUnary on float32 (reference cgt/core.py:1160-1218)."""
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    rc = lib().oracle_elwise_unary_f32(_c_int(UNARY_OPS.index(opname)), _c_long(x.size), _p(x), _p(out))
+    assert rc == 0
+    return out
+
+
+def elwise_binary_out_dtype(opname, xdtype, ydtype):
+    """typ_apply of ElwiseBinary (reference cgt/core.py:1319-1333)."""
+    if opname in ("<", ">", "<=", ">=", "==", "!="):
+        return np.dtype(np.int8)
+    if opname == "/":
+        return np.dtype(np.float32)
+    return np.dtype(np.float32) if np.float32 in (np.dtype(xdtype), np.dtype(ydtype)) else np.dtype(np.int8)
+
+
+def elwise_binary(opname, x, y):
+    """ElwiseBinary on float32 / int8 operands; a 0-d operand is the scalar side
+    (scalar_mask, reference cgt/core.py:1243-1349)."""
+    x, y = (a if a.ndim == 0 else np.ascontiguousarray(a) for a in (np.asarray(x), np.asarray(y)))
+    assert x.dtype in (np.float32, np.int8) and y.dtype in (np.float32, np.int8)
+    sx, sy = x.ndim == 0, y.ndim == 0
+    shape = y.shape if sx else x.shape
+    if not sx and not sy:
+        assert x.shape == y.shape, "no implicit broadcasting"
+    out = np.empty(shape, elwise_binary_out_dtype(opname, x.dtype, y.dtype))
+    fn = getattr(lib(), "oracle_elwise_binary_%s%s" % ("f" if x.dtype == np.float32 else "b",
+                                                        "f" if y.dtype == np.float32 else "b"))
+    rc = fn(_c_int(BINARY_OPS.index(opname)), _c_long(out.size), _p(x), _c_int(sx), _p(y), _c_int(sy), _p(out))
+    assert rc == 0
+    return out
+
+
+def repeat(x, axes, reps):
+    """Repeat(axes) with repeat counts `reps` (reference cgt/core.py:1511-1557)."""
+    x = np.ascontiguousarray(x)
+    oshape = list(x.shape)
+    flags = [0] * x.ndim
+    for ax, rep in zip(axes, reps):
+        assert x.shape[ax] == 1
+        oshape[ax] = int(rep)
+        flags[ax] = 1
+    out = np.empty(oshape, x.dtype)
+    rc = lib().oracle_repeat(_p(x), _c_int(x.dtype.itemsize), _c_int(x.ndim), (ctypes.c_long * max(x.ndim, 1))(*oshape),
+                             (ctypes.c_int * max(x.ndim, 1))(*flags), _p(out))
+    assert rc == 0
+    return out
+
+
+def sum_keepdims(x, axes):
+    """Sum(axes), keepdims (reference cgt/core.py:1663-1709): sequential, in the array's dtype."""
+    x = _c(x)
+    flags = [1 if a in axes else 0 for a in range(x.ndim)]
+    oshape = [1 if f else s for s, f in zip(x.shape, flags)]
+    out = np.empty(oshape, x.dtype)
+    fn = lib().oracle_sum_f32 if x.dtype == np.float32 else lib().oracle_sum_f64
+    rc = fn(_p(x), _c_int(x.ndim), (ctypes.c_long * max(x.ndim, 1))(*x.shape), (ctypes.c_int * max(x.ndim, 1))(*flags), _p(out))
+    assert rc == 0
+    return out

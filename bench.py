@@ -85,7 +85,7 @@ class Stage(object):
 class LayerOnGpu(object):
     """One configured layer with every buffer pre-allocated on the device."""
 
-    def __init__(self, cfg, overlap=True):
+    def __init__(self, cfg, overlap=True, glue=False):
         from cgt_amd import capi, kernels as K
         from cgt_amd.gpuarray import empty, to_gpu
         # two streams (default priority): the weight-gradient GEMM depends only on
@@ -167,6 +167,32 @@ class LayerOnGpu(object):
                         2 * Bmn * L * Z, "mfma"))
         self.stages = st
         self.conv_flops = 6 * Bmn * L * Z
+        # The glue a SpatialConvolution training step adds around this layer
+        # (bias add, ReLU = x*(x>=0), their gradients, scalar loss): timed in the
+        # per-kernel table only, never part of step() / `value`.
+        self.extra_stages = []
+        if glue:
+            ex = self.extra_stages
+            ny = nelem(self.y)
+            self.bias = to_gpu(np.zeros((1, L, 1, 1), np.float32))
+            self.zero = to_gpu(np.float32(0).reshape(()))
+            self.bias_full, self.pre, self.act = empty(self.y.shape), empty(self.y.shape), empty(self.y.shape)
+            self.mask_ge = empty(self.y.shape, np.int8)
+            self.gpre, self.gbias, self.loss = empty(self.y.shape), empty((1, L, 1, 1)), empty((1, 1, 1, 1))
+            ex.append(Stage("repeat_bias", "repeat_rkr_kernel",
+                            lambda: K.repeat(self.bias, (0, 2, 3), (B, m, n), out=self.bias_full, stream=s), 4 * ny, "hbm"))
+            ex.append(Stage("add_bias", "elwise_binary_kernel",
+                            lambda: K.elwise_binary("+", self.y, self.bias_full, out=self.pre, stream=s), 12 * ny, "hbm"))
+            ex.append(Stage("relu_mask_ge", "elwise_binary_kernel",
+                            lambda: K.elwise_binary(">=", self.pre, self.zero, out=self.mask_ge, stream=s), 5 * ny, "hbm"))
+            ex.append(Stage("relu_mul", "elwise_binary_kernel",
+                            lambda: K.elwise_binary("*", self.pre, self.mask_ge, out=self.act, stream=s), 9 * ny, "hbm"))
+            ex.append(Stage("relu_grad_mul", "elwise_binary_kernel",
+                            lambda: K.elwise_binary("*", self.mask_ge, self.gy, out=self.gpre, stream=s), 9 * ny, "hbm"))
+            ex.append(Stage("bias_grad_sum", "sum_rkr_kernel",
+                            lambda: K.sum_keepdims(self.gpre, (0, 2, 3), out=self.gbias, stream=s), 4 * ny, "hbm"))
+            ex.append(Stage("loss_sum", "sum_rkr_kernel",
+                            lambda: K.sum_keepdims(self.act, (0, 1, 2, 3), out=self.loss, stream=s), 4 * ny, "hbm"))
 
     def step(self):
         from cgt_amd import capi
@@ -192,7 +218,7 @@ class LayerOnGpu(object):
 
     def time_stages(self, reps):
         from cgt_amd import capi
-        for st in self.stages:
+        for st in self.stages + getattr(self, "extra_stages", []):
             st.fn()
             e0, e1 = capi.Event(), capi.Event()
             e0.record(self.stream)
@@ -317,6 +343,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-overlap", action="store_true",
                     help="issue every stage on one stream (default: weight-gradient GEMM on a second stream)")
+    ap.add_argument("--glue", action="store_true",
+                    help="also time the conv-layer glue kernels (bias add, ReLU, their gradients, loss sum) on the "
+                         "layer's activation; they appear in `glue_stages`, outside the step")
     ap.add_argument("--no-check", action="store_true",
                     help="skip the parity gate (profiling runs: keeps its small launches out of the kernel statistics)")
     args = ap.parse_args()
@@ -333,7 +362,7 @@ def main():
         parity = {"ok": True, "skipped": True} if args.no_check else check_gemm_against_oracle()
     else:
         cfg = WORKLOADS[args.workload]
-        layer = LayerOnGpu(cfg, overlap=not args.no_overlap)
+        layer = LayerOnGpu(cfg, overlap=not args.no_overlap, glue=args.glue)
         parity = {"ok": True, "skipped": True} if args.no_check else check_against_oracle(cfg)
 
     for _ in range(args.warmup):
@@ -361,6 +390,11 @@ def main():
             gemm_flops += st.work
             gemm_ms += st.ms
         stages.append(row)
+    glue_stages = []
+    for st in getattr(layer, "extra_stages", []):
+        gbs = st.work / (st.ms * 1e-3) / 1e9
+        glue_stages.append({"stage": st.name, "kernel": st.kernel, "ms": round(st.ms, 4), "bound": "hbm",
+                            "bytes": st.work, "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4)})
     gemm_tf = gemm_flops / (gemm_ms * 1e-3) / 1e12
     value = layer.conv_flops / (ms_per_step * 1e-3) / 1e12
 
@@ -385,6 +419,7 @@ def main():
                      "traffic": TRAFFIC.get((args.workload, dominant.name))},
         "gemm_all_launches": {"TFLOPs": round(gemm_tf, 2), "frac": round(gemm_tf / FP32_MFMA_PEAK_TFLOPS, 4)},
         "stages": stages,
+        "glue_stages": glue_stages,
         "parity": parity,
         "device": capi.device_name(),
     }

@@ -10,10 +10,12 @@ There is no CPU fallback: the HIP library must be built (python -m cgt_amd.build
 and a GPU visible, or calls raise.
 """
 from . import capi  # noqa: F401
-from .core import (BatchedMul22, MethodNotDefined, Mul22, NativeCallable, NativeCompileInfo, Node, Op,  # noqa: F401
-                   Reshape, Result, SrcFile, TensorType, Transport, Transpose, TupleType, as_node,
-                   batched_matmul, constant, dot, floatX, grad, reshape, shape, size, to_device,
-                   transpose, unpack)
+from .core import (BatchedMul22, ElwiseBinary, ElwiseUnary, Fill, MethodNotDefined, Mul22,  # noqa: F401
+                   NativeCallable, NativeCompileInfo, Node, Op, Repeat, Reshape, Result, SrcFile, Sum,
+                   TensorType, Transport, Transpose, TupleType, abs, as_node, batched_matmul, broadcast,
+                   constant, cos, dot, elwise_binary, exp, fill, floatX, grad, greater_equal, log, mean,
+                   neg, ones, ones_like, power, reshape, shape, sigmoid, sign, sin, size, sqrt, square,
+                   sum, tanh, to_device, transpose, unpack, zeros, zeros_like)
 from .gpuarray import GpuArray, empty, to_gpu  # noqa: F401
 
 __all__ = ["nn", "core", "capi", "kernels", "compilation", "rt"]

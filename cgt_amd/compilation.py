@@ -196,6 +196,13 @@ def prebuild_standard_ops():
         (core.Mul22(False, True), [T2, T2]),
         (core.BatchedMul22(False, False), [T3, T3]),
         (core.Transpose((0, 3, 1, 2)), [T4]),
+        # conv-layer glue: the closure code is generic over element type and
+        # rank, so one library per op class serves every use
+        (core.ElwiseUnary("exp"), [T4]),
+        (core.ElwiseBinary("+", (False, False)), [T4, T4]),
+        (core.Repeat((0, 2, 3)), [T4, S, S, S]),
+        (core.Sum((0, 2, 3)), [T4]),
+        (core.Fill(0.0), [S, S, S, S]),
     ]
     built = []
     for op, types in todo:

@@ -115,6 +115,55 @@ class Node(object):
             return unpack(self)[i]
         raise TypeError("only tuple-valued nodes can be indexed")
 
+    # arithmetic and comparisons build ElwiseBinary / ElwiseUnary results
+    # (reference core.py:204-262)
+    def __neg__(self):
+        return Result(ElwiseUnary("neg"), [self])
+
+    def __add__(self, other):
+        return elwise_binary("+", self, other)
+
+    def __sub__(self, other):
+        return elwise_binary("-", self, other)
+
+    def __mul__(self, other):
+        return elwise_binary("*", self, other)
+
+    def __truediv__(self, other):
+        return elwise_binary("/", self, other)
+
+    def __pow__(self, other):
+        return elwise_binary("**", self, other)
+
+    def __radd__(self, other):
+        return elwise_binary("+", other, self)
+
+    def __rsub__(self, other):
+        return elwise_binary("-", other, self)
+
+    def __rmul__(self, other):
+        return elwise_binary("*", other, self)
+
+    def __rtruediv__(self, other):
+        return elwise_binary("/", other, self)
+
+    def __lt__(self, other):
+        return elwise_binary("<", self, other)
+
+    def __le__(self, other):
+        return elwise_binary("<=", self, other)
+
+    def __gt__(self, other):
+        return elwise_binary(">", self, other)
+
+    def __ge__(self, other):
+        return elwise_binary(">=", self, other)
+
+    def sum(self, axis=None, keepdims=False):
+        return sum(self, axis=axis, keepdims=keepdims)
+
+    __hash__ = object.__hash__
+
     def __repr__(self):
         return "Node(%s, op=%s)" % (self.typ, self.op)
 
@@ -185,6 +234,12 @@ class Op(object):
     def pullback(self, inputs, output, goutput):
         """grad wrt each input given the gradient of the output (J^T g)."""
         raise MethodNotDefined
+
+    def pullback_wanted(self, inputs, output, goutput, wanted):
+        """pullback, told which inputs' gradients will be used.  Nodes are
+        evaluated as they are built, so an op whose gradient expressions are
+        separate kernels overrides this to launch only the wanted ones."""
+        return self.pullback(inputs, output, goutput)
 
     def get_native_compile_info(self, input_types, devtype):
         """Returns NativeCompileInfo."""
@@ -337,12 +392,16 @@ def unpack(node):
 
 # ================================================================ autodiff
 
-def grad(output, wrt, goutput):
+def grad(output, wrt, goutput=None):
     """Gradients of <output, goutput> with respect to the nodes in `wrt`, by
     walking back through each op's pullback (the reference's `grad`,
-    core.py:633-728, takes a scalar cost; here the cotangent of `output` is
-    given explicitly because the elementwise/reduction ops that would build a
-    scalar cost are outside the hot path)."""
+    core.py:633-728).  With `goutput` omitted, `output` must be a scalar cost,
+    as in the reference, and its cotangent is 1."""
+    if goutput is None:
+        output = as_node(output)
+        if output.value.size != 1:
+            raise ValueError("grad of a non-scalar needs its cotangent (goutput=...)")
+        goutput = fill(1.0, shape(output))
     order, seen = [], set()
 
     def visit(n):
@@ -354,9 +413,18 @@ def grad(output, wrt, goutput):
         order.append(n)
 
     visit(output)
+    # nodes whose value depends differentiably on a `wrt` node: only they need a
+    # gradient (the reference's differentiably_influenced_by, core.py:620-631)
+    active = set(id(w) for w in wrt)
+    for node in order:
+        if node.op is None:
+            continue
+        diff = [True] * len(node.parents) if isinstance(node.op, TupleIndex) else node.op.get_diff(len(node.parents))
+        if any(d and id(p) in active for p, d in zip(node.parents, diff)):
+            active.add(id(node))
     gmap = {id(output): as_node(goutput)}
     for node in reversed(order):
-        if node.op is None:
+        if node.op is None or id(node) not in active:
             continue
         if isinstance(node.op, TupleIndex):
             # route the member's gradient to the producing tuple node
@@ -369,17 +437,18 @@ def grad(output, wrt, goutput):
         g = gmap.get(id(node))
         if g is None:
             continue
-        gins = node.op.pullback(node.parents, node, g)
-        for p, gp, d in zip(node.parents, gins, node.op.get_diff(len(node.parents))):
-            if gp is None or not d:
+        wanted = [bool(d) and id(p) in active for p, d in zip(node.parents, node.op.get_diff(len(node.parents)))]
+        gins = node.op.pullback_wanted(node.parents, node, g, wanted)
+        for p, gp, w in zip(node.parents, gins, wanted):
+            if gp is None or not w:
                 continue
             gmap[id(p)] = gp if id(p) not in gmap else add(gmap[id(p)], gp)
     return [gmap.get(id(w)) for w in wrt]
 
 
 def add(a, b):
-    raise MethodNotDefined("a node feeding several consumers needs the elementwise add op, "
-                           "which is outside the CNN hot path")
+    """Sum of the gradients reaching a node that feeds several consumers."""
+    return elwise_binary("+", a, b)
 
 
 # ================================================================ ops
@@ -594,3 +663,425 @@ def dot(a, b):
 
 def batched_matmul(a, b):
     return Result(BatchedMul22(False, False), [a, b])
+
+
+# ================================================================ conv-layer glue ops
+#
+# The ops either side of conv2d in a training step -- bias add, ReLU, the
+# scalar loss, the bias gradient -- as the reference spells them: ElwiseUnary /
+# ElwiseBinary over expression tables, Repeat for broadcasting, Sum for
+# reductions, Fill for constants.  One compiled closure per op class; the op
+# code travels in the closure struct and the closure calls the HIP library.
+
+UnaryInfo = namedtuple("UnaryInfo", ("short", "diff", "gradexpr"))
+
+# reference UNARY_INFO (core.py:1118-1134), the float -> float entries
+UNARY_INFO = {
+    "abs": UnaryInfo("abs", True, lambda x, y, gy: gy * sign(x)),
+    "cos": UnaryInfo("cos", True, lambda x, y, gy: -gy * sin(x)),
+    "exp": UnaryInfo("exp", True, lambda x, y, gy: gy * exp(x)),
+    "log": UnaryInfo("log", True, lambda x, y, gy: gy / x),
+    "neg": UnaryInfo("negative", True, lambda x, y, gy: -gy),
+    "sign": UnaryInfo("sign", False, None),
+    "sin": UnaryInfo("sin", True, lambda x, y, gy: gy * cos(x)),
+    "square": UnaryInfo("square", True, lambda x, y, gy: 2.0 * gy * x),
+    "sqrt": UnaryInfo("sqrt", True, lambda x, y, gy: gy / (2.0 * y)),
+    "tanh": UnaryInfo("tanh", True, lambda x, y, gy: gy * (1 - square(y))),
+    "sigmoid": UnaryInfo("sigmoid", True, lambda x, y, gy: gy * y * (1 - y)),
+}
+UNARY_CODES = ["abs", "cos", "exp", "log", "neg", "sign", "sin", "square", "sqrt", "tanh", "sigmoid"]
+
+BinaryInfo = namedtuple("BinaryInfo", ("short", "diff", "typeinfo", "gradexpr"))
+
+# reference BINARY_INFO (core.py:1139-1152)
+BINARY_INFO = {
+    "*": BinaryInfo("multiply", (True, True), "p", lambda x, y, z, gz: [y * gz, x * gz]),
+    "+": BinaryInfo("add", (True, True), "p", lambda x, y, z, gz: [gz, gz]),
+    "-": BinaryInfo("subtract", (True, True), "p", lambda x, y, z, gz: [gz, -gz]),
+    "/": BinaryInfo("divide", (True, True), "f", lambda x, y, z, gz: [gz / y, -gz * z / y]),
+    "<": BinaryInfo("less", (False, False), "i1", None),
+    ">": BinaryInfo("greater", (False, False), "i1", None),
+    "<=": BinaryInfo("less_equal", (False, False), "i1", None),
+    ">=": BinaryInfo("greater_equal", (False, False), "i1", None),
+    "**": BinaryInfo("power", (True, True), "p", lambda x, y, z, gz: [gz * y * power(x, y - 1), gz * z * log(x)]),
+    "==": BinaryInfo("equal", (False, False), "i1", None),
+    "!=": BinaryInfo("not_equal", (False, False), "i1", None),
+}
+BINARY_CODES = ["*", "+", "-", "/", "<", ">", "<=", ">=", "**", "==", "!="]
+
+
+class ElwiseUnary(Op):
+    """Elementwise unary operation (reference core.py:1160-1241)."""
+    available_impls = ("native_gpu",)
+
+    def __init__(self, opname):
+        self.opname = opname
+        self.info = UNARY_INFO[opname]
+
+    def get_diff(self, _):
+        return [self.info.diff]
+
+    def __repr__(self):
+        return self.info.short
+
+    def pullback(self, inputs, y, gy):
+        return [self.info.gradexpr(inputs[0], y, gy)]
+
+    def shp_apply(self, inputs):
+        return shape(inputs[0])
+
+    def typ_apply(self, input_types):
+        assert input_types[0].dtype == "f4", "unary ops take float32 here"
+        return TensorType(floatX, input_types[0].ndim)
+
+    def get_closure(self):
+        return [("op", ctypes.c_int, UNARY_CODES.index(self.opname))]
+
+    def get_native_compile_info(self, input_types, devtype):
+        assert devtype == "gpu"
+        code = r"""
+            CGT_EXPORT_C void $function($closure* cl, cgtArray** reads, cgtArray* write) {
+                cgtArray* read = reads[0];
+                int rc = cgt_amd_elwise_unary_f32(cl->op, read->size(), (const float*)read->data(),
+                    (float*)write->data(), cgt_get_stream());
+                cgt_check(rc == CGT_AMD_OK, "ElwiseUnary: %s", cgt_amd_last_error());
+            }"""
+        return NativeCompileInfo(code, includes=["cgt_amd.h"], closure_triples=self.get_closure(),
+                                 gpu_deref_mask=(True,))
+
+
+def _promote(d0, d1):
+    return "f4" if "f4" in (d0, d1) else "i1"
+
+
+class ElwiseBinary(Op):
+    """Elementwise binary operation; scalar_mask says which operand is a 0-d
+    array (reference core.py:1243-1378)."""
+    available_impls = ("native_gpu",)
+
+    def __init__(self, opname, scalar_mask):
+        assert opname in BINARY_INFO
+        self.opname = opname
+        self.info = BINARY_INFO[opname]
+        self.scalar_mask = tuple(bool(m) for m in scalar_mask)
+
+    def get_diff(self, _):
+        return list(self.info.diff)
+
+    def __repr__(self):
+        return self.info.short
+
+    def pullback(self, inputs, z, gz):
+        return self.pullback_wanted(inputs, z, gz, [True, True])
+
+    def pullback_wanted(self, inputs, z, gz, wanted):
+        x, y = inputs
+        # the table's expressions, one operand at a time so that only the wanted one runs
+        exprs = {
+            "*": (lambda: y * gz, lambda: x * gz),
+            "+": (lambda: gz, lambda: gz),
+            "-": (lambda: gz, lambda: -gz),
+            "/": (lambda: gz / y, lambda: -gz * z / y),
+            "**": (lambda: gz * y * power(x, y - 1), lambda: gz * z * log(x)),
+        }[self.opname]
+        gin = [e() if w else None for e, w in zip(exprs, wanted)]
+        return [None if gv is None else (sum(gv) if (v.ndim == 0 and gv.ndim > 0) else gv)
+                for v, gv in zip([x, y], gin)]
+
+    def shp_apply(self, inputs):
+        ind4shape = 1 if self.scalar_mask[0] else 0
+        if self.scalar_mask == (False, False) and shape(inputs[0]) != shape(inputs[1]):
+            raise ValueError("mismatched shapes %s %s. Note that implicit broadcasting isn't allowed. "
+                             "Use the broadcast(...) function" % (shape(inputs[0]), shape(inputs[1])))
+        return shape(inputs[ind4shape])
+
+    def typ_apply(self, input_types):
+        assert ((input_types[0].ndim == 0) == self.scalar_mask[0]) and ((input_types[1].ndim == 0) == self.scalar_mask[1])
+        if self.scalar_mask == (False, False):
+            assert input_types[0].ndim == input_types[1].ndim
+        for t in input_types:
+            assert t.dtype in ("f4", "i1"), "elementwise ops take f4 / i1 arrays here, got %s" % t.dtype
+        typeinfo = self.info.typeinfo
+        if typeinfo == "p":
+            out_dtype = _promote(input_types[0].dtype, input_types[1].dtype)
+        elif typeinfo == "f":
+            out_dtype = floatX
+        else:
+            out_dtype = typeinfo
+        ind4shape = 1 if self.scalar_mask[0] else 0
+        return TensorType(out_dtype, input_types[ind4shape].ndim)
+
+    def get_closure(self):
+        return [("op", ctypes.c_int, BINARY_CODES.index(self.opname)),
+                ("scalar0", ctypes.c_int, int(self.scalar_mask[0])),
+                ("scalar1", ctypes.c_int, int(self.scalar_mask[1]))]
+
+    def get_native_compile_info(self, input_types, devtype):
+        assert devtype == "gpu"
+        code = r"""
+            CGT_EXPORT_C void $function($closure* cl, cgtArray** reads, cgtArray* write) {
+                long n = reads[cl->scalar0 ? 1 : 0]->size();
+                cgt_check(write->size() == n, "Shape error in elementwise binary operation. You might be missing a call to cgt.broadcast(...)");
+                int rc = cgt_amd_elwise_binary(cl->op, (int)reads[0]->dtype(), (int)reads[1]->dtype(), n,
+                    reads[0]->data(), cl->scalar0, reads[1]->data(), cl->scalar1, write->data(), cgt_get_stream());
+                cgt_check(rc == CGT_AMD_OK, "ElwiseBinary: %s", cgt_amd_last_error());
+            }"""
+        return NativeCompileInfo(code, includes=["cgt_amd.h"], closure_triples=self.get_closure(),
+                                 gpu_deref_mask=(True, True))
+
+
+def _scalar_operand(v, like):
+    """python numbers become 0-d device arrays of the other operand's float type."""
+    if isinstance(v, Node):
+        return v
+    if isinstance(v, (int, float, np.integer, np.floating)) or (isinstance(v, np.ndarray) and v.ndim == 0):
+        return constant(np.float32(v))
+    return as_node(v)
+
+
+def elwise_binary(opname, x, y):
+    """reference core.py:1380-1386"""
+    x, y = _scalar_operand(x, y), _scalar_operand(y, x)
+    scalar_mask = ((x.ndim == 0), (y.ndim == 0))
+    if scalar_mask == (False, False):
+        assert x.ndim == y.ndim
+    return Result(ElwiseBinary(opname, scalar_mask), [x, y])
+
+
+class Repeat(Op):
+    """Blow up singleton axes: inputs (x, count per axis in `axes`), counts are
+    host integers (reference core.py:1511-1557, cpu-only there)."""
+    available_impls = ("native_gpu",)
+
+    def __init__(self, axes):
+        self.axes = tuple(int(a) for a in axes)
+
+    def get_diff(self, num_inputs):
+        return [True] + [False] * (num_inputs - 1)
+
+    def __repr__(self):
+        return "Repeat{%s}" % ",".join(map(str, self.axes))
+
+    def pullback(self, inputs, output, goutput):
+        return [sum(goutput, self.axes, keepdims=True)] + [None] * (len(inputs) - 1)
+
+    def shp_apply(self, inputs):
+        out = shape(inputs[0])
+        for ax, rep in zip(self.axes, inputs[1:]):
+            if out[ax] != 1:
+                raise ValueError("Repeat: axis %d has extent %d, not 1" % (ax, out[ax]))
+            out[ax] = int(np.asarray(as_node(rep).value))
+        return out
+
+    def typ_apply(self, input_types):
+        assert all(t.dtype == "i8" for t in input_types[1:])
+        assert input_types[0].ndim <= 8
+        return input_types[0]
+
+    def get_closure(self):
+        mask = 0
+        for a in self.axes:
+            mask |= 1 << a
+        return [("axes_mask", ctypes.c_int, mask)]
+
+    def get_native_compile_info(self, input_types, devtype):
+        assert devtype == "gpu"
+        code = r"""
+            CGT_EXPORT_C void $function($closure* cl, cgtArray** reads, cgtArray* write) {
+                cgtArray* read = reads[0];
+                int nd = read->ndim();
+                long oshape[8];
+                int rep[8];
+                for (int a = 0; a < nd; ++a) {
+                    oshape[a] = write->shape()[a];
+                    rep[a] = (cl->axes_mask >> a) & 1;
+                    cgt_check(!rep[a] || read->shape()[a] == 1, "Repeat: a repeated axis must have extent 1");
+                }
+                int rc = cgt_amd_repeat(read->data(), cgt_itemsize(read->dtype()), nd, oshape, rep,
+                    write->data(), cgt_get_stream());
+                cgt_check(rc == CGT_AMD_OK, "Repeat: %s", cgt_amd_last_error());
+            }"""
+        return NativeCompileInfo(code, includes=["cgt_amd.h"], closure_triples=self.get_closure(),
+                                 gpu_deref_mask=(True,) + (False,) * (len(input_types) - 1))
+
+
+class Sum(Op):
+    """Sum over `axes`, keeping them with extent 1 (reference core.py:1687-1709,
+    cpu-only there)."""
+    available_impls = ("native_gpu",)
+
+    def __init__(self, axes):
+        self.axes = tuple(int(a) for a in axes)
+
+    def get_diff(self, _):
+        return [True]
+
+    def __repr__(self):
+        return "Sum{%s}" % ",".join(map(str, self.axes))
+
+    def pullback(self, inputs, output, goutput):
+        return [Result(Repeat(self.axes), [goutput] + [size(inputs[0], ax) for ax in self.axes])]
+
+    def shp_apply(self, inputs):
+        s = shape(inputs[0])
+        return [1 if i in self.axes else s[i] for i in range(len(s))]
+
+    def typ_apply(self, input_types):
+        assert input_types[0].dtype == "f4" and input_types[0].ndim <= 8
+        return input_types[0]
+
+    def get_closure(self):
+        mask = 0
+        for a in self.axes:
+            mask |= 1 << a
+        return [("axes_mask", ctypes.c_int, mask)]
+
+    def get_native_compile_info(self, input_types, devtype):
+        assert devtype == "gpu"
+        code = r"""
+            CGT_EXPORT_C void $function($closure* cl, cgtArray** reads, cgtArray* write) {
+                cgtArray* read = reads[0];
+                int nd = read->ndim();
+                int red[8];
+                for (int a = 0; a < nd; ++a) red[a] = (cl->axes_mask >> a) & 1;
+                int rc = cgt_amd_sum_f32((const float*)read->data(), nd, read->shape(), red,
+                    (float*)write->data(), cgt_get_stream());
+                cgt_check(rc == CGT_AMD_OK, "Sum: %s", cgt_amd_last_error());
+            }"""
+        return NativeCompileInfo(code, includes=["cgt_amd.h"], closure_triples=self.get_closure(),
+                                 gpu_deref_mask=(True,))
+
+
+class Fill(Op):
+    """(shape...) -> float32 array filled with `value` (reference core.py:966-1007,
+    cpu-only there)."""
+    available_impls = ("native_gpu",)
+
+    def __init__(self, value):
+        self.value = float(value)
+
+    def get_diff(self, num_inputs):
+        return [False] * num_inputs
+
+    def __repr__(self):
+        return "Fill{%g}" % self.value
+
+    def pullback(self, inputs, output, goutput):
+        raise MethodNotDefined("Fill is not differentiable")
+
+    def shp_apply(self, inputs):
+        return [int(np.asarray(as_node(i).value)) for i in inputs]
+
+    def typ_apply(self, input_types):
+        assert all(t.dtype == "i8" and t.ndim == 0 for t in input_types), \
+            "Fill Op should have integer scalars as arguments"
+        return TensorType(floatX, len(input_types))
+
+    def get_closure(self):
+        return [("value", ctypes.c_double, self.value)]
+
+    def get_native_compile_info(self, input_types, devtype):
+        assert devtype == "gpu"
+        code = r"""
+            CGT_EXPORT_C void $function($closure* cl, cgtArray** reads, cgtArray* write) {
+                int rc = cgt_amd_fill_f32((float*)write->data(), (float)cl->value, write->size(), cgt_get_stream());
+                cgt_check(rc == CGT_AMD_OK, "Fill: %s", cgt_amd_last_error());
+            }"""
+        return NativeCompileInfo(code, includes=["cgt_amd.h"], closure_triples=self.get_closure(),
+                                 gpu_deref_mask=(False,) * len(input_types))
+
+
+# ---------------------------------------------------------------- functions over the glue ops (reference cgt/api.py)
+
+def _unary(opname):
+    def f(x):
+        return Result(ElwiseUnary(opname), [x])
+    f.__name__ = opname
+    f.__doc__ = "elementwise %s (reference cgt/api_autogen.py)" % opname
+    return f
+
+
+abs = _unary("abs")            # noqa: A001  (the reference exports these names)
+cos = _unary("cos")
+exp = _unary("exp")
+log = _unary("log")
+neg = _unary("neg")
+sign = _unary("sign")
+sin = _unary("sin")
+square = _unary("square")
+sqrt = _unary("sqrt")
+tanh = _unary("tanh")
+sigmoid = _unary("sigmoid")
+
+
+def power(x, y):
+    return elwise_binary("**", x, y)
+
+
+def greater_equal(x, y):
+    return elwise_binary(">=", x, y)
+
+
+def broadcast(opname, a, b, bcpat):
+    """Elementwise binary op with singleton axes expanded first; bcpat names
+    them, e.g. "xxxx,1x11" for activation + bias (reference cgt/api.py:92-120)."""
+    x, y = as_node(a), as_node(b)
+    xpat, ypat = bcpat.split(",")
+    xbcaxes, ybcaxes = [[i for i, letter in enumerate(pat) if letter == "1"] for pat in (xpat, ypat)]
+    assert x.ndim == y.ndim
+    if xbcaxes:
+        x = Result(Repeat(xbcaxes), [x] + [size(y, ax) for ax in xbcaxes])
+    if ybcaxes:
+        y = Result(Repeat(ybcaxes), [y] + [size(x, ax) for ax in ybcaxes])
+    return elwise_binary(opname, x, y)
+
+
+def _red_axes(axis, ndim):
+    if axis is None:
+        return list(range(ndim))
+    if isinstance(axis, int):
+        return [axis]
+    return list(axis)
+
+
+def sum(x, axis=None, keepdims=False):      # noqa: A001
+    """Like numpy.sum (reference cgt/api.py:647-659)."""
+    x = as_node(x)
+    axes = _red_axes(axis, x.ndim)
+    if len(axes) == 0:
+        return x
+    out = Result(Sum(axes), [x])
+    if not keepdims:
+        out = reshape(out, [size(x, i) for i in range(x.ndim) if i not in axes])
+    return out
+
+
+def mean(x, axis=None, keepdims=False):
+    """Like numpy.mean (reference cgt/api.py:470-476)."""
+    x = as_node(x)
+    axes = _red_axes(axis, x.ndim)
+    n = 1
+    for ax in axes:
+        n *= size(x, ax)
+    return sum(x, axis=axes, keepdims=keepdims) / float(n)
+
+
+def fill(val, shp):
+    """Array of shape `shp` filled with the scalar `val` (reference cgt/api.py:246-258)."""
+    return Result(Fill(val), [int(s) for s in shp])
+
+
+def zeros(shp):
+    return fill(0.0, shp)
+
+
+def ones(shp):
+    return fill(1.0, shp)
+
+
+def zeros_like(x):
+    return zeros(shape(x))
+
+
+def ones_like(x):
+    return ones(shape(x))

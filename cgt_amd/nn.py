@@ -23,6 +23,36 @@ def conv2d(x_BKRC, f_LKrc, kernelshape, pad=(0, 0), stride=(1, 1)):
     return col_Bmn_L.reshape([B, m, n, L]).transpose([0, 3, 1, 2])
 
 
+def rectify(x):
+    """ReLU as the reference builds it: x * (x >= 0) (cgt/nn.py:44-45)."""
+    x = core.as_node(x)
+    return x * (x >= 0)
+
+
+class SpatialConvolution(object):
+    """conv2d plus a per-channel bias [1, L, 1, 1] (reference cgt/nn.py:216-233).
+    Weights and bias are device-resident leaf nodes."""
+
+    def __init__(self, input_channels, output_channels, kernelshape, pad, stride=(1, 1), name=None,
+                 weight_init=None, bias_init=None):
+        import numpy as np
+        input_channels, output_channels = int(input_channels), int(output_channels)
+        self.kernelshape = tuple(map(int, kernelshape))
+        self.pad = tuple(map(int, pad))
+        self.stride = tuple(map(int, stride))
+        self.name = "unnamed" if name is None else name
+        wshape = (output_channels, input_channels) + self.kernelshape
+        w = np.zeros(wshape, np.float32) if weight_init is None else np.asarray(weight_init, np.float32).reshape(wshape)
+        b = np.zeros((1, output_channels, 1, 1), np.float32) if bias_init is None else \
+            np.asarray(bias_init, np.float32).reshape(1, output_channels, 1, 1)
+        self.weight = core.constant(w)
+        self.bias = core.constant(b)
+
+    def __call__(self, x):
+        tmp = conv2d(x, self.weight, self.kernelshape, self.pad, self.stride)
+        return core.broadcast("+", tmp, self.bias, "xxxx,1x11")
+
+
 def max_pool_2d(x, kernelshape, pad=(0, 0), stride=(1, 1)):
     kernel_h, kernel_w = kernelshape
     pad_h, pad_w = pad

@@ -228,7 +228,7 @@ def from_cgt_handle(h, owner=None):
     ndim = L.cgt_rt_array_ndim(h)
     shp = L.cgt_rt_array_shape(h)
     shape = tuple(shp[i] for i in range(ndim))
-    dtype = {11: np.float32, 5: np.int32, 7: np.int64, 12: np.float64}[L.cgt_rt_array_dtype(h)]
+    dtype = {11: np.float32, 5: np.int32, 7: np.int64, 12: np.float64, 1: np.int8}[L.cgt_rt_array_dtype(h)]
     data = L.cgt_rt_array_data(h)
     nbytes = L.cgt_rt_array_nbytes(h)
     if L.cgt_rt_array_devtype(h) == GPU:

@@ -98,7 +98,7 @@ def test_closure_struct_layouts():
 
 def test_prebuild_standard_ops_exports_call_symbols():
     built = compilation.prebuild_standard_ops()
-    assert len(built) == 9
+    assert len(built) == 14
     for c in built:
         assert c.fptr_address and c.return_type == "byref" and c.kind == "native"
     cache = compilation.get_compile_info()["CACHE_ROOT"]
@@ -217,3 +217,43 @@ def test_interpreter_alloc_reuse_and_byref():
     assert np.array_equal(it.get_array(6)[0], x + 1 + y + 7)
     with pytest.raises(ValueError):
         it.alloc(np.int64, [], (99, cpu))
+
+
+# ---------------------------------------------------------------- conv-layer glue ops (host logic only)
+
+def test_elwise_binary_type_rules():
+    # reference core.py:1319-1333: 'p' promotes, 'f' gives floatX, comparisons give i1;
+    # the output takes the rank of the non-scalar operand
+    F4, B4, F0 = core.TensorType("f4", 4), core.TensorType("i1", 4), core.TensorType("f4", 0)
+    assert core.ElwiseBinary("*", (False, False)).typ_apply([F4, B4]) == F4
+    assert core.ElwiseBinary("*", (False, False)).typ_apply([B4, B4]) == B4
+    assert core.ElwiseBinary("/", (False, False)).typ_apply([B4, B4]) == F4
+    assert core.ElwiseBinary(">=", (False, True)).typ_apply([F4, F0]) == B4
+    assert core.ElwiseBinary("+", (True, False)).typ_apply([F0, F4]) == F4
+    with pytest.raises(AssertionError):
+        core.ElwiseBinary("+", (False, False)).typ_apply([F4, F0])       # mask must match the ranks
+    assert core.ElwiseBinary("<", (False, False)).get_diff(2) == [False, False]
+    assert core.ElwiseBinary("-", (False, False)).get_diff(2) == [True, True]
+
+
+def test_glue_closures_and_hashes():
+    # one compiled library per op class: the op code / axes / value travel in the closure
+    a, b = core.ElwiseBinary("+", (False, False)), core.ElwiseBinary("*", (False, True))
+    assert a.get_hash() != b.get_hash()
+    ca = a.get_native_compile_info([core.TensorType("f4", 2)] * 2, "gpu")
+    cb = b.get_native_compile_info([core.TensorType("f4", 2), core.TensorType("f4", 0)], "gpu")
+    assert ca.func_code == cb.func_code and ca.gpu_deref_mask == (True, True)
+    assert [t[2] for t in b.get_closure()] == [core.BINARY_CODES.index("*"), 0, 1]
+    assert core.Repeat((0, 2, 3)).get_closure()[0][2] == 0b1101
+    assert core.Sum((1,)).get_closure()[0][2] == 0b10
+    S = core.TensorType("i8", 0)
+    nci = core.Repeat((0, 2, 3)).get_native_compile_info([core.TensorType("f4", 4), S, S, S], "gpu")
+    assert nci.gpu_deref_mask == (True, False, False, False)        # repeat counts stay on the host
+    assert core.Fill(2.0).typ_apply([S, S, S]) == core.TensorType("f4", 3)
+    assert core.ElwiseUnary("sign").get_diff(1) == [False] and core.ElwiseUnary("tanh").get_diff(1) == [True]
+    # op codes agree with the C header
+    hdr = open(os.path.join(os.path.dirname(__file__), "..", "include", "cgt_amd.h")).read()
+    for i, name in enumerate(["MUL", "ADD", "SUB", "DIV", "LT", "GT", "LE", "GE", "POW", "EQ", "NE"]):
+        assert "#define CGT_AMD_BIN_%s %d\n" % (name, i) in hdr
+    for i, name in enumerate(["ABS", "COS", "EXP", "LOG", "NEG", "SIGN", "SIN", "SQUARE", "SQRT", "TANH", "SIGMOID"]):
+        assert "#define CGT_AMD_UN_%s %d\n" % (name, i) in hdr

@@ -314,7 +314,14 @@ def cpu_baseline(cfg, sample_batch):
 
     best, reps = CB.timed(run, min_seconds=8.0, max_reps=20)
     flops = 6 * sample_batch * m * n * L * C * r * c
-    return {"value": flops / best / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+    # the same stages one by one (GB/s for the single-threaded C loops, TFLOP/s for OpenBLAS)
+    per_stage = {}
+    for name, (sec, work) in CB.stage_times(x, f, gy, pad, stride, cfg["pool"], cfg["lrn"]).items():
+        if name.startswith("gemm"):
+            per_stage[name] = {"ms": round(sec * 1e3, 3), "TFLOPs": round(work / sec / 1e12, 4)}
+        else:
+            per_stage[name] = {"ms": round(sec * 1e3, 3), "GBps": round(work / sec / 1e9, 3)}
+    return {"value": flops / best / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port", "stages": per_stage,
             "sample": "%d of %d images of the workload, best of %d passes (%.2f s each); im2col/col2im/"
                       "transpose/pool/LRN single-threaded C, GEMM %s with %d threads; host %s, %d cores usable"
                       % (sample_batch, cfg["x"][0], reps, best, CB.blas_config(), threads, CB.cpu_model(), CB.host_cores())}

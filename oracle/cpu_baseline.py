@@ -99,3 +99,44 @@ def timed(fn, min_seconds=2.0, max_reps=50):
         total += dt
         reps += 1
     return best, reps
+
+
+def stage_times(x, f, gy, pad, stride, pool=None, lrn=None, min_seconds=0.5):
+    """Best-of wall time of each CPU stage of the layer on the sample, in the
+    order the reference's graph runs them: {stage: (seconds, bytes or flops)}."""
+    L, K, r, c = f.shape
+    out = {}
+    col = O.im2col(x, (r, c), pad, stride)
+    B, m, n, Z = col.shape
+    col2, f_LZ = col.reshape(B * m * n, Z), f.reshape(L, Z)
+    io = 4 * (x.size + col.size)
+    flops = 2 * B * m * n * L * Z
+    out["im2col"] = (timed(lambda: O.im2col(x, (r, c), pad, stride), min_seconds, 5)[0], io)
+    out["gemm_fwd_NT"] = (timed(lambda: sgemm(col2, f_LZ, False, True), min_seconds, 5)[0], flops)
+    y2 = sgemm(col2, f_LZ, False, True).reshape(B, m, n, L)
+    out["transpose_0312"] = (timed(lambda: O.transpose4(y2, (0, 3, 1, 2)), min_seconds, 5)[0], 8 * y2.size)
+    y = O.transpose4(y2, (0, 3, 1, 2))
+    act = y
+    if lrn:
+        size, alpha, beta, k = lrn
+        out["lrn_fwd"] = (timed(lambda: O.lrn_fwd(y, size, alpha, beta, k), min_seconds, 5)[0], 12 * y.size)
+        act, scale = O.lrn_fwd(y, size, alpha, beta, k)
+    g = gy
+    if pool:
+        pk, pp, ps = pool
+        out["max_pool_fwd"] = (timed(lambda: O.max_pool(act, pk, pp, ps), min_seconds, 5)[0], None)
+        pooled, mask = O.max_pool(act, pk, pp, ps)
+        out["max_pool_fwd"] = (out["max_pool_fwd"][0], 4 * (act.size + 2 * pooled.size))
+        gp = np.ones_like(pooled)
+        out["max_pool_bwd"] = (timed(lambda: O.max_pool_pullback(act.shape, mask, gp), min_seconds, 5)[0],
+                               4 * (2 * pooled.size + act.size))
+        g = O.max_pool_pullback(act.shape, mask, gp)
+    if lrn:
+        out["lrn_bwd"] = (timed(lambda: O.lrn_bwd(y, act, scale, g, size, alpha, beta), min_seconds, 5)[0], 20 * y.size)
+    out["transpose_0231"] = (timed(lambda: O.transpose4(g, (0, 2, 3, 1)), min_seconds, 5)[0], 8 * y.size)
+    gc = O.transpose4(g, (0, 2, 3, 1)).reshape(B * m * n, L)
+    out["gemm_dgrad_NN"] = (timed(lambda: sgemm(gc, f_LZ, False, False), min_seconds, 5)[0], flops)
+    gcol = sgemm(gc, f_LZ, False, False).reshape(B, m, n, Z)
+    out["col2im"] = (timed(lambda: O.col2im(gcol, x.shape, (r, c), pad, stride), min_seconds, 5)[0], io)
+    out["gemm_wgrad_TN"] = (timed(lambda: sgemm(gc, col2, True, False), min_seconds, 5)[0], flops)
+    return out

@@ -1,0 +1,96 @@
+"""Edge behaviour of the C ABI itself, called with raw pointers as a foreign
+host would: empty inputs are accepted and touch nothing, bad arguments come
+back as CGT_AMD_ERR_ARG with a message (the reference's kernels print and carry
+on, include/cgt_cuda.h:11-21; here nothing is launched), and the library stays
+usable after an error."""
+import ctypes
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+OK, ERR_ARG = 0, 1
+
+
+@pytest.fixture(scope="module")
+def L():
+    from cgt_amd import capi
+    capi.require_gpu()
+    return capi.lib()
+
+
+def gpu(a):
+    from cgt_amd.gpuarray import to_gpu
+    return to_gpu(a)
+
+
+def _err(L):
+    return L.cgt_amd_last_error().decode()
+
+
+def test_empty_inputs_are_ok(L):
+    x = gpu(np.zeros((4,), np.float32))
+    p = x.ptr
+    assert L.cgt_amd_im2col_f32(p, 0, 3, 8, 8, 3, 3, 1, 1, 1, 1, p, None) == OK
+    assert L.cgt_amd_col2im_f32(p, 0, 3, 8, 8, 3, 3, 1, 1, 1, 1, p, None) == OK
+    assert L.cgt_amd_max_pool_f32(p, 0, 3, 8, 8, 2, 2, 0, 0, 2, 2, 3, 3, p, p, None) == OK
+    assert L.cgt_amd_lrn_fwd_f32(p, 0, 8, 4, 4, 5, 1e-4, 0.75, 1.0, p, p, None) == OK
+    assert L.cgt_amd_sgemm(0, 0, 0, 5, 7, p, 7, p, 5, p, 5, None) == OK
+    assert L.cgt_amd_sgemm_batched(0, 0, 0, 4, 4, 4, p, 4, 16, p, 4, 16, p, 4, 16, None) == OK
+    assert L.cgt_amd_elwise_unary_f32(0, 0, p, p, None) == OK
+    assert L.cgt_amd_elwise_binary(1, 11, 11, 0, p, 0, p, 0, p, None) == OK
+    assert L.cgt_amd_fill_f32(p, 1.0, 0, None) == OK
+    assert np.array_equal(x.get(), np.zeros(4, np.float32))
+
+
+def test_gemm_with_k_zero_writes_zeros(L):
+    # C = A[M,0] . B[0,N] is all zeros, and C must be overwritten, not skipped
+    c = gpu(np.full((5, 7), 3.0, np.float32))
+    a = gpu(np.zeros((1,), np.float32))
+    assert L.cgt_amd_sgemm(0, 0, 5, 7, 0, a.ptr, 0, a.ptr, 7, c.ptr, 7, None) == OK
+    assert np.array_equal(c.get(), np.zeros((5, 7), np.float32))
+
+
+@pytest.mark.parametrize("call,needle", [
+    (lambda L, p: L.cgt_amd_im2col_f32(p, 1, 1, 2, 2, 5, 5, 0, 0, 1, 1, p, None), "kernel larger"),
+    (lambda L, p: L.cgt_amd_im2col_f32(p, 1, 1, 8, 8, 3, 3, 0, 0, 0, 1, p, None), "geometry"),
+    (lambda L, p: L.cgt_amd_im2col_f32(None, 1, 1, 8, 8, 3, 3, 0, 0, 1, 1, p, None), "null"),
+    (lambda L, p: L.cgt_amd_col2im_f32(p, 1, -1, 8, 8, 3, 3, 0, 0, 1, 1, p, None), "negative"),
+    (lambda L, p: L.cgt_amd_max_pool_f32(p, 1, 1, 8, 8, 2, 2, 0, 0, 2, 2, 9, 4, p, p, None), "does not fit"),
+    (lambda L, p: L.cgt_amd_max_pool_pullback_f32(p, p, 1, 1, 8, 8, 2, 2, 0, 0, -2, 2, 4, 4, p, None), "geometry"),
+    (lambda L, p: L.cgt_amd_lrn_fwd_f32(p, 1, 3, 4, 4, 5, 1e-4, 0.75, 1.0, p, p, None), "size"),
+    (lambda L, p: L.cgt_amd_lrn_fwd_f32(p, 1, 8, 4, 4, 5, 1e-4, 0.75, 0.0, p, p, None), "k must be positive"),
+    (lambda L, p: L.cgt_amd_lrn_bwd_f32(p, p, p, p, 1, 8, 4, 4, 0, 1e-4, 0.75, p, None), "size"),
+    (lambda L, p: L.cgt_amd_sgemm(0, 0, 4, 4, 4, p, 3, p, 4, p, 4, None), "leading dimension"),
+    (lambda L, p: L.cgt_amd_sgemm(0, 0, 4, 4, 4, p, 4, p, 4, None, 4, None), "null"),
+    (lambda L, p: L.cgt_amd_sgemm(0, 0, -1, 4, 4, p, 4, p, 4, p, 4, None), "negative"),
+    (lambda L, p: L.cgt_amd_transpose4_f32(p, (ctypes.c_long * 4)(1, 2, 3, 4), (ctypes.c_int * 4)(0, 1, 1, 3), p, None),
+     "permutation"),
+    (lambda L, p: L.cgt_amd_elwise_unary_f32(99, 4, p, p, None), "unknown op"),
+    (lambda L, p: L.cgt_amd_elwise_binary(99, 11, 11, 4, p, 0, p, 0, p, None), "unknown op"),
+    (lambda L, p: L.cgt_amd_elwise_binary(1, 7, 11, 4, p, 0, p, 0, p, None), "unsupported dtypes"),
+    (lambda L, p: L.cgt_amd_repeat(p, 2, 1, (ctypes.c_long * 1)(4), (ctypes.c_int * 1)(0), p, None), "itemsize"),
+    (lambda L, p: L.cgt_amd_repeat(p, 4, 9, (ctypes.c_long * 9)(*[1] * 9), (ctypes.c_int * 9)(*[0] * 9), p, None), "ndim"),
+    (lambda L, p: L.cgt_amd_sum_f32(p, 1, (ctypes.c_long * 1)(-4), (ctypes.c_int * 1)(1), p, None), "negative"),
+    (lambda L, p: L.cgt_amd_fill_u32(None, 0, 4, None), "null"),
+])
+def test_bad_arguments_are_reported_not_launched(L, call, needle):
+    buf = gpu(np.arange(256, dtype=np.float32))
+    rc = call(L, buf.ptr)
+    assert rc == ERR_ARG, _err(L)
+    assert needle in _err(L), _err(L)
+    # nothing was written and the library still works
+    assert np.array_equal(buf.get(), np.arange(256, dtype=np.float32))
+    assert L.cgt_amd_fill_f32(buf.ptr, 2.0, 256, None) == OK
+    assert np.array_equal(buf.get(), np.full(256, 2.0, np.float32))
+
+
+def test_pool_outsize_rule(L):
+    # ceil((H + 2p - k) / s), no "+1" (cgt/nn_ops/max_pool_2d.py:40-41)
+    assert L.cgt_amd_pool_outsize(28, 2, 0, 2) == 13
+    assert L.cgt_amd_pool_outsize(55, 3, 0, 2) == 26
+    assert L.cgt_amd_pool_outsize(56, 2, 0, 2) == 27
+    assert L.cgt_amd_pool_outsize(32, 3, 0, 2) == 15
+    assert L.cgt_amd_pool_outsize(2, 5, 0, 1) == 0
+    assert L.cgt_amd_pool_outsize(8, 2, 0, 0) == 0

@@ -38,6 +38,7 @@
 #include "common.h"
 #include <algorithm>
 #include <mutex>
+#include <type_traits>
 #include <unordered_map>
 
 namespace cgt_amd {
@@ -79,6 +80,9 @@ struct OperandTile {
     static constexpr int NV = (kPerThread + 3) / 4;
     float v[NV * 4];
 
+    // CHECK = false: the caller guarantees the whole tile slice is in range
+    // (interior tile, K range a multiple of KT) -- straight-line loads.
+    template <bool CHECK>
     __device__ __forceinline__ void load(const float* __restrict__ p, long ld, int r0, int R,
                                          int k0, int kend) {
         if (VEC) {
@@ -90,7 +94,7 @@ struct OperandTile {
                     if (KC) {
                         const int row = r0 + (idx >> 2), k = k0 + (idx & 3) * 4;
                         const float* src = p + (long)row * ld + k;
-                        if (row < R && k + 3 < kend) {
+                        if (!CHECK || (row < R && k + 3 < kend)) {
                             const float4 q = *reinterpret_cast<const float4*>(src);
                             t[0] = q.x; t[1] = q.y; t[2] = q.z; t[3] = q.w;
                         } else if (row < R) {
@@ -101,7 +105,7 @@ struct OperandTile {
                     } else {
                         const int k = k0 + idx / (ROWS / 4), row = r0 + (idx % (ROWS / 4)) * 4;
                         const float* src = p + (long)k * ld + row;
-                        if (k < kend && row + 3 < R) {
+                        if (!CHECK || (k < kend && row + 3 < R)) {
                             const float4 q = *reinterpret_cast<const float4*>(src);
                             t[0] = q.x; t[1] = q.y; t[2] = q.z; t[3] = q.w;
                         } else if (k < kend) {
@@ -122,10 +126,10 @@ struct OperandTile {
                 if (idx < kElems) {
                     if (KC) {
                         const int row = r0 + (idx >> 4), k = k0 + (idx & 15);
-                        if (row < R && k < kend) t = p[(long)row * ld + k];
+                        if (!CHECK || (row < R && k < kend)) t = p[(long)row * ld + k];
                     } else {
                         const int k = k0 + idx / ROWS, row = r0 + idx % ROWS;
-                        if (k < kend && row < R) t = p[(long)k * ld + row];
+                        if (!CHECK || (k < kend && row < R)) t = p[(long)k * ld + row];
                     }
                 }
                 v[i] = t;
@@ -179,7 +183,8 @@ __device__ __forceinline__ int xcd_remap(int id, int n) {
 }
 
 // WGM x WGN wavefronts, each TM x TN blocks of 32x32.
-template <bool AKC, bool BKC, bool VECA, bool VECB, int WGM, int WGN, int TM, int TN>
+// PIPE selects the software-pipelined main loop (k-contiguous operands only).
+template <bool AKC, bool BKC, bool VECA, bool VECB, bool PIPE, int WGM, int WGN, int TM, int TN>
 __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
     static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
@@ -274,74 +279,88 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
                                                                      acc[i][j], 0, 0, 0);
     };
     // wait for this wavefront's LDS traffic only, then workgroup barrier
-    auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    // (the scheduling fences keep the compiler from moving MFMAs across it: the
+    // barrier is meant to sit in the middle of the MFMA stream)
+    auto lds_barrier = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    };
 
     // The pipelined schedule pays off when both operands are k-contiguous
     // (16-byte fragment reads); the other layouts measure faster with the
     // plain double-buffered loop (one full barrier per slice).
-    constexpr bool kPipelined = AKC && BKC;
-    if constexpr (kPipelined) {
-        if (nk > 0) {
-            ta.load(A, a.lda, m0, a.M, kbeg, kend);
-            tb.load(B, a.ldb, n0, a.N, kbeg, kend);
-            ta.store(As[0]);
-            tb.store(Bs[0]);
-            if (nk > 1) {
-                ta.load(A, a.lda, m0, a.M, kbeg + KT, kend);
-                tb.load(B, a.ldb, n0, a.N, kbeg + KT, kend);
+    // Interior tiles (all of BM x BN inside C, K range a multiple of the slice)
+    // run a copy of the main loop with no bounds tests in its loads.
+    auto main_loop = [&](auto checked) {
+        constexpr bool CHK = decltype(checked)::value;
+        constexpr bool kPipelined = PIPE;
+        if constexpr (kPipelined) {
+            if (nk > 0) {
+                ta.template load<CHK>(A, a.lda, m0, a.M, kbeg, kend);
+                tb.template load<CHK>(B, a.ldb, n0, a.N, kbeg, kend);
+                ta.store(As[0]);
+                tb.store(Bs[0]);
+                if (nk > 1) {
+                    ta.template load<CHK>(A, a.lda, m0, a.M, kbeg + KT, kend);
+                    tb.template load<CHK>(B, a.ldb, n0, a.N, kbeg + KT, kend);
+                }
+                lds_barrier();
+                read_frags(0, As[0], Bs[0], 0);
             }
-            lds_barrier();
-            read_frags(0, As[0], Bs[0], 0);
-        }
-        for (int kt = 0; kt < nk; ++kt) {
-            const int cur = kt & 1;
-            if (kt + 1 < nk) {
-                ta.store(As[cur ^ 1]);       // slice kt+1 (waits for its global loads, issued an iteration ago)
-                tb.store(Bs[cur ^ 1]);
-            }
-            if (kt + 2 < nk) {
-                const int k0 = kbeg + (kt + 2) * KT;
-                ta.load(A, a.lda, m0, a.M, k0, kend);
-                tb.load(B, a.ldb, n0, a.N, k0, kend);
-            }
-            read_frags(1, As[cur], Bs[cur], 1);
-            __builtin_amdgcn_s_setprio(3);   // inside the MFMA stream: ahead of wavefronts issuing loads
-            mfma_steps(0, 0, 4);
-            lds_barrier();
-            if (kt + 1 < nk) read_frags(0, As[cur ^ 1], Bs[cur ^ 1], 0);
-            mfma_steps(1, 0, 4);
-            __builtin_amdgcn_s_setprio(0);
-        }
-    } else {
-        if (nk > 0) {
-            ta.load(A, a.lda, m0, a.M, kbeg, kend);
-            tb.load(B, a.ldb, n0, a.N, kbeg, kend);
-            ta.store(As[0]);
-            tb.store(Bs[0]);
-        }
-        __syncthreads();
-        for (int kt = 0; kt < nk; ++kt) {
-            const int cur = kt & 1;
-            const bool more = kt + 1 < nk;
-            if (more) {
-                const int k0 = kbeg + (kt + 1) * KT;
-                ta.load(A, a.lda, m0, a.M, k0, kend);
-                tb.load(B, a.ldb, n0, a.N, k0, kend);
-            }
-            __builtin_amdgcn_s_setprio(3);
-#pragma unroll
-            for (int kk = 0; kk < KT / 8; ++kk) {
-                read_frags(0, As[cur], Bs[cur], kk);
+            for (int kt = 0; kt < nk; ++kt) {
+                const int cur = kt & 1;
+                if (kt + 1 < nk) {
+                    ta.store(As[cur ^ 1]);       // slice kt+1 (waits for its global loads, issued an iteration ago)
+                    tb.store(Bs[cur ^ 1]);
+                }
+                if (kt + 2 < nk) {
+                    const int k0 = kbeg + (kt + 2) * KT;
+                    ta.template load<CHK>(A, a.lda, m0, a.M, k0, kend);
+                    tb.template load<CHK>(B, a.ldb, n0, a.N, k0, kend);
+                }
+                read_frags(1, As[cur], Bs[cur], 1);
+                __builtin_amdgcn_s_setprio(3);   // inside the MFMA stream: ahead of wavefronts issuing loads
                 mfma_steps(0, 0, 4);
+                lds_barrier();
+                if (kt + 1 < nk) read_frags(0, As[cur ^ 1], Bs[cur ^ 1], 0);
+                mfma_steps(1, 0, 4);
+                __builtin_amdgcn_s_setprio(0);
             }
-            __builtin_amdgcn_s_setprio(0);
-            if (more) {
-                ta.store(As[cur ^ 1]);
-                tb.store(Bs[cur ^ 1]);
+        } else {
+            if (nk > 0) {
+                ta.template load<CHK>(A, a.lda, m0, a.M, kbeg, kend);
+                tb.template load<CHK>(B, a.ldb, n0, a.N, kbeg, kend);
+                ta.store(As[0]);
+                tb.store(Bs[0]);
             }
             __syncthreads();
+            for (int kt = 0; kt < nk; ++kt) {
+                const int cur = kt & 1;
+                const bool more = kt + 1 < nk;
+                if (more) {
+                    const int k0 = kbeg + (kt + 1) * KT;
+                    ta.template load<CHK>(A, a.lda, m0, a.M, k0, kend);
+                    tb.template load<CHK>(B, a.ldb, n0, a.N, k0, kend);
+                }
+                __builtin_amdgcn_s_setprio(3);
+    #pragma unroll
+                for (int kk = 0; kk < KT / 8; ++kk) {
+                    read_frags(0, As[cur], Bs[cur], kk);
+                    mfma_steps(0, 0, 4);
+                }
+                __builtin_amdgcn_s_setprio(0);
+                if (more) {
+                    ta.store(As[cur ^ 1]);
+                    tb.store(Bs[cur ^ 1]);
+                }
+                __syncthreads();
+            }
         }
-    }
+    };
+    const bool interior = m0 + BM <= a.M && n0 + BN <= a.N && (kend - kbeg) % KT == 0;
+    if (interior) main_loop(std::false_type{});
+    else main_loop(std::true_type{});
 
     // accumulator element e of a 32x32 block: row 8*(e/4) + 4*half + e%4, column l32
     if (tail_piece >= 0) {
@@ -464,32 +483,34 @@ struct TileShape {
 // Tile shapes on offer; the 128x128 default comes first and wins ties.
 static const TileShape kShapes[] = {{128, 128}, {128, 96}, {128, 64}, {128, 32}, {96, 128}};
 
-template <bool AKC, bool BKC, bool VECA, bool VECB>
+template <bool AKC, bool BKC, bool VECA, bool VECB, bool PIPE>
 static void launch_shape(int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
     dim3 block(kGemmThreads);
     switch (shape) {
-        case 0: sgemm_kernel<AKC, BKC, VECA, VECB, 2, 2, 2, 2><<<grid, block, 0, st>>>(a); break;
-        case 1: sgemm_kernel<AKC, BKC, VECA, VECB, 4, 1, 1, 3><<<grid, block, 0, st>>>(a); break;
-        case 2: sgemm_kernel<AKC, BKC, VECA, VECB, 4, 1, 1, 2><<<grid, block, 0, st>>>(a); break;
-        case 3: sgemm_kernel<AKC, BKC, VECA, VECB, 4, 1, 1, 1><<<grid, block, 0, st>>>(a); break;
-        default: sgemm_kernel<AKC, BKC, VECA, VECB, 1, 4, 3, 1><<<grid, block, 0, st>>>(a); break;
+        case 0: sgemm_kernel<AKC, BKC, VECA, VECB, PIPE, 2, 2, 2, 2><<<grid, block, 0, st>>>(a); break;
+        case 1: sgemm_kernel<AKC, BKC, VECA, VECB, PIPE, 4, 1, 1, 3><<<grid, block, 0, st>>>(a); break;
+        case 2: sgemm_kernel<AKC, BKC, VECA, VECB, PIPE, 4, 1, 1, 2><<<grid, block, 0, st>>>(a); break;
+        case 3: sgemm_kernel<AKC, BKC, VECA, VECB, PIPE, 4, 1, 1, 1><<<grid, block, 0, st>>>(a); break;
+        default: sgemm_kernel<AKC, BKC, VECA, VECB, PIPE, 1, 4, 3, 1><<<grid, block, 0, st>>>(a); break;
     }
 }
 
-template <bool AKC, bool BKC>
+template <bool AKC, bool BKC, bool PIPE>
 static void launch_vec(bool vecA, bool vecB, int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
-    if (vecA && vecB) launch_shape<AKC, BKC, true, true>(shape, grid, st, a);
-    else if (vecA) launch_shape<AKC, BKC, true, false>(shape, grid, st, a);
-    else if (vecB) launch_shape<AKC, BKC, false, true>(shape, grid, st, a);
-    else launch_shape<AKC, BKC, false, false>(shape, grid, st, a);
+    if (vecA && vecB) launch_shape<AKC, BKC, true, true, PIPE>(shape, grid, st, a);
+    else if (vecA) launch_shape<AKC, BKC, true, false, PIPE>(shape, grid, st, a);
+    else if (vecB) launch_shape<AKC, BKC, false, true, PIPE>(shape, grid, st, a);
+    else launch_shape<AKC, BKC, false, false, PIPE>(shape, grid, st, a);
 }
 
-static void launch_trans(int tA, int tB, bool vecA, bool vecB, int shape, dim3 grid, hipStream_t st,
+static void launch_trans(int tA, int tB, bool pipe, bool vecA, bool vecB, int shape, dim3 grid, hipStream_t st,
                          const GemmArgs& a) {
-    if (!tA && !tB) launch_vec<true, false>(vecA, vecB, shape, grid, st, a);
-    else if (!tA && tB) launch_vec<true, true>(vecA, vecB, shape, grid, st, a);
-    else if (tA && !tB) launch_vec<false, false>(vecA, vecB, shape, grid, st, a);
-    else launch_vec<false, true>(vecA, vecB, shape, grid, st, a);
+    if (!tA && !tB) launch_vec<true, false, false>(vecA, vecB, shape, grid, st, a);
+    else if (!tA && tB) {
+        if (pipe) launch_vec<true, true, true>(vecA, vecB, shape, grid, st, a);
+        else launch_vec<true, true, false>(vecA, vecB, shape, grid, st, a);
+    } else if (tA && !tB) launch_vec<false, false, false>(vecA, vecB, shape, grid, st, a);
+    else launch_vec<false, true, false>(vecA, vecB, shape, grid, st, a);
 }
 
 static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const float* A, long lda,
@@ -580,7 +601,12 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     CGT_ARG_CHECK(wgs < (1L << 31), "sgemm: too many workgroups");
     hipStream_t st = as_stream(stream);
     dim3 grid((unsigned)wgs);
-    launch_trans(tA, tB, vecA, vecB, shape, grid, st, a);
+    // The pipelined loop needs ~134 registers (3 workgroups per CU instead of 4):
+    // it wins once every CU has more than a handful of tiles to work through and
+    // loses when the whole product is one round of resident workgroups
+    // (4096^3: 1024 tiles = 4 per CU).
+    const bool pipe = tiles * P >= 5L * kNumCU;
+    launch_trans(tA, tB, pipe, vecA, vecB, shape, grid, st, a);
     CGT_LAUNCH_CHECK("sgemm_kernel");
     if (a.splits > 1) {
         const long MN = M * N;

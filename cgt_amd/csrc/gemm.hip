@@ -436,16 +436,66 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restric
         if (n0 + c + j < a.N) dst[j] = o[j];
 }
 
-// C[r][c] = sum_s ws[s][r][c], s ascending.
+// C[r][c] = sum over splits of ws[s][r][c].  A workgroup takes 64 columns of
+// the flattened [M*N] index (64 x 16 bytes when VEC) and cuts the splits into 4
+// contiguous ranges, one per wavefront; each lane adds its range in ascending
+// order with 8 loads in flight, then the four range sums are added in ascending
+// order.  The order is fixed, so the result is deterministic; with hundreds of
+// splits and a small C (the MNIST / CIFAR weight gradients) a single running
+// sum per output would be one long chain of load latencies.
+constexpr int kReduceGroups = 4;
+
+template <bool VEC>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws,
                                                             float* __restrict__ C, long MN, int N,
                                                             long ldc, int splits) {
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < MN;
-         i += (long)gridDim.x * blockDim.x) {
-        float s = 0.0f;
-        for (int k = 0; k < splits; ++k) s += ws[(long)k * MN + i];
+    typedef typename std::conditional<VEC, float4, float>::type T;
+    constexpr int W = VEC ? 4 : 1;
+    __shared__ T part[kReduceGroups][64];
+    const int col = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const long i = ((long)blockIdx.x * 64 + col) * W;          // first flattened output index of this lane
+    const int per = (splits + kReduceGroups - 1) / kReduceGroups;
+    const int s0 = g * per, s1 = min(splits, s0 + per);
+    T acc;
+    if constexpr (VEC) acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    else acc = 0.0f;
+    if (i < MN) {
+        for (int sb = s0; sb < s1; sb += 8) {
+            T v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (sb + u < s1) v[u] = *reinterpret_cast<const T*>(ws + (long)(sb + u) * MN + i);
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (sb + u < s1) {
+                    if constexpr (VEC) {
+                        acc.x += v[u].x; acc.y += v[u].y; acc.z += v[u].z; acc.w += v[u].w;
+                    } else {
+                        acc += v[u];
+                    }
+                }
+        }
+    }
+    part[g][col] = acc;
+    __syncthreads();
+    if (g != 0 || i >= MN) return;
+    T tot = part[0][col];
+#pragma unroll
+    for (int k = 1; k < kReduceGroups; ++k) {
+        const T p = part[k][col];
+        if constexpr (VEC) {
+            tot.x += p.x; tot.y += p.y; tot.z += p.z; tot.w += p.w;
+        } else {
+            tot += p;
+        }
+    }
+    if constexpr (VEC) {
+        // N % 4 == 0: the four outputs share a row of C
         const long r = i / N, c = i - r * N;
-        C[r * ldc + c] = s;
+        *reinterpret_cast<float4*>(C + r * ldc + c) = tot;
+    } else {
+        const long r = i / N, c = i - r * N;
+        C[r * ldc + c] = tot;
     }
 }
 
@@ -610,8 +660,11 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     CGT_LAUNCH_CHECK("sgemm_kernel");
     if (a.splits > 1) {
         const long MN = M * N;
-        long blocks = std::min(cdiv(MN, 256L), 1L << 16);
-        splitk_reduce_kernel<<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a.ws, C, MN, (int)N, ldc, a.splits);
+        const bool vec = N % 4 == 0 && ldc % 4 == 0 && aligned16(C) && aligned16(a.ws);
+        const long blocks = cdiv(MN, vec ? 256L : 64L);
+        CGT_ARG_CHECK(blocks < (1L << 31), "sgemm: too many reduce workgroups");
+        if (vec) splitk_reduce_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a.ws, C, MN, (int)N, ldc, a.splits);
+        else splitk_reduce_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a.ws, C, MN, (int)N, ldc, a.splits);
         CGT_LAUNCH_CHECK("splitk_reduce_kernel");
     } else if (tail_tiles > 0) {
         tail_reduce_kernel<<<dim3((unsigned)cdiv(kShapes[shape].bm * kShapes[shape].bn, 1024), (unsigned)tail_tiles), dim3(256), 0, st>>>(

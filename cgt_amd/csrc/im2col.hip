@@ -293,7 +293,11 @@ __global__ __launch_bounds__(256) void col2im_gather_kernel(
 // LDS at the same offset from that boundary, with no index arithmetic at all).
 constexpr int kStageScalar = 0, kStageRuns = 1, kStageLinear = 2;
 
-template <class G, int CC, int WSUB, int MODE>
+//
+// LW = lanes along the image row per wavefront (64, 32 or 16): narrow images
+// (CIFAR's 15-wide feature maps) put 64/LW channels side by side in a
+// wavefront instead of leaving lanes idle.
+template <class G, int CC, int WSUB, int MODE, int LW = 64>
 __global__ __launch_bounds__(256) void col2im_stream_kernel(
     G g, const float* __restrict__ col, float* __restrict__ im, int C, int H, int W, int m, int n,
     int band, int bands, int tiles_w, int nchunks, long col_floats) {
@@ -302,8 +306,11 @@ __global__ __launch_bounds__(256) void col2im_stream_kernel(
     static_assert(SH <= KH && SW <= KW, "streaming col2im needs stride <= kernel");
     constexpr int KK = KH * KW, RUN = CC * KK;
     constexpr int LD = RUN | 1;                       // odd row stride: conflict-free column reads
-    constexpr int TW = 64 * WSUB;
-    constexpr int NQ = (CC * WSUB + 3) / 4;
+    constexpr int CSUB = 64 / LW;                     // channels side by side in a wavefront
+    static_assert(CC % CSUB == 0, "channel chunk must be a multiple of the channels per wavefront");
+    constexpr int CG = CC / CSUB;                     // channel groups per chunk
+    constexpr int TW = LW * WSUB;
+    constexpr int NQ = (CG * WSUB + 3) / 4;
     constexpr int NT = (KW + SW - 1) / SW;            // taps per row and pixel
     constexpr int NWB = (TW + KW - 2) / SW + 1;       // staged pixels per row, upper bound
     // staged values per thread: float4 units of full runs (VEC) or single floats
@@ -339,9 +346,9 @@ __global__ __launch_bounds__(256) void col2im_stream_kernel(
 #pragma unroll
     for (int i = 0; i < NQ; ++i) {
         const int q = wave + 4 * i;
-        cq[i] = q % CC;
-        wp[i] = wp0 + (q / CC) * 64 + lane;
-        ok[i] = (q < CC * WSUB) && (cq[i] < cc) && (wp[i] < W);
+        cq[i] = (q % CG) * CSUB + lane / LW;
+        wp[i] = wp0 + (q / CG) * LW + lane % LW;
+        ok[i] = (q < CG * WSUB) && (cq[i] < cc) && (wp[i] < W);
 #pragma unroll
         for (int j = 0; j < KH; ++j) acc[i][j] = 0.0f;
     }
@@ -488,10 +495,10 @@ __global__ __launch_bounds__(256) void col2im_stream_kernel(
     }
 }
 
-template <class G, int CC, int WSUB>
+template <class G, int CC, int WSUB, int LW = 64>
 static int launch_col2im_stream(G g, const float* col, long B, int C, int H, int W, int m, int n,
                                 float* im, hipStream_t st) {
-    constexpr int KK = G::kKH * G::kKW, RUN = CC * KK, LD = RUN | 1, TW = 64 * WSUB;
+    constexpr int KK = G::kKH * G::kKW, RUN = CC * KK, LD = RUN | 1, TW = LW * WSUB;
     const int tiles_w = (int)cdiv(W, TW), nchunks = (int)cdiv(C, CC);
     const long nwb = std::min((long)n, (long)(TW + G::kKW - 2) / G::kSW + 1);
     const size_t lds = ((size_t)nwb * LD + 8) * sizeof(float);
@@ -501,9 +508,9 @@ static int launch_col2im_stream(G g, const float* col, long B, int C, int H, int
     const bool al16 = reinterpret_cast<uintptr_t>(col) % 16 == 0;
     const int mode = (LD == RUN && C == CC && al16) ? kStageLinear
                      : (RUN % 4 == 0 && C % CC == 0 && al16) ? kStageRuns : kStageScalar;
-    auto kernel = mode == kStageLinear ? col2im_stream_kernel<G, CC, WSUB, (LD == RUN ? kStageLinear : kStageScalar)>
-                  : mode == kStageRuns ? col2im_stream_kernel<G, CC, WSUB, (RUN % 4 == 0 ? kStageRuns : kStageScalar)>
-                                       : col2im_stream_kernel<G, CC, WSUB, kStageScalar>;
+    auto kernel = mode == kStageLinear ? col2im_stream_kernel<G, CC, WSUB, (LD == RUN ? kStageLinear : kStageScalar), LW>
+                  : mode == kStageRuns ? col2im_stream_kernel<G, CC, WSUB, (RUN % 4 == 0 ? kStageRuns : kStageScalar), LW>
+                                       : col2im_stream_kernel<G, CC, WSUB, kStageScalar, LW>;
     // Bands of image rows: as many workgroups as the chip holds at once, and
     // no more.  The kernel is bound by the loads each wavefront can keep in
     // flight, so resident wavefronts are what counts; a second, partial round
@@ -631,6 +638,8 @@ static int try_col2im_stream(G, const float*, long, int, int, int, int, int, flo
 static int try_col2im_stream(StaticGeom<3, 3, 1, 1, 1, 1> g, const float* col, long B, int C, int H,
                            int W, int m, int n, float* im, hipStream_t st) {
     if (C >= 8 && W >= 24) return launch_col2im_stream<decltype(g), 8, 1>(g, col, B, C, H, W, m, n, im, st);
+    if (C >= 8 && W <= 16) return launch_col2im_stream<decltype(g), 8, 1, 16>(g, col, B, C, H, W, m, n, im, st);
+    if (C >= 8) return launch_col2im_stream<decltype(g), 8, 1, 32>(g, col, B, C, H, W, m, n, im, st);
     return -1;
 }
 static int try_col2im_stream(StaticGeom<3, 3, 0, 0, 1, 1> g, const float* col, long B, int C, int H,
@@ -641,6 +650,8 @@ static int try_col2im_stream(StaticGeom<3, 3, 0, 0, 1, 1> g, const float* col, l
 static int try_col2im_stream(StaticGeom<5, 5, 2, 2, 1, 1> g, const float* col, long B, int C, int H,
                            int W, int m, int n, float* im, hipStream_t st) {
     if (C >= 4 && W >= 24) return launch_col2im_stream<decltype(g), 4, 1>(g, col, B, C, H, W, m, n, im, st);
+    if (C >= 8 && W <= 16) return launch_col2im_stream<decltype(g), 8, 1, 16>(g, col, B, C, H, W, m, n, im, st);
+    if (C >= 4) return launch_col2im_stream<decltype(g), 4, 1, 32>(g, col, B, C, H, W, m, n, im, st);
     return -1;
 }
 static int try_col2im_stream(StaticGeom<11, 11, 0, 0, 4, 4> g, const float* col, long B, int C, int H,

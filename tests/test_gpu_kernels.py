@@ -103,6 +103,11 @@ IM2COL_CASES = [
     ((1, 3, 100, 300), (11, 11), (0, 0), (4, 4)),  # three column tiles at stride 4
     ((1, 2, 5, 2000), (3, 3), (1, 1), (1, 1)),     # rows longer than one pipelined staging buffer
     ((2, 40, 9, 30), (3, 3), (1, 1), (1, 1)),      # several channel chunks, last one partial
+    ((3, 20, 11, 12), (3, 3), (1, 1), (1, 1)),     # narrow image: 16 lanes per row, 4 channels abreast, partial chunk
+    ((2, 9, 7, 20), (3, 3), (0, 0), (1, 1)),       # 32 lanes per row
+    ((2, 6, 9, 20), (5, 5), (2, 2), (1, 1)),       # 5x5, 32 lanes per row, partial chunk
+    ((2, 12, 10, 10), (5, 5), (2, 2), (1, 1)),     # 5x5, 16 lanes per row, partial chunk
+    ((4, 64, 15, 15), (5, 5), (2, 2), (1, 1)),     # CIFAR conv2 at full channel count
 ]
 
 

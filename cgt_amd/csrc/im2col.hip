@@ -516,12 +516,12 @@ static int launch_col2im_stream(G g, const float* col, long B, int C, int H, int
     // flight, so resident wavefronts are what counts; a second, partial round
     // of workgroups costs more than it gains (measured on the AlexNet layer:
     // 2 bands 0.17 ms, 3 bands 0.21 ms), and each band re-reads kh - sh halo
-    // rows, so bands stay at least 4 kernel heights tall.
+    // rows, so bands stay at least 2 kernel heights tall.
     int wg_per_cu = 0;
     CGT_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&wg_per_cu, kernel, 256, lds));
     const long resident = (long)std::max(wg_per_cu, 1) * kNumCU;
     const long per_band = B * nchunks * tiles_w;
-    long bands = std::max(1L, std::min(resident / per_band, (long)H / (4 * G::kKH)));
+    long bands = std::max(1L, std::min(resident / per_band, (long)H / (2 * G::kKH)));
     const int band = (int)cdiv(cdiv(H, bands), G::kSH) * G::kSH;   // bands start on stride multiples
     bands = cdiv(H, band);
     const long blocks = per_band * bands;
@@ -650,6 +650,7 @@ static int try_col2im_stream(StaticGeom<3, 3, 0, 0, 1, 1> g, const float* col, l
 static int try_col2im_stream(StaticGeom<5, 5, 2, 2, 1, 1> g, const float* col, long B, int C, int H,
                            int W, int m, int n, float* im, hipStream_t st) {
     if (C >= 4 && W >= 24) return launch_col2im_stream<decltype(g), 4, 1>(g, col, B, C, H, W, m, n, im, st);
+    if (C == 3 && W >= 24) return launch_col2im_stream<decltype(g), 3, 1>(g, col, B, C, H, W, m, n, im, st);   // RGB input layer
     if (C >= 8 && W <= 16) return launch_col2im_stream<decltype(g), 8, 1, 16>(g, col, B, C, H, W, m, n, im, st);
     if (C >= 4) return launch_col2im_stream<decltype(g), 4, 1, 32>(g, col, B, C, H, W, m, n, im, st);
     return -1;

@@ -55,9 +55,12 @@ DEFAULT_WORKLOAD = "vgg_mid_conv3x3_128x56x56_b64"
 # WRITE_SIZE runs of this script (summaries and calibration in profiles/):
 # (workload, stage) -> bytes.  None where no counter run has been made.
 TRAFFIC = {
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_fwd_NT"): 1060500000,    # 2.0 * 472.6 MB fetched + 115.3 MB written
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_dgrad_NN"): 1136000000,  # 2.0 * 105.6 MB fetched + 924.8 MB written
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_wgrad_TN"): 1125500000,  # 2.0 * 529.7 MB fetched + 66.1 MB written (partials incl.)
+    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_fwd_NT"): 1059100000,    # 2.0 * 471.9 MB fetched + 115.3 MB written
+    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_dgrad_NN"): 1133000000,  # 2.0 * 104.1 MB fetched + 924.8 MB written
+    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_wgrad_TN"): 1126700000,  # 2.0 * 530.3 MB fetched + 66.1 MB written (partials incl.)
+    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_fwd_NT"): 768700000,    # 2.0 * 310.0 + 148.7
+    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_dgrad_NN"): 816600000,  # 2.0 * 79.4 + 657.8 (rows of 363 floats: partial lines)
+    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_wgrad_TN"): 903800000,  # 2.0 * 426.8 + 50.2 (partials incl.)
 }
 
 

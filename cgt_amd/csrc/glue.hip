@@ -43,6 +43,15 @@ __global__ __launch_bounds__(256) void batched_transpose_kernel(
 constexpr int kThinRows = 64;
 constexpr int kThinMaxL = 128;
 
+// Workgroups go to the 8 XCDs round-robin by id; give each XCD (one L2) a
+// contiguous range of ids, so the workgroups that share a cache line where
+// their unaligned runs meet find it in the same L2.
+__device__ __forceinline__ unsigned xcd_contiguous(unsigned id, unsigned n) {
+    const unsigned q = n / kNumXCD, r = n % kNumXCD;
+    const unsigned xcd = id % kNumXCD, local = id / kNumXCD;
+    return xcd * q + min(xcd, r) + local;
+}
+
 __device__ __forceinline__ int div_small(int n, int d, float rd) {
     // exact for 0 <= n < 2^21: the float quotient is off by at most one
     int q = (int)((float)n * rd);
@@ -57,8 +66,9 @@ __global__ __launch_bounds__(256) void thin_transpose_kernel(const float* __rest
                                                              int tiles_r) {
     extern __shared__ float tile[];          // [kThinRows][LD]
     const int LD = L | 1;
-    const int tr = blockIdx.x % tiles_r;
-    const long b = blockIdx.x / tiles_r;
+    const unsigned bid = xcd_contiguous(blockIdx.x, gridDim.x);
+    const int tr = bid % tiles_r;
+    const long b = bid / tiles_r;
     const int r0 = tr * kThinRows;
     const int rows = min(kThinRows, R - r0);
     const float rL = 1.0f / (float)L;

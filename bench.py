@@ -30,24 +30,24 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 
 WORKLOADS = {
-    # BASELINE.json configs[3]: VGG-style mid layer
+    # VGG-style mid layer (the headline configuration)
     "vgg_mid_conv3x3_128x56x56_b64": dict(
         x=(64, 128, 56, 56), f=(128, 128, 3, 3), pad=(1, 1), stride=(1, 1),
         fscale="he", lrn=None, pool=((2, 2), (0, 0), (2, 2))),
-    # BASELINE.json configs[2]: AlexNet conv1 -> LRN -> pool
+    # AlexNet conv1 -> LRN -> pool
     "alexnet_conv1_11x11s4_3x227x227_b128": dict(
         x=(128, 3, 227, 227), f=(96, 3, 11, 11), pad=(0, 0), stride=(4, 4),
         fscale=0.01, lrn=(5, 1e-4, 0.75, 1.0), pool=((3, 3), (0, 0), (2, 2))),
-    # BASELINE.json configs[1], second conv of the CIFAR stack (with its pool + LRN input side)
+    # second conv of the CIFAR stack (with its pool + LRN input side)
     "cifar_conv2_5x5_32x15x15_b128": dict(
         x=(128, 32, 15, 15), f=(64, 32, 5, 5), pad=(2, 2), stride=(1, 1),
         fscale=0.01, lrn=None, pool=None),
-    # BASELINE.json configs[0]: MNIST conv block (conv + pool)
+    # MNIST conv block (conv + pool)
     "mnist_conv3x3_1x28x28_b64": dict(
         x=(64, 1, 28, 28), f=(32, 1, 3, 3), pad=(1, 1), stride=(1, 1),
         fscale=0.1, lrn=None, pool=((2, 2), (0, 0), (2, 2))),
 }
-# BASELINE.json configs[4]: raw dense contraction
+# raw dense contraction
 GEMM_WORKLOAD = "raw_gemm_4096_and_batched_64x512"
 DEFAULT_WORKLOAD = "vgg_mid_conv3x3_128x56x56_b64"
 
@@ -361,7 +361,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (the hot path has no "
-                 "multi-GPU part: it would shard the batch axis, see DESIGN.md)" % args.gpus)
+                 "multi-GPU part: it would shard the batch axis)" % args.gpus)
 
     from cgt_amd import capi
     capi.require_gpu()

@@ -164,7 +164,7 @@ def test_conv2d_grad_through_op_pullbacks(cgt, xshape, fshape, pad, stride):
 
 
 def test_cifar_shaped_stack_forward_backward(cgt):
-    # BASELINE configs[1] in miniature: conv 5x5 p2 -> pool 3x3/2 -> LRN(5,1e-4,.75) -> conv 5x5 p2,
+    # the CIFAR-shaped stack in miniature: conv 5x5 p2 -> pool 3x3/2 -> LRN(5,1e-4,.75) -> conv 5x5 p2,
     # loss = sum of outputs; gradients wrt input and both weights.  (The ReLU between
     # conv and pool is an elementwise op outside the hot path and is left out on both sides.)
     from cgt_amd import nn

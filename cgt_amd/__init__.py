@@ -16,6 +16,7 @@ from .core import (BatchedMul22, ElwiseBinary, ElwiseUnary, Fill, MethodNotDefin
                    constant, cos, dot, elwise_binary, exp, fill, floatX, grad, greater_equal, log, mean,
                    neg, ones, ones_like, power, reshape, shape, sigmoid, sign, sin, size, sqrt, square,
                    sum, tanh, to_device, transpose, unpack, zeros, zeros_like)
+from .function import Function, function  # noqa: F401
 from .gpuarray import GpuArray, empty, to_gpu  # noqa: F401
 
 __all__ = ["nn", "core", "capi", "kernels", "compilation", "rt"]

@@ -203,6 +203,9 @@ def prebuild_standard_ops():
         (core.Repeat((0, 2, 3)), [T4, S, S, S]),
         (core.Sum((0, 2, 3)), [T4]),
         (core.Fill(0.0), [S, S, S, S]),
+        # by-value closures a compiled `function` replays
+        (core.Reshape(), [T4, S, S]),
+        (core.TupleIndex(0), [core.TupleType(T4, I4)]),
     ]
     built = []
     for op, types in todo:

@@ -360,7 +360,7 @@ def Result(op, parents):
     parents = [as_node(p) for p in parents]
     input_types = [p.typ for p in parents]
     typ = op.typ_apply(input_types)
-    if "python" in op.available_impls and "native_gpu" not in op.available_impls:
+    if "python" in op.available_impls and (op.return_type == "byval" or "native_gpu" not in op.available_impls):
         value = op.get_py_func(input_types)([p.value for p in parents])
     else:
         out = _alloc(typ, op.shp_apply(parents))
@@ -370,11 +370,21 @@ def Result(op, parents):
 
 
 class TupleIndex(Op):
-    """Member of a tuple-valued node (reference core.py:2420-2442)."""
-    available_impls = ("python",)
+    """Member of a tuple-valued node (reference core.py:2420-2442).  Evaluated in
+    python while nodes are built; the native by-value closure is what a compiled
+    `function` replays."""
+    available_impls = ("python", "native_cpu", "native_gpu")
+    return_type = "byval"
 
     def __init__(self, idx):
         self.idx = idx
+
+    def get_native_compile_info(self, input_types, devtype):
+        code = r"""
+            CGT_EXPORT_C cgtObject* $function($closure* cldata, cgtTuple** reads) {
+                return reads[0]->getitem(cldata->idx);
+            }"""
+        return NativeCompileInfo(code, closure_triples=[("idx", ctypes.c_int, self.idx)])
 
     def typ_apply(self, input_types):
         return input_types[0][self.idx]
@@ -607,9 +617,28 @@ class Transpose(Op):
 
 class Reshape(Op):
     """Zero-copy view with a new shape (reference core.py:1432-1465, a by-value op
-    whose result shares the input's data)."""
-    available_impls = ("python",)
+    whose result shares the input's data).  Evaluated in python while nodes are
+    built; the native by-value closure is what a compiled `function` replays."""
+    available_impls = ("python", "native_cpu", "native_gpu")
     return_type = "byval"
+
+    def get_native_compile_info(self, input_types, devtype):
+        # the view borrows the input's storage (kept alive by its storage slot);
+        # shape operands are host integers
+        code = r"""
+            CGT_EXPORT_C cgtObject* $function($closure* cldata, cgtArray** reads) {
+                cgtArray* in = reads[0];
+                long newshape[16];
+                long n = 1;
+                for (int i = 0; i < cldata->ndim; ++i) {
+                    newshape[i] = static_cast<long*>(reads[i + 1]->data())[0];
+                    n *= newshape[i];
+                }
+                cgt_check(n == in->size(), "Reshape: size mismatch (%ld vs %ld)", n, in->size());
+                return new cgtArray(cldata->ndim, newshape, in->dtype(), in->devtype(), in->data(), false);
+            }"""
+        return NativeCompileInfo(code, closure_triples=[("ndim", ctypes.c_int, len(input_types) - 1)],
+                                 gpu_deref_mask=(False,) * len(input_types))
 
     def get_diff(self, num_inputs):
         return [True] + [False] * (num_inputs - 1)

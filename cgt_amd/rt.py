@@ -192,6 +192,12 @@ class Interpreter(object):
         return self._ok(self._L.cgt_rt_interp_add_return_byref(self.handle, callable_.fptr_address, callable_.closure_address,
                                                                idx, dev, n, wloc[0], wloc[1]), "ReturnByRef")
 
+    def return_byval(self, callable_, read_locs, wloc):
+        idx, dev, n = self._locs(read_locs)
+        self._keep.append(callable_)
+        return self._ok(self._L.cgt_rt_interp_add_return_byval(self.handle, callable_.fptr_address, callable_.closure_address,
+                                                               idx, dev, n, wloc[0], wloc[1]), "ReturnByVal")
+
     def set_slot(self, idx, value):
         obj = to_cgt(value)
         self._keep.append(obj)

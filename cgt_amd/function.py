@@ -20,11 +20,24 @@ from .gpuarray import GpuArray, to_gpu
 
 
 class Function(object):
-    def __init__(self, inputs, outputs, device_outputs=False):
+    def __init__(self, inputs, outputs, device_outputs=False, updates=None):
         self._single = isinstance(outputs, core.Node)
         self.inputs = [core.as_node(i) for i in inputs]
         self.outputs = [outputs] if self._single else list(outputs)
         self.device_outputs = device_outputs
+        # updates: (before, after) pairs; `after` is written straight into the
+        # storage of the leaf `before` (the reference gives both the same memory
+        # owner, cgt/compilation.py:150-163).  The op that produces `after` is
+        # moved to the end of the list so every reader of the old value has run.
+        updates = list(updates.items()) if isinstance(updates, dict) else list(updates or [])
+        for before, after in updates:
+            if before.op is not None:
+                raise ValueError("the left-hand side of an update must be a leaf node (a parameter)")
+            if after.op is None or after.op.return_type != "byref" or isinstance(after.typ, core.TupleType):
+                raise ValueError("the right-hand side of an update must be the result of a by-reference op")
+            if tuple(after.shape) != tuple(before.shape) or after.typ != before.typ:
+                raise ValueError("update changes the parameter's shape or type")
+        update_target = {id(after): before for before, after in updates}
         for n in self.inputs:
             if n.op is not None:
                 raise ValueError("function inputs must be leaf nodes")
@@ -40,7 +53,11 @@ class Function(object):
 
         for o in self.outputs:
             visit(o)
+        for before, after in updates:
+            visit(before)
+            visit(after)
         self._order = order
+        deferred = []        # the ops that write the updates, emitted last
         # ---- slot assignment
         slot_of, n_slots = {}, 0
 
@@ -94,11 +111,16 @@ class Function(object):
                     members.append(m)
                 w = (new_slot(), members[0][1])
                 plan.append(("tup", members, w))
+            elif id(n) in update_target:
+                deferred.append(("byref", call, reads, slot_of[id(update_target[id(n)])]))
+                slot_of[id(n)] = slot_of[id(update_target[id(n)])]
+                continue
             else:
                 w = (new_slot(), dev(n.value))
                 plan.append(("alloc", np.dtype(n.typ.dtype), [(const_slot(d), rt.CPU) for d in n.value.shape], w))
             plan.append(("byref", call, reads, w))
             slot_of[id(n)] = w
+        plan.extend(deferred)
         # ---- emit
         it = rt.Interpreter(n_slots)
         for step in plan:
@@ -142,9 +164,10 @@ class Function(object):
         return outs[0] if self._single else outs
 
 
-def function(inputs, outputs, device_outputs=False):
+def function(inputs, outputs, device_outputs=False, updates=None):
     """Compile the nodes between `inputs` and `outputs` (reference cgt.function).
     Results come back as numpy arrays, like the reference's; with
     device_outputs=True they are device arrays that view the function's own
-    buffers and are overwritten by its next call."""
-    return Function(inputs, outputs, device_outputs)
+    buffers and are overwritten by its next call.  `updates` is a list of
+    (parameter, new value) pairs applied in place at the end of every call."""
+    return Function(inputs, outputs, device_outputs, updates)

@@ -59,3 +59,10 @@ def max_pool_2d(x, kernelshape, pad=(0, 0), stride=(1, 1)):
     stride_h, stride_w = stride
     info = PoolInfo(kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w)
     return core.Result(MaxPool(info), [x])[0]
+
+
+def sgd(cost, params, learning_rate):
+    """Stochastic gradient descent updates, param := param - learning_rate * gradient
+    (reference cgt/nn.py:240-262): a list of (param, new_param) for function(..., updates=)."""
+    grads = core.grad(cost, params)
+    return [(param, param - learning_rate * g) for param, g in zip(params, grads)]

@@ -113,3 +113,40 @@ def test_function_dispatch_is_cheaper_than_node_by_node(cgt):
     print("150 ops: compiled function %.3f ms, node by node %.3f ms" % (t_fn * 1e3, t_py * 1e3))
     assert np.array_equal(f(xg).get(), y.get())
     assert t_fn < t_py
+
+
+def test_function_with_sgd_updates_trains_in_place(cgt):
+    # loss = sum((pool(relu(conv(x) + b)))^2); five SGD steps on W and b through one compiled
+    # function against the same steps in float64 built from the oracle's pieces
+    from cgt_amd import nn
+    rs = np.random.RandomState(2)
+    x = rs.randn(4, 3, 12, 12).astype(np.float32)
+    w = (rs.randn(6, 3, 3, 3) / 5).astype(np.float32)
+    b = (0.1 * rs.randn(1, 6, 1, 1)).astype(np.float32)
+    lr = 1e-3
+    layer = nn.SpatialConvolution(3, 6, (3, 3), (1, 1), weight_init=w, bias_init=b)
+    xn = cgt.constant(x)
+    pooled = nn.max_pool_2d(nn.rectify(layer(xn)), (2, 2), (0, 0), (2, 2))
+    loss = cgt.sum(pooled * pooled)
+    params = [layer.weight, layer.bias]
+    step = cgt.function([xn], loss, updates=nn.sgd(loss, params, lr))
+    wptr = layer.weight.value.ptr
+
+    w64, b64, x64 = w.astype(np.float64), b.astype(np.float64), x.astype(np.float64)
+    losses, ref_losses = [], []
+    for _ in range(5):
+        losses.append(float(step(x)))
+        pre = O.conv2d(x64, w64, (1, 1), (1, 1)) + b64
+        act = pre * (pre >= 0)
+        p, mask = O.max_pool(act, (2, 2), (0, 0), (2, 2))
+        ref_losses.append(float((p * p).sum()))
+        gact = O.max_pool_pullback(act.shape, mask, 2 * p)
+        gpre = gact * (pre >= 0)
+        _, gw = O.conv2d_pullback(x64, w64, gpre, (1, 1), (1, 1))
+        w64 = w64 - lr * gw
+        b64 = b64 - lr * gpre.sum((0, 2, 3), keepdims=True)
+    assert layer.weight.value.ptr == wptr                       # updated in place
+    assert np.allclose(losses, ref_losses, rtol=1e-4)
+    assert losses[-1] < losses[0]
+    assert np.linalg.norm(layer.weight.get() - w64) <= 1e-4 * np.linalg.norm(w64)
+    assert np.linalg.norm(layer.bias.get() - b64) <= 1e-4 * np.linalg.norm(b64)

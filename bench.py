@@ -290,6 +290,35 @@ def check_against_oracle(cfg):
     return {"im2col_bit_exact": bool(ok), "conv2d_rel_fro": err, "ok": bool(ok and err <= 1e-4)}
 
 
+def op_api_step_ms(cfg, steps, warmup):
+    """The same layer built with the Op API (nn.conv2d / cross_channel_lrn /
+    max_pool_2d, grad through the ops' pullbacks), compiled with cgt.function and
+    replayed by the C++ interpreter on one stream: ms per step."""
+    import cgt_amd as cgt
+    from cgt_amd import capi, nn
+    x, f = make_inputs(cfg)
+    xn, fn = cgt.constant(x), cgt.constant(f)
+    out = nn.conv2d(xn, fn, tuple(cfg["f"][2:]), tuple(cfg["pad"]), tuple(cfg["stride"]))
+    if cfg["lrn"]:
+        size, alpha, beta, k = cfg["lrn"]
+        out = nn.cross_channel_lrn(out, size, alpha, beta, k)
+    if cfg["pool"]:
+        pk, pp, ps = cfg["pool"]
+        out = nn.max_pool_2d(out, pk, pp, ps)
+    gx, gf = cgt.grad(out, [xn, fn], goutput=cgt.ones(cgt.shape(out)))
+    fun = cgt.function([xn, fn], [out, gx, gf], device_outputs=True)
+    args = (xn.value, fn.value)
+    del out, gx, gf
+    for _ in range(warmup):
+        fun(*args)
+    capi.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fun(*args)
+    capi.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e3, fun.n_instructions
+
+
 def cpu_baseline(cfg, sample_batch):
     """The CPU path (oracle stages + OpenBLAS sgemm) on a bounded sample of the workload."""
     from oracle import cpu_baseline as CB
@@ -356,6 +385,7 @@ def main():
     ap.add_argument("--glue", action="store_true",
                     help="also time the conv-layer glue kernels (bias add, ReLU, their gradients, loss sum) on the "
                          "layer's activation; they appear in `glue_stages`, outside the step")
+    ap.add_argument("--no-op-api", action="store_true", help="skip timing the same step through the Op API")
     ap.add_argument("--no-check", action="store_true",
                     help="skip the parity gate (profiling runs: keeps its small launches out of the kernel statistics)")
     args = ap.parse_args()
@@ -435,6 +465,13 @@ def main():
     }
     if is_gemm:
         out["config"]["value_is"] = "flops of Mul22 4096^3 x {NN,NT,TN,TT} + BatchedMul22 64x512^3 / step time"
+    elif not args.no_op_api:
+        del layer        # the traced graph holds its own buffers
+        ms, n_instr = op_api_step_ms(cfg, args.steps, args.warmup)
+        out["op_api_step"] = {"ms_per_step": round(ms, 4), "TFLOPs": round(value * ms_per_step / ms, 3),
+                              "instructions": n_instr,
+                              "what": "the same step through nn.conv2d / cross_channel_lrn / max_pool_2d + grad, compiled "
+                                      "with cgt.function and replayed by the C++ interpreter (one stream)"}
     if not args.no_cpu and not is_gemm:
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample)
     elif not args.no_cpu:

@@ -34,6 +34,10 @@ PROTOTYPES = {
     "cgt_amd_event_destroy": (c_int, [c_void_p]),
     "cgt_amd_event_record": (c_int, [c_void_p, c_void_p]),
     "cgt_amd_stream_wait_event": (c_int, [c_void_p, c_void_p]),
+    "cgt_amd_graph_capture_begin": (c_int, [c_void_p]),
+    "cgt_amd_graph_capture_end": (c_int, [c_void_p, ctypes.POINTER(c_void_p)]),
+    "cgt_amd_graph_launch": (c_int, [c_void_p, c_void_p]),
+    "cgt_amd_graph_destroy": (c_int, [c_void_p]),
     "cgt_amd_event_elapsed_ms": (c_int, [c_void_p, c_void_p, ctypes.POINTER(ctypes.c_float)]),
     "cgt_amd_im2col_f32": (c_int, [c_void_p] + [c_long] * 4 + [c_int] * 6 + [c_void_p, c_void_p]),
     "cgt_amd_col2im_f32": (c_int, [c_void_p] + [c_long] * 4 + [c_int] * 6 + [c_void_p, c_void_p]),
@@ -135,6 +139,35 @@ class Stream(object):
     def __del__(self):
         if getattr(self, "handle", None) is not None and _LIB is not None:
             _LIB.cgt_amd_stream_destroy(self.handle)
+            self.handle = None
+
+
+class Graph(object):
+    """A captured launch sequence (HIP graph).  Use:
+        g = Graph.capture(stream, fn)   # fn() issues its launches to `stream`
+        g.launch()
+    """
+
+    def __init__(self, handle, stream):
+        self.handle, self.stream = handle, stream
+
+    @classmethod
+    def capture(cls, stream, fn):
+        h = c_void_p()
+        check(lib().cgt_amd_graph_capture_begin(stream.handle))
+        try:
+            fn()
+        finally:
+            rc = lib().cgt_amd_graph_capture_end(stream.handle, ctypes.byref(h))
+        check(rc)
+        return cls(h, stream)
+
+    def launch(self):
+        check(lib().cgt_amd_graph_launch(self.handle, self.stream.handle))
+
+    def __del__(self):
+        if getattr(self, "handle", None) is not None and _LIB is not None:
+            _LIB.cgt_amd_graph_destroy(self.handle)
             self.handle = None
 
 

@@ -148,6 +148,40 @@ CGT_API int cgt_amd_stream_wait_event(void* stream, void* event) {
     return CGT_AMD_OK;
 }
 
+// ---- stream capture: a fixed sequence of launches recorded once, replayed as one graph
+
+CGT_API int cgt_amd_graph_capture_begin(void* stream) {
+    CGT_ARG_CHECK(stream, "graph_capture_begin: needs a created stream (the default stream cannot be captured)");
+    CGT_HIP_TRY(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal));
+    return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_graph_capture_end(void* stream, void** graph_exec) {
+    CGT_ARG_CHECK(stream && graph_exec, "graph_capture_end: null");
+    hipGraph_t graph = nullptr;
+    CGT_HIP_TRY(hipStreamEndCapture(as_stream(stream), &graph));
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) {
+        set_error("hipGraphInstantiate failed: %s", hipGetErrorString(e));
+        return CGT_AMD_ERR_HIP;
+    }
+    *graph_exec = exec;
+    return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_graph_launch(void* graph_exec, void* stream) {
+    CGT_ARG_CHECK(graph_exec, "graph_launch: null graph");
+    CGT_HIP_TRY(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec), as_stream(stream)));
+    return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_graph_destroy(void* graph_exec) {
+    if (graph_exec) CGT_HIP_TRY(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec)));
+    return CGT_AMD_OK;
+}
+
 CGT_API int cgt_amd_event_elapsed_ms(void* start, void* stop, float* ms) {
     CGT_ARG_CHECK(start && stop && ms, "event_elapsed: null");
     CGT_HIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(stop)));

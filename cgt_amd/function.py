@@ -20,8 +20,15 @@ from .gpuarray import GpuArray, to_gpu
 
 
 class Function(object):
-    def __init__(self, inputs, outputs, device_outputs=False, updates=None):
+    def __init__(self, inputs, outputs, device_outputs=False, updates=None, use_graph=False):
         self._single = isinstance(outputs, core.Node)
+        # use_graph: the instruction list is recorded once into a HIP graph (on a
+        # stream of its own) and replayed with one launch per call; arguments are
+        # copied into fixed staging buffers because device addresses are baked in.
+        self.use_graph = use_graph
+        self._graph = self._stream = None
+        self._staging = None
+        self.sync = True      # graph mode: wait for the replay before returning
         self.inputs = [core.as_node(i) for i in inputs]
         self.outputs = [outputs] if self._single else list(outputs)
         self.device_outputs = device_outputs
@@ -156,7 +163,10 @@ class Function(object):
                 raise ValueError("argument has shape %s; this function was compiled for %s"
                                  % (tuple(a.shape), shape))
             vals.append(a)
-        self._it.run(vals)
+        if self.use_graph:
+            self._run_graph(vals)
+        else:
+            self._it.run(vals)
         outs = [self._it.get_array(s) for s in self._out_slots]
         if not self.device_outputs:
             outs = [tuple(m.get() if isinstance(m, GpuArray) else m for m in o) if isinstance(o, tuple)
@@ -164,10 +174,43 @@ class Function(object):
         return outs[0] if self._single else outs
 
 
-def function(inputs, outputs, device_outputs=False, updates=None):
+    def _run_graph(self, vals):
+        from . import capi
+        from .gpuarray import GpuArray as GA, empty
+        if self._stream is None:
+            self._stream = capi.Stream()
+            self._staging = [empty(v.shape, v.dtype) if isinstance(v, GA) else None for v in vals]
+        staged = []
+        for v, s in zip(vals, self._staging):
+            if s is None:
+                staged.append(v)              # host operand (shape integers): read at capture time
+            else:
+                if v.ptr != s.ptr:
+                    capi.check(capi.lib().cgt_amd_memcpy(capi.GPU, capi.GPU, s.ptr, v.ptr, s.nbytes))
+                staged.append(s)
+        rt.set_stream(self._stream.handle)
+        try:
+            if self._graph is None:
+                # first call: run for real (this also grows workspaces and allocates
+                # the output buffers), then record the same sequence without running it
+                self._it.run(staged)
+                self._stream.synchronize()
+                self._graph = capi.Graph.capture(self._stream, lambda: self._it.run(staged))
+            else:
+                self._graph.launch()
+                if self.sync:
+                    self._stream.synchronize()
+        finally:
+            rt.set_stream(None)
+
+
+def function(inputs, outputs, device_outputs=False, updates=None, use_graph=False):
     """Compile the nodes between `inputs` and `outputs` (reference cgt.function).
     Results come back as numpy arrays, like the reference's; with
     device_outputs=True they are device arrays that view the function's own
     buffers and are overwritten by its next call.  `updates` is a list of
-    (parameter, new value) pairs applied in place at the end of every call."""
-    return Function(inputs, outputs, device_outputs, updates)
+    (parameter, new value) pairs applied in place at the end of every call.
+    use_graph=True records the instruction list into a HIP graph on the first
+    call and replays it with a single launch afterwards (for launch-bound graphs
+    of small kernels)."""
+    return Function(inputs, outputs, device_outputs, updates, use_graph)

@@ -82,6 +82,19 @@ int cgt_amd_event_record(void *event, void *stream);
 int cgt_amd_stream_wait_event(void *stream, void *event);
 int cgt_amd_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for stop */
 
+/* HIP graph of a fixed launch sequence: between capture_begin and capture_end
+ * every launch issued to `stream` (a created stream, not NULL) by the calling
+ * thread is recorded instead of run; graph_launch replays the recording.  For
+ * launch-bound sequences (the MNIST / CIFAR sized layers: a dozen kernels of a
+ * few microseconds).  Everything in this library can be captured except the
+ * first call that grows a workspace (split-K GEMM, sum): run the sequence once
+ * on the same stream before capturing it.  Device pointers are baked into the
+ * graph. */
+int cgt_amd_graph_capture_begin(void *stream);
+int cgt_amd_graph_capture_end(void *stream, void **graph_exec);
+int cgt_amd_graph_launch(void *graph_exec, void *stream);
+int cgt_amd_graph_destroy(void *graph_exec);
+
 /* ---------------------------------------------------------------- conv-layer glue
  *
  * The ops either side of the GEMM path in a SpatialConvolution training step:

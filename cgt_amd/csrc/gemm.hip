@@ -25,10 +25,9 @@
 // products match; only the summation order inside the group differs from
 // k-ascending.
 //
-// Global loads are 16 bytes per lane when the leading dimension and base
-// address allow it; otherwise a second instantiation reads 4 bytes per lane
-// with consecutive lanes on consecutive addresses (im2col buffers have
-// Z = 363 or 75 floats per row).
+// Global loads are 16 bytes per lane at any 4-byte aligned address (the
+// im2col buffers of the AlexNet and CIFAR layers have Z = 363 or 75 floats per
+// row: global_load_dwordx4 does not need more alignment than a float's).
 //
 // Skinny outputs (few tiles, long K: the conv weight gradient) are split along
 // K into a workspace of partial tiles, reduced afterwards in a fixed order, so
@@ -44,6 +43,12 @@
 namespace cgt_amd {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
+
+// Four consecutive floats at any 4-byte aligned address: global_load_dwordx4
+// needs no more alignment than that (rows of 363 floats start anywhere).
+struct __attribute__((packed, aligned(4))) float4u {
+    float x, y, z, w;
+};
 
 constexpr int KT = 16;
 constexpr int kGemmThreads = 256;
@@ -95,7 +100,7 @@ struct OperandTile {
                         const int row = r0 + (idx >> 2), k = k0 + (idx & 3) * 4;
                         const float* src = p + (long)row * ld + k;
                         if (!CHECK || (row < R && k + 3 < kend)) {
-                            const float4 q = *reinterpret_cast<const float4*>(src);
+                            const float4u q = *reinterpret_cast<const float4u*>(src);
                             t[0] = q.x; t[1] = q.y; t[2] = q.z; t[3] = q.w;
                         } else if (row < R) {
 #pragma unroll
@@ -106,7 +111,7 @@ struct OperandTile {
                         const int k = k0 + idx / (ROWS / 4), row = r0 + (idx % (ROWS / 4)) * 4;
                         const float* src = p + (long)k * ld + row;
                         if (!CHECK || (k < kend && row + 3 < R)) {
-                            const float4 q = *reinterpret_cast<const float4*>(src);
+                            const float4u q = *reinterpret_cast<const float4u*>(src);
                             t[0] = q.x; t[1] = q.y; t[2] = q.z; t[3] = q.w;
                         } else if (k < kend) {
 #pragma unroll
@@ -545,22 +550,22 @@ static void launch_shape(int shape, dim3 grid, hipStream_t st, const GemmArgs& a
     }
 }
 
+// Both operands always take the 16-byte load path: it needs 4-byte alignment
+// only (float4u), so odd leading dimensions (Z = 363, 75) qualify too; measured
+// 8-34 % faster than coalesced 4-byte loads on such shapes.  The 4-byte variants
+// of OperandTile remain for reference and are not instantiated.
 template <bool AKC, bool BKC, bool PIPE>
-static void launch_vec(bool vecA, bool vecB, int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
-    if (vecA && vecB) launch_shape<AKC, BKC, true, true, PIPE>(shape, grid, st, a);
-    else if (vecA) launch_shape<AKC, BKC, true, false, PIPE>(shape, grid, st, a);
-    else if (vecB) launch_shape<AKC, BKC, false, true, PIPE>(shape, grid, st, a);
-    else launch_shape<AKC, BKC, false, false, PIPE>(shape, grid, st, a);
+static void launch_vec(int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
+    launch_shape<AKC, BKC, true, true, PIPE>(shape, grid, st, a);
 }
 
-static void launch_trans(int tA, int tB, bool pipe, bool vecA, bool vecB, int shape, dim3 grid, hipStream_t st,
-                         const GemmArgs& a) {
-    if (!tA && !tB) launch_vec<true, false, false>(vecA, vecB, shape, grid, st, a);
+static void launch_trans(int tA, int tB, bool pipe, int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
+    if (!tA && !tB) launch_vec<true, false, false>(shape, grid, st, a);
     else if (!tA && tB) {
-        if (pipe) launch_vec<true, true, true>(vecA, vecB, shape, grid, st, a);
-        else launch_vec<true, true, false>(vecA, vecB, shape, grid, st, a);
-    } else if (tA && !tB) launch_vec<false, false, false>(vecA, vecB, shape, grid, st, a);
-    else launch_vec<false, true, false>(vecA, vecB, shape, grid, st, a);
+        if (pipe) launch_vec<true, true, true>(shape, grid, st, a);
+        else launch_vec<true, true, false>(shape, grid, st, a);
+    } else if (tA && !tB) launch_vec<false, false, false>(shape, grid, st, a);
+    else launch_vec<false, true, false>(shape, grid, st, a);
 }
 
 static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const float* A, long lda,
@@ -595,8 +600,6 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     a.tiles_n = (int)cdiv(N, kShapes[shape].bn);
     a.batch = (int)P;
     const long tiles = (long)a.tiles_m * a.tiles_n;
-    const bool vecA = lda % 4 == 0 && sA % 4 == 0 && aligned16(A);
-    const bool vecB = ldb % 4 == 0 && sB % 4 == 0 && aligned16(B);
     a.splits = 1;
     a.kchunk = (int)(cdiv(std::max(K, 1L), KT) * KT);
     a.ws = nullptr;
@@ -656,7 +659,7 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     // loses when the whole product is one round of resident workgroups
     // (4096^3: 1024 tiles = 4 per CU).
     const bool pipe = tiles * P >= 5L * kNumCU;
-    launch_trans(tA, tB, pipe, vecA, vecB, shape, grid, st, a);
+    launch_trans(tA, tB, pipe, shape, grid, st, a);
     CGT_LAUNCH_CHECK("sgemm_kernel");
     if (a.splits > 1) {
         const long MN = M * N;

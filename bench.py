@@ -58,9 +58,9 @@ TRAFFIC = {
     ("vgg_mid_conv3x3_128x56x56_b64", "gemm_fwd_NT"): 1059100000,    # 2.0 * 471.9 MB fetched + 115.3 MB written
     ("vgg_mid_conv3x3_128x56x56_b64", "gemm_dgrad_NN"): 1133000000,  # 2.0 * 104.1 MB fetched + 924.8 MB written
     ("vgg_mid_conv3x3_128x56x56_b64", "gemm_wgrad_TN"): 1126700000,  # 2.0 * 530.3 MB fetched + 66.1 MB written (partials incl.)
-    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_fwd_NT"): 768700000,    # 2.0 * 310.0 + 148.7
-    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_dgrad_NN"): 816600000,  # 2.0 * 79.4 + 657.8 (rows of 363 floats: partial lines)
-    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_wgrad_TN"): 903800000,  # 2.0 * 426.8 + 50.2 (partials incl.)
+    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_fwd_NT"): 815100000,    # 2.0 * 333.2 + 148.7
+    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_dgrad_NN"): 863300000,  # 2.0 * 82.1 + 699.1 (rows of 363 floats: partial lines)
+    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_wgrad_TN"): 1033000000,  # 2.0 * 491.3 + 50.4 (partials incl.)
 }
 
 

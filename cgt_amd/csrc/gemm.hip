@@ -71,96 +71,102 @@ struct GemmArgs {
     // gets an equal share of the last, partial round.  Pieces go to ws as
     // [piece][BM][BN]; tail_reduce_kernel adds them up in order.
     int main_wgs, tail_splits, tail_kchunk;
+    int wide;          // a leading dimension too large for 32-bit tile offsets: tested loads everywhere
 };
 
-// One ROWS x KT operand tile.
+// One ROWS x KT operand tile, moved with 16-byte accesses.
 // KC: element (r, k) lives at p[r*ld + k]; otherwise at p[k*ld + r].
-// VEC: 16-byte global loads (needs ld % 4 == 0 and a 16-byte aligned base).
-template <bool KC, int ROWS, bool VEC>
+//
+// Every non-matrix instruction a wavefront issues takes its SIMD away from the
+// matrix pipe for a few cycles (fp32 MFMAs and vector ALU work do not overlap
+// on this chip: measured +6 cycles per VALU instruction against 64 per MFMA), so
+// the steady-state loads carry no address arithmetic: a thread's byte offsets
+// inside the tile are fixed for the whole kernel (goff), the tile origin of the
+// current K slice is a wave-uniform pointer advanced by scalar adds, and the
+// hardware adds the two (global_load_dwordx4 v, v_off, s[base]).
+template <bool KC, int ROWS>
 struct OperandTile {
     static constexpr int LDM = ROWS + 4;
     static constexpr int kFloats = KC ? ROWS * LDK : KT * LDM;
     static constexpr int kElems = ROWS * KT;
-    static constexpr int kPerThread = (kElems + kGemmThreads - 1) / kGemmThreads;   // 8 for 128 rows
-    static constexpr int NV = (kPerThread + 3) / 4;
+    static constexpr int NV = (kElems / 4 + kGemmThreads - 1) / kGemmThreads;   // 16-byte pieces per thread
     float v[NV * 4];
+    unsigned goff[NV];
 
-    // CHECK = false: the caller guarantees the whole tile slice is in range
-    // (interior tile, K range a multiple of KT) -- straight-line loads.
-    template <bool CHECK>
-    __device__ __forceinline__ void load(const float* __restrict__ p, long ld, int r0, int R,
-                                         int k0, int kend) {
-        if (VEC) {
+    // piece i of this thread exists (always, when the tile is a whole number of rounds)
+    static __device__ __forceinline__ bool has(int i) {
+        return (i + 1) * kGemmThreads * 4 <= kElems || (threadIdx.x + i * kGemmThreads) * 4 < kElems;
+    }
+
+    // needs (ROWS - 1) * ld * 4 + 64 < 2^32 (the host checks)
+    __device__ __forceinline__ void init_offsets(long ld) {
 #pragma unroll
-            for (int i = 0; i < NV; ++i) {
-                const int idx = threadIdx.x + i * kGemmThreads;     // float4 index
-                float t[4] = {0.f, 0.f, 0.f, 0.f};
-                if (idx * 4 < kElems) {
-                    if (KC) {
-                        const int row = r0 + (idx >> 2), k = k0 + (idx & 3) * 4;
-                        const float* src = p + (long)row * ld + k;
-                        if (!CHECK || (row < R && k + 3 < kend)) {
-                            const float4u q = *reinterpret_cast<const float4u*>(src);
-                            t[0] = q.x; t[1] = q.y; t[2] = q.z; t[3] = q.w;
-                        } else if (row < R) {
+        for (int i = 0; i < NV; ++i) {
+            const int idx = threadIdx.x + i * kGemmThreads;
+            const long e = KC ? (long)(idx >> 2) * ld + (idx & 3) * 4
+                              : (long)(idx / (ROWS / 4)) * ld + (idx % (ROWS / 4)) * 4;
+            goff[i] = (unsigned)(e * 4);
+        }
+    }
+
+    // the whole tile slice is in range: origin = address of tile element (0, 0) of this slice
+    __device__ __forceinline__ void load_fast(const char* __restrict__ origin) {
 #pragma unroll
-                            for (int j = 0; j < 4; ++j)
-                                if (k + j < kend) t[j] = src[j];
-                        }
-                    } else {
-                        const int k = k0 + idx / (ROWS / 4), row = r0 + (idx % (ROWS / 4)) * 4;
-                        const float* src = p + (long)k * ld + row;
-                        if (!CHECK || (k < kend && row + 3 < R)) {
-                            const float4u q = *reinterpret_cast<const float4u*>(src);
-                            t[0] = q.x; t[1] = q.y; t[2] = q.z; t[3] = q.w;
-                        } else if (k < kend) {
+        for (int i = 0; i < NV; ++i)
+            if (has(i)) {
+                // the empty asm keeps origin + offset from being hoisted into a per-lane
+                // 64-bit pointer that is then advanced with vector adds every slice
+                asm volatile("" : "+v"(goff[i]));
+                const float4u q = *reinterpret_cast<const float4u*>(origin + goff[i]);
+                v[i * 4] = q.x; v[i * 4 + 1] = q.y; v[i * 4 + 2] = q.z; v[i * 4 + 3] = q.w;
+            }
+    }
+
+    // bounds-tested: rows >= R and k >= kend read as zero
+    __device__ __forceinline__ void load_checked(const float* __restrict__ p, long ld, int r0, int R,
+                                                 int k0, int kend) {
 #pragma unroll
-                            for (int j = 0; j < 4; ++j)
-                                if (row + j < R) t[j] = src[j];
-                        }
+        for (int i = 0; i < NV; ++i) {
+            const int idx = threadIdx.x + i * kGemmThreads;     // float4 index
+            float t[4] = {0.f, 0.f, 0.f, 0.f};
+            if (has(i)) {
+                if (KC) {
+                    const int row = r0 + (idx >> 2), k = k0 + (idx & 3) * 4;
+                    const float* src = p + (long)row * ld + k;
+                    if (row < R && k + 3 < kend) {
+                        const float4u q = *reinterpret_cast<const float4u*>(src);
+                        t[0] = q.x; t[1] = q.y; t[2] = q.z; t[3] = q.w;
+                    } else if (row < R) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            if (k + j < kend) t[j] = src[j];
+                    }
+                } else {
+                    const int k = k0 + idx / (ROWS / 4), row = r0 + (idx % (ROWS / 4)) * 4;
+                    const float* src = p + (long)k * ld + row;
+                    if (k < kend && row + 3 < R) {
+                        const float4u q = *reinterpret_cast<const float4u*>(src);
+                        t[0] = q.x; t[1] = q.y; t[2] = q.z; t[3] = q.w;
+                    } else if (k < kend) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            if (row + j < R) t[j] = src[j];
                     }
                 }
-#pragma unroll
-                for (int j = 0; j < 4; ++j) v[i * 4 + j] = t[j];
             }
-        } else {
 #pragma unroll
-            for (int i = 0; i < kPerThread; ++i) {
-                const int idx = threadIdx.x + i * kGemmThreads;     // element index
-                float t = 0.f;
-                if (idx < kElems) {
-                    if (KC) {
-                        const int row = r0 + (idx >> 4), k = k0 + (idx & 15);
-                        if (!CHECK || (row < R && k < kend)) t = p[(long)row * ld + k];
-                    } else {
-                        const int k = k0 + idx / ROWS, row = r0 + idx % ROWS;
-                        if (!CHECK || (k < kend && row < R)) t = p[(long)k * ld + row];
-                    }
-                }
-                v[i] = t;
-            }
+            for (int j = 0; j < 4; ++j) v[i * 4 + j] = t[j];
         }
     }
 
     __device__ __forceinline__ void store(float* __restrict__ tile) const {
-        if (VEC) {
 #pragma unroll
-            for (int i = 0; i < NV; ++i) {
-                const int idx = threadIdx.x + i * kGemmThreads;
-                if (idx * 4 < kElems) {
-                    float* dst = KC ? tile + (idx >> 2) * LDK + (idx & 3) * 4
-                                    : tile + (idx / (ROWS / 4)) * LDM + (idx % (ROWS / 4)) * 4;
-                    *reinterpret_cast<float4*>(dst) = make_float4(v[i * 4], v[i * 4 + 1], v[i * 4 + 2], v[i * 4 + 3]);
-                }
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < kPerThread; ++i) {
-                const int idx = threadIdx.x + i * kGemmThreads;
-                if (idx < kElems) {
-                    if (KC) tile[(idx >> 4) * LDK + (idx & 15)] = v[i];
-                    else tile[(idx / ROWS) * LDM + idx % ROWS] = v[i];
-                }
+        for (int i = 0; i < NV; ++i) {
+            const int idx = threadIdx.x + i * kGemmThreads;
+            if (has(i)) {
+                float* dst = KC ? tile + (idx >> 2) * LDK + (idx & 3) * 4
+                                : tile + (idx / (ROWS / 4)) * LDM + (idx % (ROWS / 4)) * 4;
+                *reinterpret_cast<float4*>(dst) = make_float4(v[i * 4], v[i * 4 + 1], v[i * 4 + 2], v[i * 4 + 3]);
             }
         }
     }
@@ -189,12 +195,12 @@ __device__ __forceinline__ int xcd_remap(int id, int n) {
 
 // WGM x WGN wavefronts, each TM x TN blocks of 32x32.
 // PIPE selects the software-pipelined main loop (k-contiguous operands only).
-template <bool AKC, bool BKC, bool VECA, bool VECB, bool PIPE, int WGM, int WGN, int TM, int TN>
-__global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
+template <bool AKC, bool BKC, bool PIPE, int WGM, int WGN, int TM, int TN>
+__global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmArgs a) {
     static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
-    typedef OperandTile<AKC, BM, VECA> TileA;
-    typedef OperandTile<BKC, BN, VECB> TileB;
+    typedef OperandTile<AKC, BM> TileA;
+    typedef OperandTile<BKC, BN> TileB;
     __shared__ __attribute__((aligned(16))) float As[2][TileA::kFloats];
     __shared__ __attribute__((aligned(16))) float Bs[2][TileB::kFloats];
 
@@ -292,38 +298,49 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
         __builtin_amdgcn_sched_barrier(0);
     };
 
+    // Loading one K slice of both operands into registers.  MODE kFast: the
+    // whole tile is inside the matrices and the K range is a multiple of the
+    // slice -> fixed offsets from a uniform origin, no tests.  kFastTail: the
+    // same, except that the last slice is ragged and takes the tested loads.
+    // kChecked: edge tile, tested loads throughout.
+    constexpr int kFast = 0, kFastTail = 1, kChecked = 2;
+    const char* originA = reinterpret_cast<const char*>(A + (AKC ? (long)m0 * a.lda + kbeg : (long)kbeg * a.lda + m0));
+    const char* originB = reinterpret_cast<const char*>(B + (BKC ? (long)n0 * a.ldb + kbeg : (long)kbeg * a.ldb + n0));
+    const long stepA = (AKC ? (long)KT : (long)KT * a.lda) * 4, stepB = (BKC ? (long)KT : (long)KT * a.ldb) * 4;
+    auto load_slice = [&](auto mode, TileA& ra, TileB& rb, int slice) {
+        constexpr int MODE = decltype(mode)::value;
+        const int k0 = kbeg + slice * KT;
+        if (MODE == kChecked || (MODE == kFastTail && slice == nk - 1)) {
+            ra.load_checked(A, a.lda, m0, a.M, k0, kend);
+            rb.load_checked(B, a.ldb, n0, a.N, k0, kend);
+        } else {
+            ra.load_fast(originA + slice * stepA);
+            rb.load_fast(originB + slice * stepB);
+        }
+    };
+
     // The pipelined schedule pays off when both operands are k-contiguous
     // (16-byte fragment reads); the other layouts measure faster with the
-    // plain double-buffered loop (one full barrier per slice).
-    // Interior tiles (all of BM x BN inside C, K range a multiple of the slice)
-    // run a copy of the main loop with no bounds tests in its loads.
-    auto main_loop = [&](auto checked) {
-        constexpr bool CHK = decltype(checked)::value;
-        constexpr bool kPipelined = PIPE;
-        if constexpr (kPipelined) {
+    // plain double-buffered loop (one full barrier per slice).  Both loops are
+    // unrolled by two so that the LDS buffer of a slice is a compile-time
+    // constant (fragment and store addresses are then register + immediate).
+    auto main_loop = [&](auto mode) {
+        if constexpr (PIPE) {
             if (nk > 0) {
-                ta.template load<CHK>(A, a.lda, m0, a.M, kbeg, kend);
-                tb.template load<CHK>(B, a.ldb, n0, a.N, kbeg, kend);
+                load_slice(mode, ta, tb, 0);
                 ta.store(As[0]);
                 tb.store(Bs[0]);
-                if (nk > 1) {
-                    ta.template load<CHK>(A, a.lda, m0, a.M, kbeg + KT, kend);
-                    tb.template load<CHK>(B, a.ldb, n0, a.N, kbeg + KT, kend);
-                }
+                if (nk > 1) load_slice(mode, ta, tb, 1);
                 lds_barrier();
                 read_frags(0, As[0], Bs[0], 0);
             }
-            for (int kt = 0; kt < nk; ++kt) {
-                const int cur = kt & 1;
+            auto iteration = [&](int kt, auto curc) {
+                constexpr int cur = decltype(curc)::value;
                 if (kt + 1 < nk) {
                     ta.store(As[cur ^ 1]);       // slice kt+1 (waits for its global loads, issued an iteration ago)
                     tb.store(Bs[cur ^ 1]);
                 }
-                if (kt + 2 < nk) {
-                    const int k0 = kbeg + (kt + 2) * KT;
-                    ta.template load<CHK>(A, a.lda, m0, a.M, k0, kend);
-                    tb.template load<CHK>(B, a.ldb, n0, a.N, k0, kend);
-                }
+                if (kt + 2 < nk) load_slice(mode, ta, tb, kt + 2);
                 read_frags(1, As[cur], Bs[cur], 1);
                 __builtin_amdgcn_s_setprio(3);   // inside the MFMA stream: ahead of wavefronts issuing loads
                 mfma_steps(0, 0, 4);
@@ -331,11 +348,16 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
                 if (kt + 1 < nk) read_frags(0, As[cur ^ 1], Bs[cur ^ 1], 0);
                 mfma_steps(1, 0, 4);
                 __builtin_amdgcn_s_setprio(0);
+            };
+            int kt = 0;
+            for (; kt + 1 < nk; kt += 2) {
+                iteration(kt, std::integral_constant<int, 0>{});
+                iteration(kt + 1, std::integral_constant<int, 1>{});
             }
+            if (kt < nk) iteration(kt, std::integral_constant<int, 0>{});
         } else {
             if (nk > 0) {
-                ta.template load<CHK>(A, a.lda, m0, a.M, kbeg, kend);
-                tb.template load<CHK>(B, a.ldb, n0, a.N, kbeg, kend);
+                load_slice(mode, ta, tb, 0);
                 ta.store(As[0]);
                 tb.store(Bs[0]);
             }
@@ -343,13 +365,9 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
             for (int kt = 0; kt < nk; ++kt) {
                 const int cur = kt & 1;
                 const bool more = kt + 1 < nk;
-                if (more) {
-                    const int k0 = kbeg + (kt + 1) * KT;
-                    ta.template load<CHK>(A, a.lda, m0, a.M, k0, kend);
-                    tb.template load<CHK>(B, a.ldb, n0, a.N, k0, kend);
-                }
+                if (more) load_slice(mode, ta, tb, kt + 1);
                 __builtin_amdgcn_s_setprio(3);
-    #pragma unroll
+#pragma unroll
                 for (int kk = 0; kk < KT / 8; ++kk) {
                     read_frags(0, As[cur], Bs[cur], kk);
                     mfma_steps(0, 0, 4);
@@ -363,9 +381,15 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
             }
         }
     };
-    const bool interior = m0 + BM <= a.M && n0 + BN <= a.N && (kend - kbeg) % KT == 0;
-    if (interior) main_loop(std::false_type{});
-    else main_loop(std::true_type{});
+    const bool inside = m0 + BM <= a.M && n0 + BN <= a.N && !a.wide;
+    if (inside) {
+        ta.init_offsets(a.lda);
+        tb.init_offsets(a.ldb);
+        if ((kend - kbeg) % KT == 0) main_loop(std::integral_constant<int, kFast>{});
+        else main_loop(std::integral_constant<int, kFastTail>{});
+    } else {
+        main_loop(std::integral_constant<int, kChecked>{});
+    }
 
     // accumulator element e of a 32x32 block: row 8*(e/4) + 4*half + e%4, column l32
     if (tail_piece >= 0) {
@@ -388,6 +412,34 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_kernel(GemmArgs a) {
     } else {
         out = a.C + batch * a.sC;
         ldo = a.ldc;
+    }
+    if (m0 + BM <= a.M && n0 + BN <= a.N && ldo < (1L << 27)) {
+        // Whole tile inside C.  A wavefront that is storing shares its SIMD with
+        // wavefronts that are multiplying and gets about one instruction issued
+        // per MFMA of theirs, so the store sequence carries no vector address
+        // arithmetic: row origins are wave-uniform (scalar adds), the lane's
+        // share (its column, its half's 4-row shift) is one fixed 32-bit
+        // offset, the block column an immediate.
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+        const int wm_u = wave_u / WGN, wn_u = wave_u % WGN;
+        char* origin = reinterpret_cast<char*>(out + (long)(m0 + wm_u * TM * 32) * ldo + n0 + wn_u * TN * 32);
+        unsigned lane_off = (unsigned)((4 * half * ldo + l32) * 4);
+        // rows of a lane half: 0,1,2,3, 8,9,10,11, 16,... -> steps of one row, then five
+        const long step1 = ldo * 4, step5 = ldo * 20;
+        char* row = origin;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                // keeps "uniform row origin + lane offset" from being re-associated into
+                // a per-lane 64-bit pointer that is then advanced with vector adds
+                asm volatile("" : "+v"(lane_off));
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    *reinterpret_cast<float*>(row + lane_off + j * 128) = acc[i][j][e];
+                row += (e % 4 == 3) ? step5 : step1;
+            }
+        return;
     }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -538,34 +590,25 @@ struct TileShape {
 // Tile shapes on offer; the 128x128 default comes first and wins ties.
 static const TileShape kShapes[] = {{128, 128}, {128, 96}, {128, 64}, {128, 32}, {96, 128}};
 
-template <bool AKC, bool BKC, bool VECA, bool VECB, bool PIPE>
+template <bool AKC, bool BKC, bool PIPE>
 static void launch_shape(int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
     dim3 block(kGemmThreads);
     switch (shape) {
-        case 0: sgemm_kernel<AKC, BKC, VECA, VECB, PIPE, 2, 2, 2, 2><<<grid, block, 0, st>>>(a); break;
-        case 1: sgemm_kernel<AKC, BKC, VECA, VECB, PIPE, 4, 1, 1, 3><<<grid, block, 0, st>>>(a); break;
-        case 2: sgemm_kernel<AKC, BKC, VECA, VECB, PIPE, 4, 1, 1, 2><<<grid, block, 0, st>>>(a); break;
-        case 3: sgemm_kernel<AKC, BKC, VECA, VECB, PIPE, 4, 1, 1, 1><<<grid, block, 0, st>>>(a); break;
-        default: sgemm_kernel<AKC, BKC, VECA, VECB, PIPE, 1, 4, 3, 1><<<grid, block, 0, st>>>(a); break;
+        case 0: sgemm_kernel<AKC, BKC, PIPE, 2, 2, 2, 2><<<grid, block, 0, st>>>(a); break;
+        case 1: sgemm_kernel<AKC, BKC, PIPE, 4, 1, 1, 3><<<grid, block, 0, st>>>(a); break;
+        case 2: sgemm_kernel<AKC, BKC, PIPE, 4, 1, 1, 2><<<grid, block, 0, st>>>(a); break;
+        case 3: sgemm_kernel<AKC, BKC, PIPE, 4, 1, 1, 1><<<grid, block, 0, st>>>(a); break;
+        default: sgemm_kernel<AKC, BKC, PIPE, 1, 4, 3, 1><<<grid, block, 0, st>>>(a); break;
     }
 }
 
-// Both operands always take the 16-byte load path: it needs 4-byte alignment
-// only (float4u), so odd leading dimensions (Z = 363, 75) qualify too; measured
-// 8-34 % faster than coalesced 4-byte loads on such shapes.  The 4-byte variants
-// of OperandTile remain for reference and are not instantiated.
-template <bool AKC, bool BKC, bool PIPE>
-static void launch_vec(int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
-    launch_shape<AKC, BKC, true, true, PIPE>(shape, grid, st, a);
-}
-
 static void launch_trans(int tA, int tB, bool pipe, int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
-    if (!tA && !tB) launch_vec<true, false, false>(shape, grid, st, a);
+    if (!tA && !tB) launch_shape<true, false, false>(shape, grid, st, a);
     else if (!tA && tB) {
-        if (pipe) launch_vec<true, true, true>(shape, grid, st, a);
-        else launch_vec<true, true, false>(shape, grid, st, a);
-    } else if (tA && !tB) launch_vec<false, false, false>(shape, grid, st, a);
-    else launch_vec<false, true, false>(shape, grid, st, a);
+        if (pipe) launch_shape<true, true, true>(shape, grid, st, a);
+        else launch_shape<true, true, false>(shape, grid, st, a);
+    } else if (tA && !tB) launch_shape<false, false, false>(shape, grid, st, a);
+    else launch_shape<false, true, false>(shape, grid, st, a);
 }
 
 static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const float* A, long lda,
@@ -603,6 +646,7 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     a.splits = 1;
     a.kchunk = (int)(cdiv(std::max(K, 1L), KT) * KT);
     a.ws = nullptr;
+    a.wide = (lda >= (1L << 23) || ldb >= (1L << 23)) ? 1 : 0;
     if (P == 1 && tiles < 512 && K >= 64 * KT) {
         long want = std::max(1L, 1024 / tiles);
         want = std::min(want, K / (8 * KT));                    // at least 8 slices per split

@@ -52,6 +52,46 @@ def test_gemm_with_k_zero_writes_zeros(L):
     assert np.array_equal(c.get(), np.zeros((5, 7), np.float32))
 
 
+@pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_gemm_with_huge_leading_dimension(L, tA, tB):
+    # rows 2^23 floats apart: the 32-bit tile offsets of the steady-state loads do not
+    # reach, so every tile has to take the 64-bit tested loads; results must not change
+    ld = 1 << 23
+    M, N, K = 130, 140, 37
+    rs = np.random.RandomState(5)
+    a = rs.uniform(-1, 1, (K, M) if tA else (M, K)).astype(np.float32)
+    b = rs.uniform(-1, 1, (N, K) if tB else (K, N)).astype(np.float32)
+    wide_a = np.zeros((a.shape[0], ld), np.float32)
+    wide_a[:, :a.shape[1]] = a
+    ga, gb = gpu(wide_a), gpu(b)
+    del wide_a
+    c = gpu(np.zeros((M, N), np.float32))
+    assert L.cgt_amd_sgemm(tA, tB, M, N, K, ga.ptr, ld, gb.ptr, b.shape[1], c.ptr, N, None) == OK
+    ref = (a.T if tA else a).astype(np.float64) @ (b.T if tB else b).astype(np.float64)
+    err = np.linalg.norm(c.get() - ref) / np.linalg.norm(ref)
+    assert err <= 1e-4     # relative Frobenius bar of the GEMM tests
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 16 * 9 + 5), (128, 96, 363), (384, 128, 11), (128, 128, 16)])
+@pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_gemm_whole_tiles_with_ragged_k(L, M, N, K, tA, tB):
+    # every tile is inside C, so the untested loads run for all full K slices and only
+    # the last, ragged slice is bounds-tested; memory right behind the operands is
+    # poisoned with NaN so a read past a row end that reached the sum would show
+    rs = np.random.RandomState(M + N + K)
+    a = rs.uniform(-1, 1, (K, M) if tA else (M, K)).astype(np.float32)
+    b = rs.uniform(-1, 1, (N, K) if tB else (K, N)).astype(np.float32)
+    pad = np.full(64, np.nan, np.float32)
+    ga = gpu(np.concatenate([a.ravel(), pad]))
+    gb = gpu(np.concatenate([b.ravel(), pad]))
+    c = gpu(np.zeros((M, N), np.float32))
+    assert L.cgt_amd_sgemm(tA, tB, M, N, K, ga.ptr, a.shape[1], gb.ptr, b.shape[1], c.ptr, N, None) == OK
+    ref = (a.T if tA else a).astype(np.float64) @ (b.T if tB else b).astype(np.float64)
+    out = c.get()
+    assert np.isfinite(out).all()
+    assert np.linalg.norm(out - ref) / np.linalg.norm(ref) <= 1e-4
+
+
 @pytest.mark.parametrize("call,needle", [
     (lambda L, p: L.cgt_amd_im2col_f32(p, 1, 1, 2, 2, 5, 5, 0, 0, 1, 1, p, None), "kernel larger"),
     (lambda L, p: L.cgt_amd_im2col_f32(p, 1, 1, 8, 8, 3, 3, 0, 0, 0, 1, p, None), "geometry"),

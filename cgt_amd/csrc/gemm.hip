@@ -299,31 +299,39 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
     };
 
     // Loading one K slice of both operands into registers.  MODE kFast: the
-    // whole tile is inside the matrices and the K range is a multiple of the
-    // slice -> fixed offsets from a uniform origin, no tests.  kFastTail: the
-    // same, except that the last slice is ragged and takes the tested loads.
-    // kChecked: edge tile, tested loads throughout.
-    constexpr int kFast = 0, kFastTail = 1, kChecked = 2;
+    // whole tile is inside both matrices and the K range is a multiple of the
+    // slice -> fixed offsets from a uniform origin, no tests.  kMixed: each
+    // operand on its own takes the untested loads where its side of the tile is
+    // whole (an edge tile in N still streams A untested) and the tested ones
+    // otherwise; a ragged last K slice is tested for both.
+    constexpr int kFast = 0, kMixed = 1;
+    const bool wholeA = m0 + BM <= a.M && !a.wide, wholeB = n0 + BN <= a.N && !a.wide;
+    const bool ragged_k = (kend - kbeg) % KT != 0;
     const char* originA = reinterpret_cast<const char*>(A + (AKC ? (long)m0 * a.lda + kbeg : (long)kbeg * a.lda + m0));
     const char* originB = reinterpret_cast<const char*>(B + (BKC ? (long)n0 * a.ldb + kbeg : (long)kbeg * a.ldb + n0));
     const long stepA = (AKC ? (long)KT : (long)KT * a.lda) * 4, stepB = (BKC ? (long)KT : (long)KT * a.ldb) * 4;
     auto load_slice = [&](auto mode, TileA& ra, TileB& rb, int slice) {
         constexpr int MODE = decltype(mode)::value;
-        const int k0 = kbeg + slice * KT;
-        if (MODE == kChecked || (MODE == kFastTail && slice == nk - 1)) {
-            ra.load_checked(A, a.lda, m0, a.M, k0, kend);
-            rb.load_checked(B, a.ldb, n0, a.N, k0, kend);
-        } else {
+        if (MODE == kFast) {
             ra.load_fast(originA + slice * stepA);
             rb.load_fast(originB + slice * stepB);
+        } else {
+            const int k0 = kbeg + slice * KT;
+            const bool tested = ragged_k && slice == nk - 1;
+            if (wholeA && !tested) ra.load_fast(originA + slice * stepA);
+            else ra.load_checked(A, a.lda, m0, a.M, k0, kend);
+            if (wholeB && !tested) rb.load_fast(originB + slice * stepB);
+            else rb.load_checked(B, a.ldb, n0, a.N, k0, kend);
         }
     };
 
     // The pipelined schedule pays off when both operands are k-contiguous
     // (16-byte fragment reads); the other layouts measure faster with the
-    // plain double-buffered loop (one full barrier per slice).  Both loops are
-    // unrolled by two so that the LDS buffer of a slice is a compile-time
-    // constant (fragment and store addresses are then register + immediate).
+    // plain double-buffered loop (one full barrier per slice).  The pipelined
+    // loop is unrolled by two so that the LDS buffer of a slice is a
+    // compile-time constant (fragment and store addresses are then register +
+    // immediate); the plain one is not: unrolled, it needs more than the 128
+    // registers that let four workgroups share a CU.
     auto main_loop = [&](auto mode) {
         if constexpr (PIPE) {
             if (nk > 0) {
@@ -381,78 +389,65 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
             }
         }
     };
-    const bool inside = m0 + BM <= a.M && n0 + BN <= a.N && !a.wide;
-    if (inside) {
-        ta.init_offsets(a.lda);
-        tb.init_offsets(a.ldb);
-        if ((kend - kbeg) % KT == 0) main_loop(std::integral_constant<int, kFast>{});
-        else main_loop(std::integral_constant<int, kFastTail>{});
-    } else {
-        main_loop(std::integral_constant<int, kChecked>{});
-    }
+    if (wholeA) ta.init_offsets(a.lda);
+    if (wholeB) tb.init_offsets(a.ldb);
+    if (wholeA && wholeB && !ragged_k) main_loop(std::integral_constant<int, kFast>{});
+    else main_loop(std::integral_constant<int, kMixed>{});
 
-    // accumulator element e of a 32x32 block: row 8*(e/4) + 4*half + e%4, column l32
-    if (tail_piece >= 0) {
-        // tile-local [BM][BN] piece, no bounds: the reduction clips
-        float* out = a.ws + (long)tail_piece * (BM * BN);
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int e = 0; e < 16; ++e)
-                    out[((wm * TM + i) * 32 + 8 * (e / 4) + 4 * half + (e % 4)) * BN + (wn * TN + j) * 32 + l32] = acc[i][j][e];
-        return;
-    }
+    // accumulator element e of a 32x32 block: row 8*(e/4) + 4*half + e%4, column l32.
+    // Destination: C, this split's partial matrix, or (tail pieces) a tile-local
+    // [BM][BN] block that is written whole -- the reduction clips.
     float* out;
     long ldo;
-    if (a.splits > 1) {
+    int out_m0 = m0, out_n0 = n0, out_M = a.M, out_N = a.N;
+    if (tail_piece >= 0) {
+        out = a.ws + (long)tail_piece * (BM * BN);
+        ldo = BN;
+        out_m0 = 0; out_n0 = 0; out_M = BM; out_N = BN;
+    } else if (a.splits > 1) {
         out = a.ws + (long)split * a.M * a.N;
         ldo = a.N;
     } else {
         out = a.C + batch * a.sC;
         ldo = a.ldc;
     }
-    if (m0 + BM <= a.M && n0 + BN <= a.N && ldo < (1L << 27)) {
-        // Whole tile inside C.  A wavefront that is storing shares its SIMD with
-        // wavefronts that are multiplying and gets about one instruction issued
-        // per MFMA of theirs, so the store sequence carries no vector address
-        // arithmetic: row origins are wave-uniform (scalar adds), the lane's
-        // share (its column, its half's 4-row shift) is one fixed 32-bit
-        // offset, the block column an immediate.
+    // A wavefront that is storing shares its SIMD with wavefronts that are
+    // multiplying and gets about one instruction issued per MFMA of theirs, so the
+    // store sequence carries no vector address arithmetic: row origins are
+    // wave-uniform (scalar adds), the lane's share (its column, its half's 4-row
+    // shift) is one fixed 32-bit offset, the block column an immediate.  Edge
+    // tiles mask lanes by comparing the compile-time row / column of a store with
+    // the lane's count of rows / columns left in C.
+    {
         const int wave_u = __builtin_amdgcn_readfirstlane(wave);
         const int wm_u = wave_u / WGN, wn_u = wave_u % WGN;
-        char* origin = reinterpret_cast<char*>(out + (long)(m0 + wm_u * TM * 32) * ldo + n0 + wn_u * TN * 32);
+        const int r0 = out_m0 + wm_u * TM * 32, c0 = out_n0 + wn_u * TN * 32;
+        char* row = reinterpret_cast<char*>(out + (long)r0 * ldo + c0);
         unsigned lane_off = (unsigned)((4 * half * ldo + l32) * 4);
         // rows of a lane half: 0,1,2,3, 8,9,10,11, 16,... -> steps of one row, then five
         const long step1 = ldo * 4, step5 = ldo * 20;
-        char* row = origin;
+        const bool whole = out_m0 + BM <= out_M && out_n0 + BN <= out_N;
+        const int rows_left = out_M - r0 - 4 * half, cols_left = out_N - c0 - l32;   // of this lane
+        auto store_rows = [&](auto wholec) {
+            constexpr bool WHOLE = decltype(wholec)::value;
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                // keeps "uniform row origin + lane offset" from being re-associated into
-                // a per-lane 64-bit pointer that is then advanced with vector adds
-                asm volatile("" : "+v"(lane_off));
+                for (int e = 0; e < 16; ++e) {
+                    // keeps "uniform row origin + lane offset" from being re-associated into
+                    // a per-lane 64-bit pointer that is then advanced with vector adds
+                    asm volatile("" : "+v"(lane_off));
+                    const int r = i * 32 + 8 * (e / 4) + (e % 4);
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    *reinterpret_cast<float*>(row + lane_off + j * 128) = acc[i][j][e];
-                row += (e % 4 == 3) ? step5 : step1;
-            }
-        return;
+                    for (int j = 0; j < TN; ++j)
+                        if (WHOLE || (r < rows_left && j * 32 < cols_left))
+                            *reinterpret_cast<float*>(row + lane_off + j * 128) = acc[i][j][e];
+                    row += (e % 4 == 3) ? step5 : step1;
+                }
+        };
+        if (whole) store_rows(std::true_type{});
+        else store_rows(std::false_type{});
     }
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int col = n0 + (wn * TN + j) * 32 + l32;
-            if (col >= a.N) continue;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int row = m0 + (wm * TM + i) * 32 + 8 * (e / 4) + 4 * half + (e % 4);
-                if (row < a.M) out[(long)row * ldo + col] = acc[i][j][e];
-            }
-        }
 }
 
 // Tail tiles: C tile = sum over its K pieces, in order.  blockIdx.y = tail tile,
@@ -621,6 +616,7 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     CGT_ARG_CHECK(C, "sgemm: null C");
     CGT_ARG_CHECK(M < (1L << 31) - 128 && N < (1L << 31) - 128 && K < (1L << 31) - KT && P < 65536,
                   "sgemm: size too large");
+    CGT_ARG_CHECK(ldc < (1L << 27) || M <= 4, "sgemm: ldc >= 2^27 with more than 4 rows is not supported");
     CGT_ARG_CHECK(lda >= (tA ? M : K) && ldb >= (tB ? K : N) && ldc >= N,
                   "sgemm: leading dimension too small (lda=%ld ldb=%ld ldc=%ld)", lda, ldb, ldc);
     // tile shape: least padded work, ties to the earlier (larger) shape

@@ -229,6 +229,17 @@ class LayerOnGpu(object):
                 st.fn()
             e1.record(self.stream)
             st.ms = e0.elapsed_ms(e1) / reps
+            # the same launches once more with an event after each one: median and
+            # minimum of the individual durations (each includes the gap to the
+            # previous launch, a few microseconds)
+            ev = [capi.Event() for _ in range(reps + 1)]
+            ev[0].record(self.stream)
+            for i in range(reps):
+                st.fn()
+                ev[i + 1].record(self.stream)
+            capi.synchronize()
+            each = sorted(ev[i].elapsed_ms(ev[i + 1]) for i in range(reps))
+            st.ms_median, st.ms_min = each[len(each) // 2], each[0]
 
 
 class GemmOnGpu(object):
@@ -422,7 +433,8 @@ def main():
     gemm_flops = gemm_ms = 0.0
     dominant = max((st for st in layer.stages if st.bound == "mfma"), key=lambda st: st.ms)
     for st in layer.stages:
-        row = {"stage": st.name, "kernel": st.kernel, "ms": round(st.ms, 4), "bound": st.bound}
+        row = {"stage": st.name, "kernel": st.kernel, "ms": round(st.ms, 4), "ms_median": round(st.ms_median, 4),
+               "ms_min": round(st.ms_min, 4), "bound": st.bound}
         if st.bound == "hbm":
             gbs = st.work / (st.ms * 1e-3) / 1e9
             row.update(bytes=st.work, GBps=round(gbs, 1), frac=round(gbs / HBM_PEAK_GBS, 4))

@@ -72,6 +72,50 @@ def test_gemm_with_huge_leading_dimension(L, tA, tB):
     assert err <= 1e-4     # relative Frobenius bar of the GEMM tests
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 260, 70),        # whole and edge tiles
+                                   (2100, 2100, 300),     # 289 tiles: the last partial round is cut along K
+                                   (100, 200, 5000),      # few tiles, long K: split along K
+                                   (1024, 96, 363)])      # 128x96 tiles, ragged K
+@pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_gemm_with_padded_leading_dimensions(L, M, N, K, tA, tB):
+    # operands and result live inside wider arrays: rows are lda / ldb / ldc apart, the
+    # columns beyond the matrices hold NaN (operands) or a sentinel (result) and must
+    # neither reach the sums nor be written
+    rs = np.random.RandomState(M * 7 + N * 3 + K + tA * 2 + tB)
+    pa, pb, pc = 5, 9, 13
+    a = rs.uniform(-1, 1, (K, M) if tA else (M, K)).astype(np.float32)
+    b = rs.uniform(-1, 1, (N, K) if tB else (K, N)).astype(np.float32)
+    wa = np.full((a.shape[0], a.shape[1] + pa), np.nan, np.float32)
+    wa[:, :a.shape[1]] = a
+    wb = np.full((b.shape[0], b.shape[1] + pb), np.nan, np.float32)
+    wb[:, :b.shape[1]] = b
+    wc = np.full((M, N + pc), -7.0, np.float32)
+    ga, gb, gc = gpu(wa), gpu(wb), gpu(wc)
+    assert L.cgt_amd_sgemm(tA, tB, M, N, K, ga.ptr, wa.shape[1], gb.ptr, wb.shape[1], gc.ptr, N + pc, None) == OK
+    out = gc.get()
+    ref = (a.T if tA else a).astype(np.float64) @ (b.T if tB else b).astype(np.float64)
+    assert np.array_equal(out[:, N:], np.full((M, pc), -7.0, np.float32))
+    assert np.linalg.norm(out[:, :N] - ref) / np.linalg.norm(ref) <= 1e-4
+
+
+def test_batched_gemm_with_strides_and_shared_operand(L):
+    # batch strides larger than the matrices, and a batch stride of zero (one operand
+    # shared by every product, as a conv layer's filters would be)
+    rs = np.random.RandomState(11)
+    P, M, N, K = 5, 150, 70, 45
+    a = rs.uniform(-1, 1, (M, K)).astype(np.float32)
+    b = rs.uniform(-1, 1, (P, K + 2, N + 3)).astype(np.float32)      # each product uses b[p, :K, :N]
+    c = np.full((P, M + 1, N + 4), 3.0, np.float32)
+    ga, gb, gc = gpu(a), gpu(b), gpu(c)
+    assert L.cgt_amd_sgemm_batched(0, 0, P, M, N, K, ga.ptr, K, 0, gb.ptr, N + 3, (K + 2) * (N + 3),
+                                   gc.ptr, N + 4, (M + 1) * (N + 4), None) == OK
+    out = gc.get()
+    for p in range(P):
+        ref = a.astype(np.float64) @ b[p, :K, :N].astype(np.float64)
+        assert np.linalg.norm(out[p, :M, :N] - ref) / np.linalg.norm(ref) <= 1e-4
+    assert np.all(out[:, M:, :] == 3.0) and np.all(out[:, :, N:] == 3.0)
+
+
 @pytest.mark.parametrize("M,N,K", [(256, 256, 16 * 9 + 5), (128, 96, 363), (384, 128, 11), (128, 128, 16)])
 @pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
 def test_gemm_whole_tiles_with_ragged_k(L, M, N, K, tA, tB):

@@ -579,12 +579,25 @@ static int launch_im2col(G g, const float* im, long B, int C, int H, int W, int 
                     break;
                 }
         }
+        // all channels in one 32 KiB buffer, if two 24 KiB ones would need a second pass:
+        // a pixel's whole row of the column buffer is then written in one go (AlexNet
+        // conv1: 3 x 11 x 227 floats = 30 KB; 1452-byte rows written once instead of as
+        // 968 + 484 bytes in two phases that meet again only in L2 -- or not)
+        const bool whole = chunk < C && C * rowlen <= 32 * kIm2colThreads;
+        if (whole) {
+            chunk = C;
+            vec = aligned;
+        }
         const int nchunks = (int)cdiv(C, chunk);
-        const size_t lds = 2 * (size_t)chunk * rowlen * sizeof(float);
+        const size_t lds = (nchunks > 1 ? 2 : 1) * (size_t)chunk * rowlen * sizeof(float);
         const long blocks = B * m;
         const bool small = (long)chunk * rowlen <= 12 * kIm2colThreads;
         dim3 grid((unsigned)blocks), block(kIm2colThreads);
-        if (vec && small)
+        if (whole && vec)
+            im2col_pipe_kernel<G, true, 32><<<grid, block, lds, st>>>(g, im, col, C, H, W, m, n, chunk, nchunks);
+        else if (whole)
+            im2col_pipe_kernel<G, false, 32><<<grid, block, lds, st>>>(g, im, col, C, H, W, m, n, chunk, nchunks);
+        else if (vec && small)
             im2col_pipe_kernel<G, true, 12><<<grid, block, lds, st>>>(g, im, col, C, H, W, m, n, chunk, nchunks);
         else if (vec)
             im2col_pipe_kernel<G, true, 24><<<grid, block, lds, st>>>(g, im, col, C, H, W, m, n, chunk, nchunks);

@@ -29,6 +29,14 @@
 // im2col buffers of the AlexNet and CIFAR layers have Z = 363 or 75 floats per
 // row: global_load_dwordx4 does not need more alignment than a float's).
 //
+// fp32 MFMAs and other vector instructions do not overlap on a SIMD of this
+// chip, and a wavefront that is loading or storing while its neighbours
+// multiply is issued about one instruction per MFMA of theirs.  The steady
+// state therefore avoids vector address arithmetic altogether: loads and C
+// stores are "wave-uniform origin (scalar registers, advanced with scalar
+// adds) + one fixed 32-bit offset per lane (+ immediate)", bounds tests run
+// only on edge tiles and on a ragged last K slice.
+//
 // Skinny outputs (few tiles, long K: the conv weight gradient) are split along
 // K into a workspace of partial tiles, reduced afterwards in a fixed order, so
 // the result is deterministic.  The grid is one-dimensional and ordered so
@@ -694,10 +702,10 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     CGT_ARG_CHECK(wgs < (1L << 31), "sgemm: too many workgroups");
     hipStream_t st = as_stream(stream);
     dim3 grid((unsigned)wgs);
-    // The pipelined loop needs ~134 registers (3 workgroups per CU instead of 4):
-    // it wins once every CU has more than a handful of tiles to work through and
-    // loses when the whole product is one round of resident workgroups
-    // (4096^3: 1024 tiles = 4 per CU).
+    // The pipelined loop needs up to ~140 registers in its 128x128 form (3 workgroups
+    // per CU instead of 4): it is used once every CU has more than a handful of tiles
+    // to work through, not when the whole product is one round of resident
+    // workgroups (4096^3: 1024 tiles = 4 per CU).
     const bool pipe = tiles * P >= 5L * kNumCU;
     launch_trans(tA, tB, pipe, shape, grid, st, a);
     CGT_LAUNCH_CHECK("sgemm_kernel");

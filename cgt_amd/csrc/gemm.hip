@@ -203,7 +203,8 @@ __device__ __forceinline__ int xcd_remap(int id, int n) {
 
 // WGM x WGN wavefronts, each TM x TN blocks of 32x32.
 // PIPE selects the software-pipelined main loop (k-contiguous operands only).
-template <bool AKC, bool BKC, bool PIPE, int WGM, int WGN, int TM, int TN>
+// DEEP (plain loop only) keeps two K slices of global loads in flight instead of one.
+template <bool AKC, bool BKC, bool PIPE, int WGM, int WGN, int TM, int TN, bool DEEP = false>
 __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmArgs a) {
     static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
@@ -372,28 +373,68 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
             }
             if (kt < nk) iteration(kt, std::integral_constant<int, 0>{});
         } else {
-            if (nk > 0) {
-                load_slice(mode, ta, tb, 0);
-                ta.store(As[0]);
-                tb.store(Bs[0]);
-            }
-            __syncthreads();
-            for (int kt = 0; kt < nk; ++kt) {
-                const int cur = kt & 1;
-                const bool more = kt + 1 < nk;
-                if (more) load_slice(mode, ta, tb, kt + 1);
-                __builtin_amdgcn_s_setprio(3);
-#pragma unroll
-                for (int kk = 0; kk < KT / 8; ++kk) {
-                    read_frags(0, As[cur], Bs[cur], kk);
-                    mfma_steps(0, 0, 4);
-                }
-                __builtin_amdgcn_s_setprio(0);
-                if (more) {
-                    ta.store(As[cur ^ 1]);
-                    tb.store(Bs[cur ^ 1]);
+            if constexpr (DEEP) {
+                // Two register sets: the loads of slices kt+1 and kt+2 are in flight while
+                // slice kt is multiplied.  Pays when the whole product is one round of
+                // resident workgroups that start together and therefore load in bursts
+                // (4096^3: +5 %); costs a longer prologue, so it is not used for short K.
+                TileA ta1 = ta;
+                TileB tb1 = tb;
+                if (nk > 0) {
+                    load_slice(mode, ta, tb, 0);
+                    if (nk > 1) load_slice(mode, ta1, tb1, 1);
+                    ta.store(As[0]);
+                    tb.store(Bs[0]);
+                    if (nk > 2) load_slice(mode, ta, tb, 2);
                 }
                 __syncthreads();
+                // iteration kt: pa/pb hold slice kt+1, the other set slice kt+2
+                auto iteration = [&](int kt, TileA& pa, TileB& pb) {
+                    const int cur = kt & 1;
+                    __builtin_amdgcn_s_setprio(3);
+#pragma unroll
+                    for (int kk = 0; kk < KT / 8; ++kk) {
+                        read_frags(0, As[cur], Bs[cur], kk);
+                        mfma_steps(0, 0, 4);
+                    }
+                    __builtin_amdgcn_s_setprio(0);
+                    if (kt + 1 < nk) {
+                        pa.store(As[cur ^ 1]);
+                        pb.store(Bs[cur ^ 1]);
+                    }
+                    if (kt + 3 < nk) load_slice(mode, pa, pb, kt + 3);
+                    __syncthreads();
+                };
+                int kt = 0;
+                for (; kt + 1 < nk; kt += 2) {
+                    iteration(kt, ta1, tb1);
+                    iteration(kt + 1, ta, tb);
+                }
+                if (kt < nk) iteration(kt, ta1, tb1);
+            } else {
+                if (nk > 0) {
+                    load_slice(mode, ta, tb, 0);
+                    ta.store(As[0]);
+                    tb.store(Bs[0]);
+                }
+                __syncthreads();
+                for (int kt = 0; kt < nk; ++kt) {
+                    const int cur = kt & 1;
+                    const bool more = kt + 1 < nk;
+                    if (more) load_slice(mode, ta, tb, kt + 1);
+                    __builtin_amdgcn_s_setprio(3);
+#pragma unroll
+                    for (int kk = 0; kk < KT / 8; ++kk) {
+                        read_frags(0, As[cur], Bs[cur], kk);
+                        mfma_steps(0, 0, 4);
+                    }
+                    __builtin_amdgcn_s_setprio(0);
+                    if (more) {
+                        ta.store(As[cur ^ 1]);
+                        tb.store(Bs[cur ^ 1]);
+                    }
+                    __syncthreads();
+                }
             }
         }
     };
@@ -605,7 +646,14 @@ static void launch_shape(int shape, dim3 grid, hipStream_t st, const GemmArgs& a
     }
 }
 
-static void launch_trans(int tA, int tB, bool pipe, int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
+static void launch_trans(int tA, int tB, bool pipe, bool deep, int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
+    dim3 block(kGemmThreads);
+    if (deep) {     // 128x128 tiles, plain loop, not NT (there the second register set spills)
+        if (!tA && !tB) sgemm_kernel<true, false, false, 2, 2, 2, 2, true><<<grid, block, 0, st>>>(a);
+        else if (tA && !tB) sgemm_kernel<false, false, false, 2, 2, 2, 2, true><<<grid, block, 0, st>>>(a);
+        else sgemm_kernel<false, true, false, 2, 2, 2, 2, true><<<grid, block, 0, st>>>(a);
+        return;
+    }
     if (!tA && !tB) launch_shape<true, false, false>(shape, grid, st, a);
     else if (!tA && tB) {
         if (pipe) launch_shape<true, true, true>(shape, grid, st, a);
@@ -707,7 +755,11 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     // to work through, not when the whole product is one round of resident
     // workgroups (4096^3: 1024 tiles = 4 per CU).
     const bool pipe = tiles * P >= 5L * kNumCU;
-    launch_trans(tA, tB, pipe, shape, grid, st, a);
+    // two slices of loads in flight: one round of resident workgroups (they start together
+    // and load in bursts) with a long K range each
+    const long slices = cdiv(a.splits > 1 ? (long)a.kchunk : K, KT);
+    const bool deep = shape == 0 && !(!tA && tB) && wgs <= 4L * kNumCU && slices >= 32;
+    launch_trans(tA, tB, pipe, deep, shape, grid, st, a);
     CGT_LAUNCH_CHECK("sgemm_kernel");
     if (a.splits > 1) {
         const long MN = M * N;

@@ -118,14 +118,16 @@ struct OperandTile {
     }
 
     // the whole tile slice is in range: origin = address of tile element (0, 0) of this slice
-    __device__ __forceinline__ void load_fast(const char* __restrict__ origin) {
+    // `offs`: the goff of the operand's first register set (a second set, used for deeper
+    // prefetch, shares it instead of holding a copy in four more registers)
+    __device__ __forceinline__ void load_fast(const char* __restrict__ origin, unsigned (&offs)[NV]) {
 #pragma unroll
         for (int i = 0; i < NV; ++i)
             if (has(i)) {
                 // the empty asm keeps origin + offset from being hoisted into a per-lane
                 // 64-bit pointer that is then advanced with vector adds every slice
-                asm volatile("" : "+v"(goff[i]));
-                const float4u q = *reinterpret_cast<const float4u*>(origin + goff[i]);
+                asm volatile("" : "+v"(offs[i]));
+                const float4u q = *reinterpret_cast<const float4u*>(origin + offs[i]);
                 v[i * 4] = q.x; v[i * 4 + 1] = q.y; v[i * 4 + 2] = q.z; v[i * 4 + 3] = q.w;
             }
     }
@@ -322,14 +324,14 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
     auto load_slice = [&](auto mode, TileA& ra, TileB& rb, int slice) {
         constexpr int MODE = decltype(mode)::value;
         if (MODE == kFast) {
-            ra.load_fast(originA + slice * stepA);
-            rb.load_fast(originB + slice * stepB);
+            ra.load_fast(originA + slice * stepA, ta.goff);
+            rb.load_fast(originB + slice * stepB, tb.goff);
         } else {
             const int k0 = kbeg + slice * KT;
             const bool tested = ragged_k && slice == nk - 1;
-            if (wholeA && !tested) ra.load_fast(originA + slice * stepA);
+            if (wholeA && !tested) ra.load_fast(originA + slice * stepA, ta.goff);
             else ra.load_checked(A, a.lda, m0, a.M, k0, kend);
-            if (wholeB && !tested) rb.load_fast(originB + slice * stepB);
+            if (wholeB && !tested) rb.load_fast(originB + slice * stepB, tb.goff);
             else rb.load_checked(B, a.ldb, n0, a.N, k0, kend);
         }
     };
@@ -378,8 +380,8 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                 // slice kt is multiplied.  Pays when the whole product is one round of
                 // resident workgroups that start together and therefore load in bursts
                 // (4096^3: +5 %); costs a longer prologue, so it is not used for short K.
-                TileA ta1 = ta;
-                TileB tb1 = tb;
+                TileA ta1;
+                TileB tb1;
                 if (nk > 0) {
                     load_slice(mode, ta, tb, 0);
                     if (nk > 1) load_slice(mode, ta1, tb1, 1);

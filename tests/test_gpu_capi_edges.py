@@ -116,7 +116,10 @@ def test_batched_gemm_with_strides_and_shared_operand(L):
     assert np.all(out[:, M:, :] == 3.0) and np.all(out[:, :, N:] == 3.0)
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 256, 16 * 9 + 5), (128, 96, 363), (384, 128, 11), (128, 128, 16)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 16 * 9 + 5), (128, 96, 363), (384, 128, 11), (128, 128, 16),
+                                   # one round of workgroups with >= 32 K slices each: the loop that keeps
+                                   # two slices of loads in flight (whole slices only / ragged last slice)
+                                   (512, 384, 640), (512, 384, 16 * 40 + 5)])
 @pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
 def test_gemm_whole_tiles_with_ragged_k(L, M, N, K, tA, tB):
     # every tile is inside C, so the untested loads run for all full K slices and only

@@ -75,7 +75,8 @@ def test_gemm_with_huge_leading_dimension(L, tA, tB):
 @pytest.mark.parametrize("M,N,K", [(300, 260, 70),        # whole and edge tiles
                                    (2100, 2100, 300),     # 289 tiles: the last partial round is cut along K
                                    (100, 200, 5000),      # few tiles, long K: split along K
-                                   (1024, 96, 363)])      # 128x96 tiles, ragged K
+                                   (1024, 96, 363),       # 128x96 tiles, ragged K
+                                   (600, 500, 700)])      # edge tiles in the two-slices-in-flight loop
 @pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
 def test_gemm_with_padded_leading_dimensions(L, M, N, K, tA, tB):
     # operands and result live inside wider arrays: rows are lda / ldb / ldc apart, the

@@ -5,7 +5,7 @@
 // accumulate, 16 accumulator registers per block and lane).  The default is
 // 128x128 with 2x2 wavefronts of 2x2 blocks; narrow outputs (the conv GEMMs
 // have N = 32 / 64 / 96 filters, or M = 96 for the weight gradient) use
-// 128 x {32,64,96} with the wavefronts stacked along M, or 96 x 128 with the
+// 128 x {32,64,96} with the wavefronts stacked along M, or {64,96} x 128 with the
 // wavefronts stacked along N, so no matrix-core work is spent on padding.
 //
 // K is walked in slices of 16 through double-buffered LDS tiles: while the
@@ -634,7 +634,7 @@ struct TileShape {
 };
 
 // Tile shapes on offer; the 128x128 default comes first and wins ties.
-static const TileShape kShapes[] = {{128, 128}, {128, 96}, {128, 64}, {128, 32}, {96, 128}};
+static const TileShape kShapes[] = {{128, 128}, {128, 96}, {128, 64}, {128, 32}, {96, 128}, {64, 128}};
 
 template <bool AKC, bool BKC, bool PIPE>
 static void launch_shape(int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
@@ -644,7 +644,8 @@ static void launch_shape(int shape, dim3 grid, hipStream_t st, const GemmArgs& a
         case 1: sgemm_kernel<AKC, BKC, PIPE, 4, 1, 1, 3><<<grid, block, 0, st>>>(a); break;
         case 2: sgemm_kernel<AKC, BKC, PIPE, 4, 1, 1, 2><<<grid, block, 0, st>>>(a); break;
         case 3: sgemm_kernel<AKC, BKC, PIPE, 4, 1, 1, 1><<<grid, block, 0, st>>>(a); break;
-        default: sgemm_kernel<AKC, BKC, PIPE, 1, 4, 3, 1><<<grid, block, 0, st>>>(a); break;
+        case 4: sgemm_kernel<AKC, BKC, PIPE, 1, 4, 3, 1><<<grid, block, 0, st>>>(a); break;
+        default: sgemm_kernel<AKC, BKC, PIPE, 1, 4, 2, 1><<<grid, block, 0, st>>>(a); break;
     }
 }
 

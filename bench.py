@@ -56,8 +56,8 @@ DEFAULT_WORKLOAD = "vgg_mid_conv3x3_128x56x56_b64"
 # (workload, stage) -> bytes.  None where no counter run has been made.
 TRAFFIC = {
     ("vgg_mid_conv3x3_128x56x56_b64", "gemm_fwd_NT"): 1080300000,    # 2.0 * 482.5 MB fetched + 115.3 MB written
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_dgrad_NN"): 1114400000,  # 2.0 * 94.8 + 924.8
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_wgrad_TN"): 1130700000,  # 2.0 * 532.3 + 66.1 (split-K partials incl.)
+    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_dgrad_NN"): 1116000000,  # 2.0 * 95.6 + 924.8
+    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_wgrad_TN"): 1124500000,  # 2.0 * 529.2 + 66.1 (split-K partials incl.)
     ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_fwd_NT"): 833100000,     # 2.0 * 342.2 + 148.7
     ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_dgrad_NN"): 798400000,   # 2.0 * 100.0 + 598.4 (rows of 363 floats)
     ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_wgrad_TN"): 1079200000,  # 2.0 * 514.4 + 50.4 (partials incl.)

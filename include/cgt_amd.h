@@ -238,14 +238,18 @@ int cgt_amd_lrn_bwd_f32(const float *x, const float *top, const float *scale,
  * Replaces the cblas_sgemm / cublasSgemm_v2 call of the Mul22 op body
  * (cgt/core.py:2194-2224).  May use a split-K workspace owned by the library
  * (one per stream); the reduction order is fixed, so results are
- * deterministic. */
+ * deterministic.  Limits: M, N, K < 2^31 - 128; ldc < 2^27 unless M <= 4
+ * (CGT_AMD_ERR_ARG otherwise); lda / ldb of 2^23 floats and more are accepted
+ * and take a slower, fully bounds-tested load path.  Operands need 4-byte
+ * alignment only. */
 int cgt_amd_sgemm(int tA, int tB, long M, long N, long K,
                   const float *A, long lda, const float *B, long ldb,
                   float *C, long ldc, void *stream);
 
 /* P independent products at A + p*strideA, B + p*strideB, C + p*strideC.
  * Replaces the cblas_sgemm loop of BatchedMul22 (cgt/core.py:2272-2285);
- * the reference has no GPU implementation of it. */
+ * the reference has no GPU implementation of it.  A stride of 0 shares one
+ * operand between all products.  P < 65536; other limits as cgt_amd_sgemm. */
 int cgt_amd_sgemm_batched(int tA, int tB, long P, long M, long N, long K,
                           const float *A, long lda, long strideA,
                           const float *B, long ldb, long strideB,

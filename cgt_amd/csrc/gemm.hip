@@ -10,16 +10,21 @@
 //
 // K is walked in slices of 16 through double-buffered LDS tiles: while the
 // matrix cores work on slice t from LDS buffer t&1, the global loads of slice
-// t+1 are in flight into registers and are written to the other buffer
-// afterwards -- one barrier per slice.
+// t+1 are in flight -- straight into the other LDS buffer
+// (global_load_lds_dwordx4: no staging registers, no LDS store instructions)
+// when the tile and the slice are whole, through registers with bounds tests
+// otherwise -- one barrier per slice.
 //
-// LDS layouts, chosen so that both the global loads and the fragment reads are
-// contiguous:
+// LDS layouts are dense, because a direct load deposits a wavefront's 64 x 16
+// bytes lane after lane:
 //   operand stored k-contiguous in memory (A not transposed, B transposed):
-//       tile[row][k], row stride 20 floats; a lane reads its four k values of
-//       an 8-wide k group with one 16-byte LDS read;
+//       tile[row][16]; the four 16-byte chunks of a row are permuted (chunk c
+//       of row r sits in slot c ^ ((r >> 2) & 3)) -- the permutation is applied
+//       by choosing which chunk a lane fetches, costs nothing, and makes the
+//       16-byte fragment reads (a lane reads its four k values of an 8-wide k
+//       group at once) and the register-path writes bank-conflict free;
 //   operand stored row-contiguous (A transposed, B not transposed):
-//       tile[k][row], row stride ROWS+4 floats; four 4-byte reads per k group.
+//       tile[k][rows]; four 4-byte reads per k group, lanes on consecutive rows.
 // Inside an 8-wide k group MFMA step i takes k = 4*half + i from lane half
 // `half` (lanes 0-31 / 32-63).  A and B use the same assignment, so the
 // products match; only the summation order inside the group differs from
@@ -60,7 +65,17 @@ struct __attribute__((packed, aligned(4))) float4u {
 
 constexpr int KT = 16;
 constexpr int kGemmThreads = 256;
-constexpr int LDK = KT + 4;    // row stride of a k-contiguous tile [ROWS][LDK]
+constexpr int LDK = KT;        // row stride of a k-contiguous tile [ROWS][LDK]: dense
+// slot of 16-byte chunk `chunk` in row `row` of a k-contiguous tile (an involution)
+__device__ __forceinline__ int chunk_pos(int row, int chunk) { return chunk ^ ((row >> 2) & 3); }
+
+// One 16-byte-per-lane load straight into LDS: lane l's data lands at lds_addr + 16*l.
+// Written as inline asm so that the compiler's wait-count insertion does not see it and
+// make every later LDS read wait for it; the loops wait with explicit s_waitcnt vmcnt.
+__device__ __forceinline__ void load_to_lds16(const void* base, unsigned voff, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
 
 struct GemmArgs {
     const float* A;
@@ -94,7 +109,7 @@ struct GemmArgs {
 // hardware adds the two (global_load_dwordx4 v, v_off, s[base]).
 template <bool KC, int ROWS>
 struct OperandTile {
-    static constexpr int LDM = ROWS + 4;
+    static constexpr int LDM = ROWS;       // row-contiguous tile [KT][LDM]: dense
     static constexpr int kFloats = KC ? ROWS * LDK : KT * LDM;
     static constexpr int kElems = ROWS * KT;
     static constexpr int NV = (kElems / 4 + kGemmThreads - 1) / kGemmThreads;   // 16-byte pieces per thread
@@ -111,7 +126,9 @@ struct OperandTile {
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int idx = threadIdx.x + i * kGemmThreads;
-            const long e = KC ? (long)(idx >> 2) * ld + (idx & 3) * 4
+            // the piece this thread fetches is the one whose LDS slot it fills: slot idx & 3
+            // of row idx >> 2 holds chunk chunk_pos(row, idx & 3) (the permutation is an involution)
+            const long e = KC ? (long)(idx >> 2) * ld + chunk_pos(idx >> 2, idx & 3) * 4
                               : (long)(idx / (ROWS / 4)) * ld + (idx % (ROWS / 4)) * 4;
             goff[i] = (unsigned)(e * 4);
         }
@@ -132,6 +149,18 @@ struct OperandTile {
             }
     }
 
+    // the same pieces straight into the LDS tile (dense layout: piece idx -> floats [4*idx, 4*idx+4))
+    __device__ __forceinline__ void load_direct(const char* __restrict__ origin, unsigned (&offs)[NV],
+                                                float* tile, int wave_u) const {
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+            if ((i + 1) * kGemmThreads * 4 <= kElems || (wave_u * 64 + i * kGemmThreads) * 4 < kElems) {
+                const unsigned lds = (unsigned)(size_t)(__attribute__((address_space(3))) float*)tile +
+                                     (unsigned)(i * kGemmThreads + wave_u * 64) * 16u;
+                load_to_lds16(origin, offs[i], lds);
+            }
+    }
+
     // bounds-tested: rows >= R and k >= kend read as zero
     __device__ __forceinline__ void load_checked(const float* __restrict__ p, long ld, int r0, int R,
                                                  int k0, int kend) {
@@ -141,7 +170,8 @@ struct OperandTile {
             float t[4] = {0.f, 0.f, 0.f, 0.f};
             if (has(i)) {
                 if (KC) {
-                    const int row = r0 + (idx >> 2), k = k0 + (idx & 3) * 4;
+                    // like the untested loads: the chunk that belongs in this thread's LDS slot
+                    const int row = r0 + (idx >> 2), k = k0 + chunk_pos(idx >> 2, idx & 3) * 4;
                     const float* src = p + (long)row * ld + k;
                     if (row < R && k + 3 < kend) {
                         const float4u q = *reinterpret_cast<const float4u*>(src);
@@ -185,7 +215,7 @@ struct OperandTile {
     static __device__ __forceinline__ void frag(const float* __restrict__ tile, int row, int kk,
                                                 int half, float (&f)[4]) {
         if (KC) {
-            const float4 t = *reinterpret_cast<const float4*>(tile + row * LDK + kk * 8 + half * 4);
+            const float4 t = *reinterpret_cast<const float4*>(tile + row * LDK + chunk_pos(row, kk * 2 + half) * 4);
             f[0] = t.x; f[1] = t.y; f[2] = t.z; f[3] = t.w;
         } else {
             const float* q = tile + (kk * 8 + half * 4) * LDM + row;
@@ -344,7 +374,45 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
     // immediate); the plain one is not: unrolled, it needs more than the 128
     // registers that let four workgroups share a CU.
     auto main_loop = [&](auto mode) {
-        if constexpr (PIPE) {
+        if constexpr (PIPE && decltype(mode)::value == kFast) {
+            // whole tile, whole slices: slice kt+2 goes straight into the LDS buffer that
+            // slice kt leaves behind, issued right after the barrier in the middle of
+            // iteration kt (every wavefront has read its last fragments of slice kt by
+            // then); it has to have landed by the barrier of iteration kt+1.
+            const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+            if (nk > 0) {
+                ta.load_direct(originA, ta.goff, As[0], wave_u);
+                tb.load_direct(originB, tb.goff, Bs[0], wave_u);
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                read_frags(0, As[0], Bs[0], 0);
+                if (nk > 1) {
+                    ta.load_direct(originA + stepA, ta.goff, As[1], wave_u);
+                    tb.load_direct(originB + stepB, tb.goff, Bs[1], wave_u);
+                }
+            }
+            auto iteration = [&](int kt, auto curc) {
+                constexpr int cur = decltype(curc)::value;
+                read_frags(1, As[cur], Bs[cur], 1);
+                __builtin_amdgcn_s_setprio(3);
+                mfma_steps(0, 0, 4);
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // slice kt+1 is in LDS
+                lds_barrier();
+                if (kt + 2 < nk) {
+                    ta.load_direct(originA + (kt + 2) * stepA, ta.goff, As[cur], wave_u);
+                    tb.load_direct(originB + (kt + 2) * stepB, tb.goff, Bs[cur], wave_u);
+                }
+                if (kt + 1 < nk) read_frags(0, As[cur ^ 1], Bs[cur ^ 1], 0);
+                mfma_steps(1, 0, 4);
+                __builtin_amdgcn_s_setprio(0);
+            };
+            int kt = 0;
+            for (; kt + 1 < nk; kt += 2) {
+                iteration(kt, std::integral_constant<int, 0>{});
+                iteration(kt + 1, std::integral_constant<int, 1>{});
+            }
+            if (kt < nk) iteration(kt, std::integral_constant<int, 0>{});
+        } else if constexpr (PIPE) {
             if (nk > 0) {
                 load_slice(mode, ta, tb, 0);
                 ta.store(As[0]);
@@ -413,6 +481,34 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                     iteration(kt + 1, ta, tb);
                 }
                 if (kt < nk) iteration(kt, ta1, tb1);
+            } else if constexpr (decltype(mode)::value == kFast) {
+                // Whole tile, whole slices: the global loads of slice kt+1 go straight into
+                // the other LDS buffer while slice kt is multiplied -- no staging registers,
+                // no LDS store instructions.  The buffer being filled was last read in
+                // iteration kt-1, which every wavefront left through the barrier.
+                const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+                if (nk > 0) {
+                    ta.load_direct(originA, ta.goff, As[0], wave_u);
+                    tb.load_direct(originB, tb.goff, Bs[0], wave_u);
+                }
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                for (int kt = 0; kt < nk; ++kt) {
+                    const int cur = kt & 1;
+                    if (kt + 1 < nk) {
+                        ta.load_direct(originA + (kt + 1) * stepA, ta.goff, As[cur ^ 1], wave_u);
+                        tb.load_direct(originB + (kt + 1) * stepB, tb.goff, Bs[cur ^ 1], wave_u);
+                    }
+                    __builtin_amdgcn_s_setprio(3);
+#pragma unroll
+                    for (int kk = 0; kk < KT / 8; ++kk) {
+                        read_frags(0, As[cur], Bs[cur], kk);
+                        mfma_steps(0, 0, 4);
+                    }
+                    __builtin_amdgcn_s_setprio(0);
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    __syncthreads();
+                }
             } else {
                 if (nk > 0) {
                     load_slice(mode, ta, tb, 0);

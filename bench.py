@@ -55,12 +55,12 @@ DEFAULT_WORKLOAD = "vgg_mid_conv3x3_128x56x56_b64"
 # WRITE_SIZE runs of this script (summaries and calibration in profiles/):
 # (workload, stage) -> bytes.  None where no counter run has been made.
 TRAFFIC = {
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_fwd_NT"): 1080300000,    # 2.0 * 482.5 MB fetched + 115.3 MB written
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_dgrad_NN"): 1116000000,  # 2.0 * 95.6 + 924.8
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_wgrad_TN"): 1124500000,  # 2.0 * 529.2 + 66.1 (split-K partials incl.)
-    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_fwd_NT"): 833100000,     # 2.0 * 342.2 + 148.7
-    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_dgrad_NN"): 798400000,   # 2.0 * 100.0 + 598.4 (rows of 363 floats)
-    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_wgrad_TN"): 1079200000,  # 2.0 * 514.4 + 50.4 (partials incl.)
+    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_fwd_NT"): 1087900000,    # 2.0 * 486.3 MB fetched + 115.3 MB written
+    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_dgrad_NN"): 1091000000,  # 2.0 * 83.1 + 924.8
+    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_wgrad_TN"): 1128100000,  # 2.0 * 531.0 + 66.1 (split-K partials incl.)
+    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_fwd_NT"): 828500000,     # 2.0 * 339.9 + 148.7
+    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_dgrad_NN"): 831400000,   # 2.0 * 117.2 + 597.0 (rows of 363 floats)
+    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_wgrad_TN"): 1095000000,  # 2.0 * 522.4 + 50.2 (partials incl.)
 }
 
 

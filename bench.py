@@ -222,7 +222,8 @@ class LayerOnGpu(object):
     def time_stages(self, reps):
         from cgt_amd import capi
         for st in self.stages + getattr(self, "extra_stages", []):
-            st.fn()
+            for _ in range(5):          # warm-up launches of this kernel (clock and caches settle)
+                st.fn()
             e0, e1 = capi.Event(), capi.Event()
             e0.record(self.stream)
             for _ in range(reps):

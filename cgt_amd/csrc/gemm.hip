@@ -510,16 +510,34 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                     __syncthreads();
                 }
             } else {
+                // Edge tile and / or ragged K.  Each operand on its own still loads straight
+                // into LDS wherever its side of the tile is whole and the slice is whole (an
+                // edge tile in N streams A that way); the rest goes through registers with
+                // bounds tests and is parked in LDS after the multiply.
+                const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+                auto issue = [&](int slice, float* as, float* bs) {
+                    const bool tested = ragged_k && slice == nk - 1;
+                    const int k0 = kbeg + slice * KT;
+                    if (wholeA && !tested) ta.load_direct(originA + slice * stepA, ta.goff, as, wave_u);
+                    else ta.load_checked(A, a.lda, m0, a.M, k0, kend);
+                    if (wholeB && !tested) tb.load_direct(originB + slice * stepB, tb.goff, bs, wave_u);
+                    else tb.load_checked(B, a.ldb, n0, a.N, k0, kend);
+                };
+                auto park = [&](int slice, float* as, float* bs) {
+                    const bool tested = ragged_k && slice == nk - 1;
+                    if (!wholeA || tested) ta.store(as);
+                    if (!wholeB || tested) tb.store(bs);
+                };
                 if (nk > 0) {
-                    load_slice(mode, ta, tb, 0);
-                    ta.store(As[0]);
-                    tb.store(Bs[0]);
+                    issue(0, As[0], Bs[0]);
+                    park(0, As[0], Bs[0]);
                 }
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 __syncthreads();
                 for (int kt = 0; kt < nk; ++kt) {
                     const int cur = kt & 1;
                     const bool more = kt + 1 < nk;
-                    if (more) load_slice(mode, ta, tb, kt + 1);
+                    if (more) issue(kt + 1, As[cur ^ 1], Bs[cur ^ 1]);
                     __builtin_amdgcn_s_setprio(3);
 #pragma unroll
                     for (int kk = 0; kk < KT / 8; ++kk) {
@@ -527,10 +545,8 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                         mfma_steps(0, 0, 4);
                     }
                     __builtin_amdgcn_s_setprio(0);
-                    if (more) {
-                        ta.store(As[cur ^ 1]);
-                        tb.store(Bs[cur ^ 1]);
-                    }
+                    if (more) park(kt + 1, As[cur ^ 1], Bs[cur ^ 1]);
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                     __syncthreads();
                 }
             }

@@ -55,12 +55,12 @@ DEFAULT_WORKLOAD = "vgg_mid_conv3x3_128x56x56_b64"
 # WRITE_SIZE runs of this script (summaries and calibration in profiles/):
 # (workload, stage) -> bytes.  None where no counter run has been made.
 TRAFFIC = {
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_fwd_NT"): 1087900000,    # 2.0 * 486.3 MB fetched + 115.3 MB written
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_dgrad_NN"): 1091000000,  # 2.0 * 83.1 + 924.8
+    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_fwd_NT"): 1087300000,    # 2.0 * 486.0 MB fetched + 115.3 MB written
+    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_dgrad_NN"): 1088800000,  # 2.0 * 82.0 + 924.8
     ("vgg_mid_conv3x3_128x56x56_b64", "gemm_wgrad_TN"): 1128100000,  # 2.0 * 531.0 + 66.1 (split-K partials incl.)
-    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_fwd_NT"): 828500000,     # 2.0 * 339.9 + 148.7
-    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_dgrad_NN"): 831400000,   # 2.0 * 117.2 + 597.0 (rows of 363 floats)
-    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_wgrad_TN"): 1095000000,  # 2.0 * 522.4 + 50.2 (partials incl.)
+    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_fwd_NT"): 828900000,     # 2.0 * 340.1 + 148.7
+    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_dgrad_NN"): 811500000,   # 2.0 * 106.8 + 597.9 (rows of 363 floats)
+    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_wgrad_TN"): 1099100000,  # 2.0 * 524.4 + 50.3 (partials incl.)
 }
 
 

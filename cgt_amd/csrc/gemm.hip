@@ -868,8 +868,9 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     // The pipelined loop needs up to ~140 registers in its 128x128 form (3 workgroups
     // per CU instead of 4): it is used once every CU has more than a handful of tiles
     // to work through, not when the whole product is one round of resident
-    // workgroups (4096^3: 1024 tiles = 4 per CU).
-    const bool pipe = tiles * P >= 5L * kNumCU;
+    // workgroups (4096^3: 1024 tiles = 4 per CU), and not for a ragged K, where its
+    // tiles would all take the register-staged variant (K = 363: plain loop +3 %).
+    const bool pipe = tiles * P >= 5L * kNumCU && K % KT == 0;
     // two slices of loads in flight: one round of resident workgroups (they start together
     // and load in bursts) with a long K range each
     const long slices = cdiv(a.splits > 1 ? (long)a.kchunk : K, KT);

@@ -412,36 +412,6 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                 iteration(kt + 1, std::integral_constant<int, 1>{});
             }
             if (kt < nk) iteration(kt, std::integral_constant<int, 0>{});
-        } else if constexpr (PIPE) {
-            if (nk > 0) {
-                load_slice(mode, ta, tb, 0);
-                ta.store(As[0]);
-                tb.store(Bs[0]);
-                if (nk > 1) load_slice(mode, ta, tb, 1);
-                lds_barrier();
-                read_frags(0, As[0], Bs[0], 0);
-            }
-            auto iteration = [&](int kt, auto curc) {
-                constexpr int cur = decltype(curc)::value;
-                if (kt + 1 < nk) {
-                    ta.store(As[cur ^ 1]);       // slice kt+1 (waits for its global loads, issued an iteration ago)
-                    tb.store(Bs[cur ^ 1]);
-                }
-                if (kt + 2 < nk) load_slice(mode, ta, tb, kt + 2);
-                read_frags(1, As[cur], Bs[cur], 1);
-                __builtin_amdgcn_s_setprio(3);   // inside the MFMA stream: ahead of wavefronts issuing loads
-                mfma_steps(0, 0, 4);
-                lds_barrier();
-                if (kt + 1 < nk) read_frags(0, As[cur ^ 1], Bs[cur ^ 1], 0);
-                mfma_steps(1, 0, 4);
-                __builtin_amdgcn_s_setprio(0);
-            };
-            int kt = 0;
-            for (; kt + 1 < nk; kt += 2) {
-                iteration(kt, std::integral_constant<int, 0>{});
-                iteration(kt + 1, std::integral_constant<int, 1>{});
-            }
-            if (kt < nk) iteration(kt, std::integral_constant<int, 0>{});
         } else {
             if constexpr (DEEP) {
                 // Two register sets: the loads of slices kt+1 and kt+2 are in flight while

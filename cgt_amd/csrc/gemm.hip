@@ -394,7 +394,6 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
             auto iteration = [&](int kt, auto curc) {
                 constexpr int cur = decltype(curc)::value;
                 read_frags(1, As[cur], Bs[cur], 1);
-                __builtin_amdgcn_s_setprio(3);
                 mfma_steps(0, 0, 4);
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // slice kt+1 is in LDS
                 lds_barrier();
@@ -404,7 +403,6 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                 }
                 if (kt + 1 < nk) read_frags(0, As[cur ^ 1], Bs[cur ^ 1], 0);
                 mfma_steps(1, 0, 4);
-                __builtin_amdgcn_s_setprio(0);
             };
             int kt = 0;
             for (; kt + 1 < nk; kt += 2) {
@@ -431,13 +429,11 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                 // iteration kt: pa/pb hold slice kt+1, the other set slice kt+2
                 auto iteration = [&](int kt, TileA& pa, TileB& pb) {
                     const int cur = kt & 1;
-                    __builtin_amdgcn_s_setprio(3);
 #pragma unroll
                     for (int kk = 0; kk < KT / 8; ++kk) {
                         read_frags(0, As[cur], Bs[cur], kk);
                         mfma_steps(0, 0, 4);
                     }
-                    __builtin_amdgcn_s_setprio(0);
                     if (kt + 1 < nk) {
                         pa.store(As[cur ^ 1]);
                         pb.store(Bs[cur ^ 1]);
@@ -469,13 +465,11 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                         ta.load_direct(originA + (kt + 1) * stepA, ta.goff, As[cur ^ 1], wave_u);
                         tb.load_direct(originB + (kt + 1) * stepB, tb.goff, Bs[cur ^ 1], wave_u);
                     }
-                    __builtin_amdgcn_s_setprio(3);
 #pragma unroll
                     for (int kk = 0; kk < KT / 8; ++kk) {
                         read_frags(0, As[cur], Bs[cur], kk);
                         mfma_steps(0, 0, 4);
                     }
-                    __builtin_amdgcn_s_setprio(0);
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                     __syncthreads();
                 }
@@ -508,13 +502,11 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                     const int cur = kt & 1;
                     const bool more = kt + 1 < nk;
                     if (more) issue(kt + 1, As[cur ^ 1], Bs[cur ^ 1]);
-                    __builtin_amdgcn_s_setprio(3);
 #pragma unroll
                     for (int kk = 0; kk < KT / 8; ++kk) {
                         read_frags(0, As[cur], Bs[cur], kk);
                         mfma_steps(0, 0, 4);
                     }
-                    __builtin_amdgcn_s_setprio(0);
                     if (more) park(kt + 1, As[cur ^ 1], Bs[cur ^ 1]);
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                     __syncthreads();

@@ -50,31 +50,40 @@ __device__ __forceinline__ float pow_neg_beta(float s, float nbeta) {
 // loads -- H*W is odd in the AlexNet layer -- so depth has to come from here).
 constexpr int kLrnChunk = 8;
 
-template <int SIZE>
-__global__ __launch_bounds__(kLrnThreads) void lrn_fwd_kernel(
-    const float* __restrict__ x, float* __restrict__ top, float* __restrict__ scale, int C,
-    int HW, int crun, float aos, float nbeta, float kconst) {
-    constexpr int PRE = (SIZE - 1) / 2, POST = SIZE - PRE - 1, U = kLrnChunk;
-    const LrnBlock blk = lrn_block(HW, C, crun);
+// DOWN: the run is walked from its last channel to its first.  Odd runs walk down and
+// even runs up, so the channels two neighbouring runs both need (each run's halo is the
+// other's edge) are loaded by both at the same end of their walk -- at about the same
+// time, which lets one of the two find them in L2 instead of fetching them again.  A
+// downward walk is the upward one on the mirrored channel axis v = C-1-c: window
+// [c-PRE, c+POST] becomes [v-POST, v+PRE], pointers step by -H*W.
+template <int SIZE, bool DOWN>
+__device__ __forceinline__ void lrn_fwd_run(const float* __restrict__ x, float* __restrict__ top,
+                                            float* __restrict__ scale, int C, int HW, const LrnBlock& blk,
+                                            int crun, float aos, float nbeta, float kconst) {
+    constexpr int PRE0 = (SIZE - 1) / 2, POST0 = SIZE - PRE0 - 1, U = kLrnChunk;
+    constexpr int PRE = DOWN ? POST0 : PRE0, POST = DOWN ? PRE0 : POST0;
     const int p = blk.px * kLrnThreads + threadIdx.x;
     if (p >= HW) return;
     const long n = blk.n;
-    const int cs = blk.run * crun, ce = min(C, cs + crun);
-    const float* xp = x + n * C * (long)HW + p;
-    float* tp = top + n * C * (long)HW + p;
-    float* sp = scale + n * C * (long)HW + p;
+    const int cs0 = blk.run * crun, ce0 = min(C, cs0 + crun);
+    const int cs = DOWN ? C - ce0 : cs0, ce = DOWN ? C - cs0 : ce0;     // the run on the walked axis
+    const long hs = DOWN ? -(long)HW : (long)HW;
+    const long origin = n * C * (long)HW + p + (DOWN ? (long)(C - 1) * HW : 0);
+    const float* xp = x + origin;
+    float* tp = top + origin;
+    float* sp = scale + origin;
 
     float win[U + SIZE - 1];  // win[j] = x[c0 - PRE + j]
 #pragma unroll
     for (int j = 0; j < SIZE - 1; ++j) {
         const int c = cs - PRE + j;
-        win[j] = (c >= 0 && c < C) ? xp[(long)c * HW] : 0.0f;
+        win[j] = (c >= 0 && c < C) ? xp[c * hs] : 0.0f;
     }
     for (int c0 = cs; c0 < ce; c0 += U) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int ch = c0 + POST + u;
-            win[SIZE - 1 + u] = (ch < C) ? xp[(long)ch * HW] : 0.0f;
+            win[SIZE - 1 + u] = (ch < C) ? xp[ch * hs] : 0.0f;
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -83,13 +92,22 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_fwd_kernel(
             for (int j = 0; j < SIZE; ++j) acc += win[u + j] * win[u + j];
             const float s = kconst + acc * aos;
             if (c0 + u < ce) {
-                sp[(long)(c0 + u) * HW] = s;
-                tp[(long)(c0 + u) * HW] = win[u + PRE] * pow_neg_beta(s, nbeta);
+                sp[(c0 + u) * hs] = s;
+                tp[(c0 + u) * hs] = win[u + PRE] * pow_neg_beta(s, nbeta);
             }
         }
 #pragma unroll
         for (int j = 0; j < SIZE - 1; ++j) win[j] = win[U + j];
     }
+}
+
+template <int SIZE>
+__global__ __launch_bounds__(kLrnThreads) void lrn_fwd_kernel(
+    const float* __restrict__ x, float* __restrict__ top, float* __restrict__ scale, int C,
+    int HW, int crun, float aos, float nbeta, float kconst) {
+    const LrnBlock blk = lrn_block(HW, C, crun);
+    if (blk.run & 1) lrn_fwd_run<SIZE, true>(x, top, scale, C, HW, blk, crun, aos, nbeta, kconst);
+    else lrn_fwd_run<SIZE, false>(x, top, scale, C, HW, blk, crun, aos, nbeta, kconst);
 }
 
 // Any window length: re-reads the window through the cache.
@@ -116,19 +134,21 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_fwd_generic_kernel(
     }
 }
 
-template <int SIZE>
-__global__ __launch_bounds__(kLrnThreads) void lrn_bwd_kernel(
-    const float* __restrict__ x, const float* __restrict__ top, const float* __restrict__ scale,
-    const float* __restrict__ top_diff, float* __restrict__ bottom_diff, int C, int HW, int crun,
-    float nbeta, float ratio) {
-    // transposed window: [c - PRE, c + POST]
-    constexpr int PRE = SIZE - (SIZE + 1) / 2, POST = SIZE - PRE - 1, U = kLrnChunk;
-    const LrnBlock blk = lrn_block(HW, C, crun);
+template <int SIZE, bool DOWN>
+__device__ __forceinline__ void lrn_bwd_run(const float* __restrict__ x, const float* __restrict__ top,
+                                            const float* __restrict__ scale, const float* __restrict__ top_diff,
+                                            float* __restrict__ bottom_diff, int C, int HW, const LrnBlock& blk,
+                                            int crun, float nbeta, float ratio) {
+    // transposed window: [c - PRE0, c + POST0]; mirrored when walking down (see lrn_fwd_run)
+    constexpr int PRE0 = SIZE - (SIZE + 1) / 2, POST0 = SIZE - PRE0 - 1, U = kLrnChunk;
+    constexpr int PRE = DOWN ? POST0 : PRE0, POST = DOWN ? PRE0 : POST0;
     const int p = blk.px * kLrnThreads + threadIdx.x;
     if (p >= HW) return;
     const long n = blk.n;
-    const int cs = blk.run * crun, ce = min(C, cs + crun);
-    const long base = n * C * (long)HW + p;
+    const int cs0 = blk.run * crun, ce0 = min(C, cs0 + crun);
+    const int cs = DOWN ? C - ce0 : cs0, ce = DOWN ? C - cs0 : ce0;
+    const long hs = DOWN ? -(long)HW : (long)HW;
+    const long base = n * C * (long)HW + p + (DOWN ? (long)(C - 1) * HW : 0);
     const float* xp = x + base;
     const float* tp = top + base;
     const float* sp = scale + base;
@@ -143,9 +163,9 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_bwd_kernel(
         const int c = cs - PRE + j;
         float d = 0.0f, sc = 1.0f, t = 0.0f;
         if (c >= 0 && c < C) {
-            d = dp[(long)c * HW];
-            sc = sp[(long)c * HW];
-            t = tp[(long)c * HW];
+            d = dp[c * hs];
+            sc = sp[c * hs];
+            t = tp[c * hs];
         }
         tr[j] = d * t / sc;
         if (j >= PRE) {           // channel >= cs: also a centre later on
@@ -160,14 +180,14 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_bwd_kernel(
             const int ch = c0 + POST + u;
             float d = 0.0f, sc = 1.0f, t = 0.0f;
             if (ch < C) {
-                d = dp[(long)ch * HW];
-                sc = sp[(long)ch * HW];
-                t = tp[(long)ch * HW];
+                d = dp[ch * hs];
+                sc = sp[ch * hs];
+                t = tp[ch * hs];
             }
             dr[POST + u] = d;
             sr[POST + u] = sc;
             tn[u] = t;
-            xc[u] = (c0 + u < ce) ? xp[(long)(c0 + u) * HW] : 0.0f;
+            xc[u] = (c0 + u < ce) ? xp[(c0 + u) * hs] : 0.0f;
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) tr[SIZE - 1 + u] = dr[POST + u] * tn[u] / sr[POST + u];
@@ -177,7 +197,7 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_bwd_kernel(
 #pragma unroll
             for (int j = 0; j < SIZE; ++j) acc += tr[u + j];
             if (c0 + u < ce)
-                bp[(long)(c0 + u) * HW] = dr[u] * pow_neg_beta(sr[u], nbeta) - ratio * xc[u] * acc;
+                bp[(c0 + u) * hs] = dr[u] * pow_neg_beta(sr[u], nbeta) - ratio * xc[u] * acc;
         }
 #pragma unroll
         for (int j = 0; j < SIZE - 1; ++j) tr[j] = tr[U + j];
@@ -187,6 +207,16 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_bwd_kernel(
             sr[j] = sr[U + j];
         }
     }
+}
+
+template <int SIZE>
+__global__ __launch_bounds__(kLrnThreads) void lrn_bwd_kernel(
+    const float* __restrict__ x, const float* __restrict__ top, const float* __restrict__ scale,
+    const float* __restrict__ top_diff, float* __restrict__ bottom_diff, int C, int HW, int crun,
+    float nbeta, float ratio) {
+    const LrnBlock blk = lrn_block(HW, C, crun);
+    if (blk.run & 1) lrn_bwd_run<SIZE, true>(x, top, scale, top_diff, bottom_diff, C, HW, blk, crun, nbeta, ratio);
+    else lrn_bwd_run<SIZE, false>(x, top, scale, top_diff, bottom_diff, C, HW, blk, crun, nbeta, ratio);
 }
 
 __global__ __launch_bounds__(kLrnThreads) void lrn_bwd_generic_kernel(

@@ -21,6 +21,19 @@ constexpr int kNumCU = 256;  // MI355X compute units
 
 __host__ __device__ inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 
+// Streaming (non-temporal) 16-byte store for data that is written once, in whole cache
+// lines, and not read again by the same kernel: the lines are not kept in L2.  Measured
+// on this chip: the VGG im2col (925 MB written in aligned 1152-byte runs) goes from 4.9 to
+// 5.9 TB/s with it and the 96 x 3025 transpose from 5.2 to 7.1 TB/s, while 4-byte stores
+// and runs that start anywhere (rows of 363 floats, planes of 3025) get SLOWER without
+// L2's write combining (AlexNet im2col -27 %, pool pullback -59 %), so only aligned
+// vector stores use it.
+typedef float v4f __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void stream_store4(float* p, float a, float b, float c, float d) {
+    v4f v = {a, b, c, d};
+    __builtin_nontemporal_store(v, reinterpret_cast<v4f*>(p));
+}
+
 // Geometry known at compile time (hot shapes) ...
 template <int KH, int KW, int PH, int PW, int SH, int SW>
 struct StaticGeom {

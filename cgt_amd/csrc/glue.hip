@@ -112,7 +112,7 @@ __global__ __launch_bounds__(256) void thin_transpose_kernel(const float* __rest
             for (int i = threadIdx.x * 4; i < n; i += 1024) {
                 const int r = div_small(i, L, rL), c = i - r * L;
                 const float* t = tile + r * LD + c;
-                *reinterpret_cast<float4*>(blk_out + i) = make_float4(t[0], t[1], t[2], t[3]);
+                stream_store4(blk_out + i, t[0], t[1], t[2], t[3]);
             }
         } else {
             for (int i = threadIdx.x; i < n; i += 256) {
@@ -150,10 +150,11 @@ static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 1
 static int launch_batched_transpose(const float* in, float* out, long B, long R, long Cn,
                                     hipStream_t st) {
     CGT_ARG_CHECK(R < (1L << 31) && Cn < (1L << 31), "transpose: too large");
-    // thin paths: the short extent is not a multiple of the square tile (which
-    // would idle lanes) or the long one is odd (unaligned rows either way)
-    const bool thin_in = Cn <= kThinMaxL && R >= 4 * kThinRows && (Cn % kTile != 0 || R % 4 != 0);
-    const bool thin_out = R <= kThinMaxL && Cn >= 4 * kThinRows && (R % kTile != 0 || Cn % 4 != 0);
+    // thin paths whenever one extent fits a workgroup whole: no idle lanes when
+    // it is not a multiple of the square tile, and one side of the copy is a
+    // contiguous block moved 16 bytes at a time (streamed on the way out)
+    const bool thin_in = Cn <= kThinMaxL && R >= 4 * kThinRows;
+    const bool thin_out = R <= kThinMaxL && Cn >= 4 * kThinRows;
     if (thin_in || thin_out) {
         const long L = thin_in ? Cn : R, longdim = thin_in ? R : Cn;
         const long tiles = cdiv(longdim, kThinRows);

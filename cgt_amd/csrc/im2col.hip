@@ -99,8 +99,7 @@ __global__ __launch_bounds__(kIm2colThreads) void im2col_rows_kernel(
         const long ostep = (long)slots * Z;
         for (int w = w0; w < n; w += slots) {
             if (VEC) {
-                *reinterpret_cast<float4*>(out) =
-                    make_float4(tile[off[0]], tile[off[UW > 1 ? 1 : 0]], tile[off[UW > 2 ? 2 : 0]], tile[off[UW > 3 ? 3 : 0]]);
+                stream_store4(out, tile[off[0]], tile[off[UW > 1 ? 1 : 0]], tile[off[UW > 2 ? 2 : 0]], tile[off[UW > 3 ? 3 : 0]]);
             } else {
                 out[0] = tile[off[0]];
             }
@@ -192,8 +191,7 @@ __global__ __launch_bounds__(kIm2colThreads) void im2col_pipe_kernel(
                 const long ostep = (long)slots * Z;
                 for (int w = w0; w < n; w += slots) {
                     if (VEC) {
-                        *reinterpret_cast<float4*>(out) =
-                            make_float4(cur[off[0]], cur[off[UW > 1 ? 1 : 0]], cur[off[UW > 2 ? 2 : 0]], cur[off[UW > 3 ? 3 : 0]]);
+                        stream_store4(out, cur[off[0]], cur[off[UW > 1 ? 1 : 0]], cur[off[UW > 2 ? 2 : 0]], cur[off[UW > 3 ? 3 : 0]]);
                     } else {
                         out[0] = cur[off[0]];
                     }

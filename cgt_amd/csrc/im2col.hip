@@ -280,8 +280,8 @@ __global__ __launch_bounds__(256) void col2im_gather_kernel(
 //
 // Each row is staged through LDS as contiguous runs of CC*kh*kw floats
 // (coalesced; the buffer is read once apart from kh-sh halo rows per band and
-// the kw-sw halo columns per tile).  The global loads of row h-1 are issued
-// into registers before row h is consumed, so their latency is hidden.
+// the kw-sw halo columns per tile).  Two rows are in flight in registers: the
+// loads of row h-2 are issued right after row h is parked in LDS.
 //
 // Staging modes: kStageScalar (4-byte loads), kStageRuns (16-byte loads inside
 // each run; needs CC*kh*kw % 4 == 0 and C % CC == 0), kStageLinear (CC == C, so
@@ -298,7 +298,7 @@ constexpr int kStageScalar = 0, kStageRuns = 1, kStageLinear = 2;
 template <class G, int CC, int WSUB, int MODE, int LW = 64>
 __global__ __launch_bounds__(256) void col2im_stream_kernel(
     G g, const float* __restrict__ col, float* __restrict__ im, int C, int H, int W, int m, int n,
-    int band, int bands, int tiles_w, int nchunks, long col_floats) {
+    int band, int bands, int tiles_w, int nchunks) {
     constexpr bool VEC = MODE == kStageRuns, LIN = MODE == kStageLinear;
     constexpr int KH = G::kKH, KW = G::kKW, PH = G::kPH, PW = G::kPW, SH = G::kSH, SW = G::kSW;
     static_assert(SH <= KH && SW <= KW, "streaming col2im needs stride <= kernel");
@@ -357,105 +357,72 @@ __global__ __launch_bounds__(256) void col2im_stream_kernel(
     const int t_bot = hp0 + PH - (KH - 1);
     const int h_bot = t_bot >= 0 ? (t_bot + SH - 1) / SH : -((-t_bot) / SH);
 
-    typedef typename std::conditional<VEC || LIN, float4, float>::type PreT;
+    // Live rows are those inside [0, m); the ones outside only slide the window.
+    int live_hi = min(h_top, m - 1), live_lo = max(h_bot, 0);
+    if (nw <= 0 || live_hi < live_lo) {               // nothing to read: slide through the whole range
+        live_hi = h_bot - 1;
+        live_lo = h_bot;
+    }
+
+    // Staging is branch-free: every thread issues all NP loads of a row (indices
+    // past the end are clamped to the last unit, whose value then lands twice in
+    // the same LDS slot) and parks all of them.  A load that some lanes skip
+    // leaves its destination registers "possibly in flight" on the skipped
+    // path, and every later load into them then has to wait for the memory
+    // pipeline to drain; with straight-line code the waits count loads instead.
+    typedef typename std::conditional<VEC || LIN, v4f, float>::type PreT;
     PreT pre0[NP], pre1[NP];        // two rows in flight
     int lead = 0, lead0 = 0, lead1 = 0;   // LIN: floats between the 16-byte boundary and the row's first float
-    auto prefetch = [&](PreT (&pre)[NP], int& lead_next, int h) {
-        if (h < 0 || h >= m || nw <= 0) return;
+    auto prefetch = [&](PreT (&pre)[NP], int& lead_next, int h) __attribute__((always_inline)) {
         const float* src = col + ((b * m + h) * (long)n + w_lo) * Z + (long)c0 * KK;
         if constexpr (LIN) {
+            // col is 16-byte aligned and holds a multiple of 4 floats, so every
+            // aligned unit that starts inside the buffer lies inside it
             lead_next = (int)((reinterpret_cast<uintptr_t>(src) >> 2) & 3);
-            const float* al = src - lead_next;           // col is 16-byte aligned: never below it
-            const long off = al - col;
-            const int n4 = (nw * RUN + lead_next + 3) >> 2;
+            const v4f* al = reinterpret_cast<const v4f*>(src - lead_next);
+            const int last = ((nw * RUN + lead_next + 3) >> 2) - 1;
+#pragma unroll
+            for (int u = 0; u < NP; ++u) pre[u] = al[min((int)threadIdx.x + u * 256, last)];
+        } else {
 #pragma unroll
             for (int u = 0; u < NP; ++u) {
-                const int idx = threadIdx.x + u * 256;
-                if (idx < n4) {
-                    if (off + 4L * idx + 3 < col_floats) {
-                        pre[u] = reinterpret_cast<const float4*>(al)[idx];
-                    } else {                             // last floats of the whole buffer
-                        float t[4];
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) t[j] = off + 4L * idx + j < col_floats ? al[4 * idx + j] : 0.0f;
-                        pre[u] = make_float4(t[0], t[1], t[2], t[3]);
-                    }
+                const int idx = min((int)threadIdx.x + u * 256, total - 1);
+                if constexpr (VEC) {
+                    const int w = idx / (RUN / 4), z4 = (idx - w * (RUN / 4)) * 4;
+                    pre[u] = *reinterpret_cast<const v4f*>(src + (long)w * Z + z4);
+                } else {
+                    const int w = full ? idx / RUN : idx / run;
+                    const int zc = idx - w * run;
+                    pre[u] = src[(long)w * Z + zc];
                 }
-            }
-            return;
-        }
-#pragma unroll
-        for (int u = 0; u < NP; ++u) {
-            const int idx = threadIdx.x + u * 256;
-            if constexpr (VEC) {
-                const int w = idx / (RUN / 4), z4 = (idx - w * (RUN / 4)) * 4;
-                if (idx < total) pre[u] = *reinterpret_cast<const float4*>(src + (long)w * Z + z4);
-            } else if constexpr (!LIN) {
-                const int w = full ? idx / RUN : idx / run;
-                const int zc = idx - w * run;
-                if (idx < total) pre[u] = src[(long)w * Z + zc];
             }
         }
     };
-    auto park = [&](const PreT (&pre)[NP], int lead_next) {
+    auto park = [&](const PreT (&pre)[NP], int lead_next) __attribute__((always_inline)) {
         if constexpr (LIN) {
-            lead = lead_next;
-            const int n4 = (nw * RUN + lead + 3) >> 2;
+            lead = lead_next;                         // the staging area holds NP * 256 units
+#pragma unroll
+            for (int u = 0; u < NP; ++u) reinterpret_cast<v4f*>(stage)[threadIdx.x + u * 256] = pre[u];
+        } else {
 #pragma unroll
             for (int u = 0; u < NP; ++u) {
-                const int idx = threadIdx.x + u * 256;
-                if (idx < n4) reinterpret_cast<float4*>(stage)[idx] = pre[u];
-            }
-            return;
-        }
-#pragma unroll
-        for (int u = 0; u < NP; ++u) {
-            const int idx = threadIdx.x + u * 256;
-            if constexpr (VEC) {
-                const int w = idx / (RUN / 4), z4 = (idx - w * (RUN / 4)) * 4;
-                if (idx < total) {
+                const int idx = min((int)threadIdx.x + u * 256, total - 1);
+                if constexpr (VEC) {
+                    const int w = idx / (RUN / 4), z4 = (idx - w * (RUN / 4)) * 4;
                     float* d = stage + w * LD + z4;
                     d[0] = pre[u].x; d[1] = pre[u].y; d[2] = pre[u].z; d[3] = pre[u].w;
+                } else {
+                    const int w = full ? idx / RUN : idx / run;
+                    const int zc = idx - w * run;
+                    stage[w * LD + zc] = pre[u];
                 }
-            } else if constexpr (!LIN) {
-                const int w = full ? idx / RUN : idx / run;
-                const int zc = idx - w * run;
-                if (idx < total) stage[w * LD + zc] = pre[u];
             }
         }
     };
 
-    // one column-buffer row: park it (its loads were issued two rows ago), refill
-    // the same registers with the row two below, then consume it from LDS
-    auto row_step = [&](PreT (&pre)[NP], int& lead_slot, int h) {
-        const bool live = h >= 0 && h < m && nw > 0;      // uniform over the workgroup
-        if (live) {
-            park(pre, lead_slot);
-            __syncthreads();
-        }
-        if (h - 2 >= h_bot) prefetch(pre, lead_slot, h - 2);
-        if (live) {
-#pragma unroll
-            for (int i = 0; i < NQ; ++i) {
-                if (!ok[i]) continue;
-                // tap t of pixel column wp: wo = r + t*SW from staged pixel wq - t;
-                // for one accumulator the taps come in ascending wo
-                const int wpp = wp[i] + PW;
-                const int r = wpp % SW, wq = wpp / SW;
-                const float* sp = stage + lead + (wq - w_lo) * LD + cq[i] * KK + r;
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    const int wo = r + t * SW, w = wq - t;
-                    if (wo < KW && w >= 0 && w <= w_hi) {
-                        const float* st = sp + t * (SW - LD);
-#pragma unroll
-                        for (int ho = 0; ho < KH; ++ho) acc[i][ho] += st[ho * KW];
-                    }
-                }
-            }
-            __syncthreads();
-        }
-        // image rows h*SH - PH + ho, ho >= KH - SH, are complete: write and slide
+    // image rows h*SH - PH + ho, ho >= KH - SH, can receive nothing from the rows
+    // below h: write them and slide the window down by SH
+    auto flush = [&](int h) __attribute__((always_inline)) {
         const int base = h * SH - PH;
 #pragma unroll
         for (int i = 0; i < NQ; ++i) {
@@ -473,12 +440,59 @@ __global__ __launch_bounds__(256) void col2im_stream_kernel(
             for (int ho = 0; ho < SH; ++ho) acc[i][ho] = 0.0f;
         }
     };
-    prefetch(pre0, lead0, h_top);
-    if (h_top - 1 >= h_bot) prefetch(pre1, lead1, h_top - 1);
-    for (int h = h_top; h >= h_bot; h -= 2) {
-        row_step(pre0, lead0, h);
-        if (h - 1 >= h_bot) row_step(pre1, lead1, h - 1);
+
+    // one live column-buffer row: park it (its loads were issued two rows ago),
+    // refill the same registers with the row two below, then consume it from LDS
+    // STEADY: the row two below is known to be live, so the refill is unconditional
+    auto row_step = [&](auto steady, PreT (&pre)[NP], int& lead_slot, int h) __attribute__((always_inline)) {
+        park(pre, lead_slot);
+        __syncthreads();
+        if (decltype(steady)::value || h - 2 >= live_lo) prefetch(pre, lead_slot, h - 2);
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            if (!ok[i]) continue;
+            // tap t of pixel column wp: wo = r + t*SW from staged pixel wq - t;
+            // for one accumulator the taps come in ascending wo
+            const int wpp = wp[i] + PW;
+            const int r = wpp % SW, wq = wpp / SW;
+            const float* sp = stage + lead + (wq - w_lo) * LD + cq[i] * KK + r;
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const int wo = r + t * SW, w = wq - t;
+                if (wo < KW && w >= 0 && w <= w_hi) {
+                    const float* st = sp + t * (SW - LD);
+#pragma unroll
+                    for (int ho = 0; ho < KH; ++ho) acc[i][ho] += st[ho * KW];
+                }
+            }
+        }
+        __syncthreads();
+        flush(h);
+    };
+    for (int hd = h_top; hd > live_hi; --hd) flush(hd);
+    // The steady loop has no branch around a load: where a load is skipped on
+    // some path, the compiler must assume on the other that nothing was issued
+    // after it and waits for the whole queue, which would leave one row in
+    // flight instead of two.  The last rows run in a second, conditional loop.
+    int h = live_hi;
+    if (h - 3 >= live_lo) {
+        prefetch(pre0, lead0, h);
+        __builtin_amdgcn_sched_barrier(0);            // keep the issue order the loop's waits count on
+        prefetch(pre1, lead1, h - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        for (; h - 3 >= live_lo; h -= 2) {
+            row_step(std::true_type(), pre0, lead0, h);
+            row_step(std::true_type(), pre1, lead1, h - 1);
+        }
+    } else if (h >= live_lo) {
+        prefetch(pre0, lead0, h);
+        if (h - 1 >= live_lo) prefetch(pre1, lead1, h - 1);
     }
+    for (; h >= live_lo; h -= 2) {
+        row_step(std::false_type(), pre0, lead0, h);
+        if (h - 1 >= live_lo) row_step(std::false_type(), pre1, lead1, h - 1);
+    }
+    for (int hd = live_lo - 1; hd >= h_bot; --hd) flush(hd);
     // rows of the band below the lowest window (still open in the window)
     const int base = (h_bot - 1) * SH - PH;
 #pragma unroll
@@ -499,12 +513,15 @@ static int launch_col2im_stream(G g, const float* col, long B, int C, int H, int
     constexpr int KK = G::kKH * G::kKW, RUN = CC * KK, LD = RUN | 1, TW = LW * WSUB;
     const int tiles_w = (int)cdiv(W, TW), nchunks = (int)cdiv(C, CC);
     const long nwb = std::min((long)n, (long)(TW + G::kKW - 2) / G::kSW + 1);
-    const size_t lds = ((size_t)nwb * LD + 8) * sizeof(float);
+    // linear staging parks NP * 256 aligned 16-byte units whatever the row needs
+    constexpr int NWB = (TW + G::kKW - 2) / G::kSW + 1;
+    constexpr size_t lin_units = (size_t)(((NWB * RUN + 6) / 4 + 255) / 256) * 256;
+    const size_t lds = std::max(((size_t)nwb * LD + 8) * sizeof(float), LD == RUN ? lin_units * 16 : 0);
     CGT_ARG_CHECK(lds <= 64 * 1024, "col2im: tile configuration out of range");
     const long Z = (long)C * KK;
     const long col_floats = B * m * (long)n * Z;
     const bool al16 = reinterpret_cast<uintptr_t>(col) % 16 == 0;
-    const int mode = (LD == RUN && C == CC && al16) ? kStageLinear
+    const int mode = (LD == RUN && C == CC && al16 && col_floats % 4 == 0) ? kStageLinear
                      : (RUN % 4 == 0 && C % CC == 0 && al16) ? kStageRuns : kStageScalar;
     auto kernel = mode == kStageLinear ? col2im_stream_kernel<G, CC, WSUB, (LD == RUN ? kStageLinear : kStageScalar), LW>
                   : mode == kStageRuns ? col2im_stream_kernel<G, CC, WSUB, (RUN % 4 == 0 ? kStageRuns : kStageScalar), LW>
@@ -525,7 +542,7 @@ static int launch_col2im_stream(G g, const float* col, long B, int C, int H, int
     const long blocks = per_band * bands;
     CGT_ARG_CHECK(blocks < (1L << 31), "col2im: too many workgroups");
     kernel<<<dim3((unsigned)blocks), dim3(256), lds, st>>>(g, col, im, C, H, W, m, n, band, (int)bands,
-                                                           tiles_w, nchunks, col_floats);
+                                                           tiles_w, nchunks);
     CGT_LAUNCH_CHECK("col2im_stream_kernel");
     return CGT_AMD_OK;
 }

@@ -21,10 +21,14 @@ __global__ __launch_bounds__(256) void batched_transpose_kernel(
     float* dst = out + b * (long)R * Cn;
     const int lx = threadIdx.x % kTile, ly = threadIdx.x / kTile;  // 64 x 4
     const int r0 = tr * kTile, c0 = tc * kTile;
-    for (int i = ly; i < kTile; i += 4) {
-        const int r = r0 + i, c = c0 + lx;
-        if (r < R && c < Cn) tile[i][lx] = src[(long)r * Cn + c];
-    }
+    // all 16 loads of a thread are issued before the first LDS store; rows and
+    // columns past the edge are clamped, not skipped, so no load is conditional
+    float v[kTile / 4];
+    const int c = min(c0 + lx, Cn - 1);
+#pragma unroll
+    for (int k = 0; k < kTile / 4; ++k) v[k] = src[(long)min(r0 + ly + 4 * k, R - 1) * Cn + c];
+#pragma unroll
+    for (int k = 0; k < kTile / 4; ++k) tile[ly + 4 * k][lx] = v[k];
     __syncthreads();
     for (int i = ly; i < kTile; i += 4) {
         const int c = c0 + i, r = r0 + lx;
@@ -80,17 +84,37 @@ __global__ __launch_bounds__(256) void thin_transpose_kernel(const float* __rest
     const int n = rows * L;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     if (L_INNER_IN) {
+        // All loads of a pass are issued before the first LDS store, and none is
+        // skipped (indices past the end are clamped): a load that some lanes skip
+        // makes the compiler wait for the whole memory queue before the next one.
         if (VEC) {
-            for (int i = threadIdx.x * 4; i < n; i += 1024) {
-                const float4 v = *reinterpret_cast<const float4*>(blk_in + i);
-                const int r = div_small(i, L, rL), c = i - r * L;
-                float* t = tile + r * LD + c;
-                t[0] = v.x; t[1] = v.y; t[2] = v.z; t[3] = v.w;
+            constexpr int U = kThinRows * kThinMaxL / 1024;      // covers the largest block in one pass
+            v4f v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = *reinterpret_cast<const v4f*>(blk_in + min((int)threadIdx.x * 4 + u * 1024, n - 4));
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int i = threadIdx.x * 4 + u * 1024;
+                if (i < n) {
+                    const int r = div_small(i, L, rL), c = i - r * L;
+                    float* t = tile + r * LD + c;
+                    t[0] = v[u].x; t[1] = v[u].y; t[2] = v[u].z; t[3] = v[u].w;
+                }
             }
         } else {
-            for (int i = threadIdx.x; i < n; i += 256) {
-                const int r = div_small(i, L, rL), c = i - r * L;
-                tile[r * LD + c] = blk_in[i];
+            constexpr int U = 8;
+            for (int i0 = threadIdx.x; i0 < n; i0 += 256 * U) {
+                float v[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) v[u] = blk_in[min(i0 + u * 256, n - 1)];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int i = i0 + u * 256;
+                    if (i < n) {
+                        const int r = div_small(i, L, rL), c = i - r * L;
+                        tile[r * LD + c] = v[u];
+                    }
+                }
             }
         }
         __syncthreads();

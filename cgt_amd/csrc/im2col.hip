@@ -68,9 +68,19 @@ __global__ __launch_bounds__(kIm2colThreads) void im2col_rows_kernel(
         const bool rowok = hp >= 0 && hp < H;
         const float* src = im + ((b * C + c0 + c) * (long)H + (rowok ? hp : 0)) * W;
         float* dst = tile + r * Wp;
-        for (int x = lane; x < Wp; x += kWave) {
-            const int wp = x - g.pw();
-            dst[x] = (rowok && wp >= 0 && wp < W) ? src[wp] : 0.0f;
+        // four loads in flight per lane; padding reads the row's first float and is zeroed
+        for (int x0 = lane; x0 < Wp; x0 += 4 * kWave) {
+            float v[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int wp = x0 + k * kWave - g.pw();
+                v[k] = src[(wp >= 0 && wp < W) ? wp : 0];
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int x = x0 + k * kWave, wp = x - g.pw();
+                if (x < Wp) dst[x] = (rowok && wp >= 0 && wp < W) ? v[k] : 0.0f;
+            }
         }
     }
     __syncthreads();
@@ -142,16 +152,24 @@ __global__ __launch_bounds__(kIm2colThreads) void im2col_pipe_kernel(
         const int hp = hbase + ho, wp = x - g.pw();
         soff[i] = (e < buflen && hp >= 0 && hp < H && wp >= 0 && wp < W) ? (int)(c * plane + hp * W + wp) : -1;
     }
+    // Every thread issues all NI loads, padding included (those read the chunk's
+    // first float and are zeroed afterwards): a load that some lanes skip sits
+    // behind a branch, and the compiler then drains the memory queue before
+    // each following load instead of keeping NI of them in flight.
     float reg[NI];
-    auto load = [&](int ck) {
+    auto load = [&](int ck) __attribute__((always_inline)) {
         const int c0 = ck * chunk;
         const int lim = min(chunk, C - c0) * rowlen;
         const float* base = im + (b * C + c0) * plane;
+        bool ok[NI];
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             const int e = threadIdx.x + i * kIm2colThreads;
-            reg[i] = (soff[i] >= 0 && e < lim) ? base[soff[i]] : 0.0f;
+            ok[i] = soff[i] >= 0 && e < lim;
+            reg[i] = base[ok[i] ? soff[i] : 0];
         }
+#pragma unroll
+        for (int i = 0; i < NI; ++i) reg[i] = ok[i] ? reg[i] : 0.0f;
     };
     auto stash = [&](float* buf) {
 #pragma unroll
@@ -203,6 +221,116 @@ __global__ __launch_bounds__(kIm2colThreads) void im2col_pipe_kernel(
         }
         if (more) stash(tile + ((ck + 1) & 1) * buflen);
         __syncthreads();
+    }
+}
+
+// Linear writer for rows that are not a whole number of 16-byte units (Z % 4 != 0,
+// e.g. 3 x 11 x 11 = 363).  With all channels staged at once, the workgroup's
+// output -- the n*Z floats of row (b, h) -- is ONE contiguous region.  It is
+// written as aligned 16-byte units wherever its first float falls: unit q holds
+// floats f = head + 4q .. +3 of the region, float f is pixel w = f / Z, element
+// z = f % Z, and since z = (c*kh + ho)*kw + wo the staged value sits at LDS row
+// z / kw, column w*sw + z % kw -- one division by a compile-time constant per
+// float.  (w, z) advance by a fixed step per pass, so nothing is divided by Z
+// inside the loop.  The up to three floats before the first and after the last
+// whole unit are written singly.
+template <class G, int NI>
+__global__ __launch_bounds__(kIm2colThreads) void im2col_linear_kernel(
+    G g, const float* __restrict__ im, float* __restrict__ col, int C, int H, int W, int m, int n) {
+    extern __shared__ float tile[];  // [C*kh][Wp]
+    constexpr int KH = G::kKH, KW = G::kKW, SW = G::kSW;
+    static_assert(KW >= 3, "a unit of four floats may carry only once out of the kernel column");
+    const int Wp = W + 2 * g.pw();
+    const int rowlen = KH * Wp;
+    const int buflen = C * rowlen;               // <= NI * 256
+    const long bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int h = (int)(bid % m);
+    const long b = bid / m;
+    const int hbase = h * g.sh() - g.ph();
+    const long plane = (long)H * W;
+    const float* base = im + b * C * plane;
+
+    float reg[NI];
+    bool ok[NI];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int e = threadIdx.x + i * kIm2colThreads;
+        const int c = e / rowlen, rem = e - c * rowlen;
+        const int ho = rem / Wp, x = rem - ho * Wp;
+        const int hp = hbase + ho, wp = x - g.pw();
+        ok[i] = e < buflen && hp >= 0 && hp < H && wp >= 0 && wp < W;
+        reg[i] = base[ok[i] ? (int)(c * plane + hp * W + wp) : 0];
+    }
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int e = threadIdx.x + i * kIm2colThreads;
+        if (e < buflen) tile[e] = ok[i] ? reg[i] : 0.0f;
+    }
+    __syncthreads();
+
+    const int Z = C * KH * KW;
+    const int len = n * Z;                                   // floats in the region
+    const long start = (b * m + h) * (long)len;              // col is 16-byte aligned
+    float* out = col + start;
+    const int head = (int)((4 - (start & 3)) & 3);
+    const int nunits = len > head ? (len - head) >> 2 : 0;
+    auto value = [&](int w, int z) __attribute__((always_inline)) {
+        if (z >= Z) {
+            z -= Z;
+            ++w;
+        }
+        const int row = z / KW, wo = z - row * KW;
+        return tile[row * Wp + w * SW + wo];
+    };
+    // First unit of this thread by division, then everything advances by fixed
+    // steps: a pass moves on by 4*256 floats = dw pixels, dr LDS rows and dk
+    // kernel columns, with a carry from the kernel column into the row and from
+    // the row (past the last one, R - 1) into the pixel.  Only the LDS offset is
+    // kept up to date; the three floats after the first differ from it by j,
+    // plus the same two carries.
+    const int R = C * KH;
+    const int up_row = Wp - KW;                  // offset change when the kernel column wraps
+    const int up_pix = SW - R * Wp;              // ... when the row wraps into the next pixel
+    int f = head + 4 * (int)threadIdx.x;
+    int rho, kc, addr;
+    {
+        const int w = f / Z, z = f - w * Z;
+        rho = z / KW;
+        kc = z - rho * KW;
+        addr = rho * Wp + w * SW + kc;
+    }
+    const int step = 4 * kIm2colThreads;
+    const int dw = step / Z, dz = step - dw * Z;
+    const int dr = dz / KW, dk = dz - dr * KW;
+    const int da = dw * SW + dr * Wp + dk;
+    for (int q = threadIdx.x; q < nunits; q += kIm2colThreads) {
+        float v[4];
+        v[0] = tile[addr];
+        const bool last_row = rho == R - 1;
+#pragma unroll
+        for (int j = 1; j < 4; ++j) {
+            const bool carry = kc + j >= KW;     // one carry at most: kc + 3 < 2 * KW
+            int a = addr + j + (carry ? up_row : 0);
+            a += (carry && last_row) ? up_pix : 0;
+            v[j] = tile[a];
+        }
+        stream_store4(out + f, v[0], v[1], v[2], v[3]);
+        f += step;
+        kc += dk;
+        const bool c1 = kc >= KW;
+        kc -= c1 ? KW : 0;
+        rho += dr + (c1 ? 1 : 0);
+        addr += da + (c1 ? up_row : 0);
+        const bool c2 = rho >= R;
+        rho -= c2 ? R : 0;
+        addr += c2 ? up_pix : 0;
+    }
+    // edges: floats [0, head) and [head + 4*nunits, len)
+    const int tail0 = head + 4 * nunits;
+    const int e = (int)threadIdx.x < head ? (int)threadIdx.x : tail0 + (int)threadIdx.x - head;
+    if (e < len && ((int)threadIdx.x < head || e >= tail0)) {
+        const int we = e / Z;
+        out[e] = value(we, e - we * Z);
     }
 }
 
@@ -563,6 +691,13 @@ static int check_geom(const char* what, long B, long C, long H, long W, int kh, 
 
 static int gcd4(int v) { return (v % 4 == 0) ? 4 : (v % 2 == 0) ? 2 : 1; }
 
+// the linear writer needs the kernel width at compile time, and at least 3
+template <class G>
+constexpr bool linear_writer_ok() {
+    if constexpr (G::is_static) return G::kKW >= 3;
+    else return false;
+}
+
 template <class G>
 static int launch_im2col(G g, const float* im, long B, int C, int H, int W, int m, int n,
                          float* col, hipStream_t st) {
@@ -608,6 +743,18 @@ static int launch_im2col(G g, const float* im, long B, int C, int H, int W, int 
         const long blocks = B * m;
         const bool small = (long)chunk * rowlen <= 12 * kIm2colThreads;
         dim3 grid((unsigned)blocks), block(kIm2colThreads);
+        if constexpr (linear_writer_ok<G>()) {
+            // odd row length, all channels in one buffer: aligned 16-byte units over the linear region
+            if (!vec && nchunks == 1 && Z % 4 != 0 && reinterpret_cast<uintptr_t>(col) % 16 == 0 &&
+                (long)n * Z < (1L << 30) && (long)chunk * rowlen <= 32 * kIm2colThreads) {
+                if ((long)chunk * rowlen <= 12 * kIm2colThreads)
+                    im2col_linear_kernel<G, 12><<<grid, block, lds, st>>>(g, im, col, C, H, W, m, n);
+                else
+                    im2col_linear_kernel<G, 32><<<grid, block, lds, st>>>(g, im, col, C, H, W, m, n);
+                CGT_LAUNCH_CHECK("im2col_linear_kernel");
+                return CGT_AMD_OK;
+            }
+        }
         if (whole && vec)
             im2col_pipe_kernel<G, true, 32><<<grid, block, lds, st>>>(g, im, col, C, H, W, m, n, chunk, nchunks);
         else if (whole)

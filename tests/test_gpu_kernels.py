@@ -108,6 +108,12 @@ IM2COL_CASES = [
     ((2, 6, 9, 20), (5, 5), (2, 2), (1, 1)),       # 5x5, 32 lanes per row, partial chunk
     ((2, 12, 10, 10), (5, 5), (2, 2), (1, 1)),     # 5x5, 16 lanes per row, partial chunk
     ((4, 64, 15, 15), (5, 5), (2, 2), (1, 1)),     # CIFAR conv2 at full channel count
+    # odd Z with every channel staged at once: the row's region is written as aligned 16-byte units
+    ((5, 3, 23, 27), (11, 11), (0, 0), (4, 4)),    # Z = 363, regions of 1815 floats: every start alignment
+    ((3, 5, 9, 11), (3, 3), (1, 1), (1, 1)),       # Z = 45, a region shorter than one pass
+    ((6, 1, 6, 7), (3, 3), (0, 0), (1, 1)),        # Z = 9: a unit straddles pixels, three LDS rows in all
+    ((2, 13, 20, 57), (11, 11), (0, 0), (4, 4)),   # Z = 1573 > one pass of 1024 floats
+    ((3, 7, 40, 41), (5, 5), (2, 2), (1, 1)),      # Z = 175, several passes per region
 ]
 
 

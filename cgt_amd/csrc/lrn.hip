@@ -110,6 +110,75 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_fwd_kernel(
     else lrn_fwd_run<SIZE, false>(x, top, scale, C, HW, blk, crun, aos, nbeta, kconst);
 }
 
+// Flat variant for large arrays.  The stores are two thirds of the forward
+// traffic, and the pixel-per-lane kernel issues them 4 bytes per lane (straddling
+// cache lines when H*W is odd, as 55*55).
+// Here a thread owns one aligned unit of four consecutive floats of the flat
+// [N*C*H*W] array and writes both outputs with streamed 16-byte stores.  Its four
+// pixels lie in one channel plane (units that straddle two planes, one in
+// H*W/4, take an element-wise path), so the window is SIZE unaligned 16-byte
+// loads H*W floats apart.  Each input float is fetched SIZE times, but only
+// the first fetch goes to HBM: neighbouring channels of the same pixels are
+// loaded by workgroups close by in the grid and meet in L2.
+typedef float v4f_unaligned __attribute__((ext_vector_type(4), aligned(4)));
+
+template <int SIZE>
+__global__ __launch_bounds__(kLrnThreads) void lrn_fwd_flat_kernel(
+    const float* __restrict__ x, float* __restrict__ top, float* __restrict__ scale, int C,
+    int HW, unsigned total, float aos, float nbeta, float kconst) {
+    constexpr int PRE = (SIZE - 1) / 2;
+    // each XCD (one L2) takes a contiguous range of the flat array, so the SIZE
+    // fetches of a float come from one L2
+    const unsigned nblk = gridDim.x, q = nblk / kNumXCD, r = nblk % kNumXCD;
+    const unsigned xcd = blockIdx.x % kNumXCD, local = blockIdx.x / kNumXCD;
+    const unsigned bid = xcd * q + min(xcd, r) + local;
+    const unsigned f = 4u * (bid * kLrnThreads + threadIdx.x);
+    if (f >= total) return;
+    const unsigned plane = f / (unsigned)HW;             // image * C + channel
+    const int p0 = (int)(f - plane * (unsigned)HW);
+    const int c0 = (int)(plane % (unsigned)C);
+    if (p0 + 3 < HW && f + 3 < total) {
+        v4f w[SIZE];
+        bool ok[SIZE];
+#pragma unroll
+        for (int j = 0; j < SIZE; ++j) {
+            const int c = c0 - PRE + j;
+            ok[j] = c >= 0 && c < C;
+            // outside the window the unit's own address is loaded and discarded: no load is conditional
+            const long at = ok[j] ? (long)f + (long)(j - PRE) * HW : (long)f;
+            w[j] = *reinterpret_cast<const v4f_unaligned*>(x + at);
+        }
+        const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
+        v4f acc = zero;
+#pragma unroll
+        for (int j = 0; j < SIZE; ++j) {
+            const v4f v = ok[j] ? w[j] : zero;
+            acc += v * v;
+        }
+        const v4f s = kconst + acc * aos;
+        const v4f mid = w[PRE];
+        stream_store4(scale + f, s.x, s.y, s.z, s.w);
+        stream_store4(top + f, mid.x * pow_neg_beta(s.x, nbeta), mid.y * pow_neg_beta(s.y, nbeta),
+                      mid.z * pow_neg_beta(s.z, nbeta), mid.w * pow_neg_beta(s.w, nbeta));
+        return;
+    }
+    for (unsigned e = f; e < f + 4 && e < total; ++e) {
+        const unsigned pl = e / (unsigned)HW;
+        const int c = (int)(pl % (unsigned)C);
+        float acc = 0.0f;
+        for (int j = 0; j < SIZE; ++j) {
+            const int cc = c - PRE + j;
+            if (cc >= 0 && cc < C) {
+                const float v = x[(long)e + (long)(j - PRE) * HW];
+                acc += v * v;
+            }
+        }
+        const float s = kconst + acc * aos;
+        scale[e] = s;
+        top[e] = x[e] * pow_neg_beta(s, nbeta);
+    }
+}
+
 // Any window length: re-reads the window through the cache.
 __global__ __launch_bounds__(kLrnThreads) void lrn_fwd_generic_kernel(
     const float* __restrict__ x, float* __restrict__ top, float* __restrict__ scale, int C,
@@ -281,9 +350,18 @@ CGT_API int cgt_amd_lrn_fwd_f32(const float* x, long N, long C, long H, long W, 
     dim3 grid((unsigned)(cdiv(HW, kLrnThreads) * cdiv(C, crun) * N)), block(kLrnThreads);
     hipStream_t st = as_stream(stream);
     const float aos = (float)(alpha / size), nbeta = (float)(-beta), kc = (float)k;
+    const long total = N * C * HW;
+    // the flat kernel wins once the arrays no longer sit in the last-level cache
+    // (measured: 37 M floats 0.066 vs 0.098 ms, 24 M 0.051 vs 0.067, 9 M 0.022 vs 0.017)
+    const bool flat = total >= (16L << 20) && total < (1L << 31) && reinterpret_cast<uintptr_t>(top) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(scale) % 16 == 0;
+    const dim3 flat_grid((unsigned)cdiv(cdiv(total, 4), kLrnThreads));
 #define LRN_FWD_CASE(S)                                                                           \
     case S:                                                                                       \
-        lrn_fwd_kernel<S><<<grid, block, 0, st>>>(x, top, scale, (int)C, HW, crun, aos, nbeta, kc); \
+        if (flat)                                                                                 \
+            lrn_fwd_flat_kernel<S><<<flat_grid, block, 0, st>>>(x, top, scale, (int)C, HW, (unsigned)total, aos, nbeta, kc); \
+        else                                                                                      \
+            lrn_fwd_kernel<S><<<grid, block, 0, st>>>(x, top, scale, (int)C, HW, crun, aos, nbeta, kc); \
         break;
     switch (size) {
         LRN_FWD_CASE(1) LRN_FWD_CASE(2) LRN_FWD_CASE(3) LRN_FWD_CASE(4) LRN_FWD_CASE(5)

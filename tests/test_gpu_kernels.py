@@ -233,6 +233,22 @@ def test_lrn_vs_oracle(K, shape, size, alpha, beta, k):
         assert relfro(gb, tgb) <= 1e-5
 
 
+@pytest.mark.parametrize("shape,size", [((5, 7, 701, 685), 5), ((5, 7, 701, 685), 4), ((2, 9, 1024, 1024), 3)])
+def test_lrn_forward_large_arrays(K, shape, size):
+    # >= 16 M floats: the forward pass takes the kernel that owns aligned units of
+    # the flat array.  Odd plane and odd total (units that straddle planes, a
+    # partial last unit), few channels (window mostly clipped), and an aligned case.
+    print("lrn large case", shape, size, flush=True)
+    rs = np.random.RandomState(4)
+    x = rs.randn(*shape).astype(np.float32)
+    rtop, rscale = O.lrn_fwd(x, size, 0.3, 0.75, 1.0)
+    top, scale = K.lrn_fwd(gpu(x), size, 0.3, 0.75, 1.0)
+    top, scale = top.get(), scale.get()
+    assert relfro(scale, rscale) <= 1e-6 and relfro(top, rtop) <= 5e-6
+    assert np.max(np.abs(scale - rscale) / rscale) <= 1e-5
+    assert np.max(np.abs(top - rtop) / (np.abs(rtop) + 1e-6)) <= 1e-4
+
+
 def test_lrn_rejects_size_above_channels(K):
     from cgt_amd.capi import CgtAmdError
     x = gpu(np.zeros((1, 3, 2, 2), np.float32))

@@ -418,15 +418,25 @@ __global__ __launch_bounds__(256) void col2im_gather_kernel(
 // 16-byte boundary below its first float, whatever its alignment, and lands in
 // LDS at the same offset from that boundary, with no index arithmetic at all).
 constexpr int kStageScalar = 0, kStageRuns = 1, kStageLinear = 2;
+constexpr int kRowBatch = 8;   // image rows collected per channel before they are written (a multiple of every static stride)
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in order
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>());
+    }
+}
 
 //
 // LW = lanes along the image row per wavefront (64, 32 or 16): narrow images
 // (CIFAR's 15-wide feature maps) put 64/LW channels side by side in a
 // wavefront instead of leaving lanes idle.
-template <class G, int CC, int WSUB, int MODE, int LW = 64>
+template <class G, int CC, int WSUB, int MODE, int LW = 64, bool BATCH = false>
 __global__ __launch_bounds__(256) void col2im_stream_kernel(
     G g, const float* __restrict__ col, float* __restrict__ im, int C, int H, int W, int m, int n,
-    int band, int bands, int tiles_w, int nchunks) {
+    int band, int bands, int tiles_w, int nchunks, int out_off) {
     constexpr bool VEC = MODE == kStageRuns, LIN = MODE == kStageLinear;
     constexpr int KH = G::kKH, KW = G::kKW, PH = G::kPH, PW = G::kPW, SH = G::kSH, SW = G::kSW;
     static_assert(SH <= KH && SW <= KW, "streaming col2im needs stride <= kernel");
@@ -548,20 +558,61 @@ __global__ __launch_bounds__(256) void col2im_stream_kernel(
         }
     };
 
+    // Finished image rows leave the window from the top of the band downwards.
+    // Written one by one they are short stores (W floats per wavefront
+    // instruction, a tenth of the kernel's bytes but a quarter of its time);
+    // with BATCH (the tile spans the whole image width, so a channel's rows are
+    // adjacent in memory) they are collected in LDS, kRowBatch rows of every
+    // channel of the chunk, and each channel's batch is written as one linear
+    // region in aligned, streamed 16-byte units.
+    constexpr int RB = kRowBatch;
+    float* obuf = stage + out_off;                    // [CC][RB][W]
+    int batch_lo = hp0 + (hp1 - 1 - hp0) / RB * RB;   // lowest row of the batch being collected
+    auto write_batch = [&]() __attribute__((always_inline)) {
+        const int rows = min(batch_lo + RB, hp1) - batch_lo;
+        const int nfl = rows * W;
+        __syncthreads();
+        for (int c = wave; c < cc; c += 4) {
+            const long g0 = ((b * C + c0 + c) * (long)H + batch_lo) * W;   // im is 16-byte aligned
+            float* dst = im + g0;
+            const float* src = obuf + c * RB * W;
+            const int head = min((int)((4 - (g0 & 3)) & 3), nfl);
+            const int nunits = (nfl - head) >> 2;
+            for (int u = lane; u < nunits; u += 64) {
+                const int e = head + 4 * u;
+                stream_store4(dst + e, src[e], src[e + 1], src[e + 2], src[e + 3]);
+            }
+            const int tail0 = head + 4 * nunits;
+            if (lane < head) dst[lane] = src[lane];
+            if (tail0 + lane < nfl) dst[tail0 + lane] = src[tail0 + lane];
+        }
+        __syncthreads();
+    };
+    // one finished image row: ho is the window slot that holds it
+    auto emit_row = [&](int hp, auto slot) __attribute__((always_inline)) {
+        constexpr int ho = decltype(slot)::value;
+        if (hp < hp0 || hp >= hp1) return;            // uniform over the workgroup
+        if constexpr (BATCH) {
+            if (hp < batch_lo) {
+                write_batch();
+                batch_lo -= RB;
+            }
+#pragma unroll
+            for (int i = 0; i < NQ; ++i)
+                if (ok[i]) obuf[(cq[i] * RB + hp - batch_lo) * W + wp[i]] = acc[i][ho];
+        } else {
+#pragma unroll
+            for (int i = 0; i < NQ; ++i)
+                if (ok[i]) im[(((b * C + c0 + cq[i]) * (long)H) + hp) * W + wp[i]] = acc[i][ho];
+        }
+    };
     // image rows h*SH - PH + ho, ho >= KH - SH, can receive nothing from the rows
-    // below h: write them and slide the window down by SH
+    // below h: emit them (highest first) and slide the window down by SH
     auto flush = [&](int h) __attribute__((always_inline)) {
         const int base = h * SH - PH;
+        static_for<SH>([&](auto k) { emit_row(base + KH - 1 - k, std::integral_constant<int, KH - 1 - decltype(k)::value>()); });
 #pragma unroll
         for (int i = 0; i < NQ; ++i) {
-            if (ok[i]) {
-                float* dst = im + ((b * C + c0 + cq[i]) * (long)H) * W + wp[i];
-#pragma unroll
-                for (int ho = KH - SH; ho < KH; ++ho) {
-                    const int hp = base + ho;
-                    if (hp >= hp0 && hp < hp1) dst[(long)hp * W] = acc[i][ho];
-                }
-            }
 #pragma unroll
             for (int ho = KH - 1; ho >= SH; --ho) acc[i][ho] = acc[i][ho - SH];
 #pragma unroll
@@ -623,16 +674,8 @@ __global__ __launch_bounds__(256) void col2im_stream_kernel(
     for (int hd = live_lo - 1; hd >= h_bot; --hd) flush(hd);
     // rows of the band below the lowest window (still open in the window)
     const int base = (h_bot - 1) * SH - PH;
-#pragma unroll
-    for (int i = 0; i < NQ; ++i) {
-        if (!ok[i]) continue;
-        float* dst = im + ((b * C + c0 + cq[i]) * (long)H) * W + wp[i];
-#pragma unroll
-        for (int ho = SH; ho < KH; ++ho) {
-            const int hp = base + ho;
-            if (hp >= hp0 && hp < hp1) dst[(long)hp * W] = acc[i][ho];
-        }
-    }
+    static_for<KH - SH>([&](auto k) { emit_row(base + KH - 1 - k, std::integral_constant<int, KH - 1 - decltype(k)::value>()); });
+    if constexpr (BATCH) write_batch();
 }
 
 template <class G, int CC, int WSUB, int LW = 64>
@@ -644,16 +687,27 @@ static int launch_col2im_stream(G g, const float* col, long B, int C, int H, int
     // linear staging parks NP * 256 aligned 16-byte units whatever the row needs
     constexpr int NWB = (TW + G::kKW - 2) / G::kSW + 1;
     constexpr size_t lin_units = (size_t)(((NWB * RUN + 6) / 4 + 255) / 256) * 256;
-    const size_t lds = std::max(((size_t)nwb * LD + 8) * sizeof(float), LD == RUN ? lin_units * 16 : 0);
+    size_t lds = std::max(((size_t)nwb * LD + 8) * sizeof(float), LD == RUN ? lin_units * 16 : 0);
     CGT_ARG_CHECK(lds <= 64 * 1024, "col2im: tile configuration out of range");
     const long Z = (long)C * KK;
     const long col_floats = B * m * (long)n * Z;
     const bool al16 = reinterpret_cast<uintptr_t>(col) % 16 == 0;
     const int mode = (LD == RUN && C == CC && al16 && col_floats % 4 == 0) ? kStageLinear
                      : (RUN % 4 == 0 && C % CC == 0 && al16) ? kStageRuns : kStageScalar;
-    auto kernel = mode == kStageLinear ? col2im_stream_kernel<G, CC, WSUB, (LD == RUN ? kStageLinear : kStageScalar), LW>
-                  : mode == kStageRuns ? col2im_stream_kernel<G, CC, WSUB, (RUN % 4 == 0 ? kStageRuns : kStageScalar), LW>
-                                       : col2im_stream_kernel<G, CC, WSUB, kStageScalar, LW>;
+    // a tile as wide as the image: finished rows are batched in LDS behind the staging area
+    const size_t out_off = (lds / sizeof(float) + 3) / 4 * 4;
+    const size_t lds_batch = (out_off + (size_t)CC * kRowBatch * W) * sizeof(float);
+    // (not for narrow images: a batch of a 15-wide plane is a few hundred bytes, and the two
+    // extra barriers per batch cost more than the stores gain -- 0.019 vs 0.016 ms on CIFAR conv2)
+    const bool batch = tiles_w == 1 && W >= 32 && reinterpret_cast<uintptr_t>(im) % 16 == 0 && lds_batch <= 40 * 1024;
+    if (batch) lds = lds_batch;
+    constexpr int M_LIN = LD == RUN ? kStageLinear : kStageScalar, M_RUNS = RUN % 4 == 0 ? kStageRuns : kStageScalar;
+    auto kernel = batch ? (mode == kStageLinear ? col2im_stream_kernel<G, CC, WSUB, M_LIN, LW, true>
+                           : mode == kStageRuns ? col2im_stream_kernel<G, CC, WSUB, M_RUNS, LW, true>
+                                                : col2im_stream_kernel<G, CC, WSUB, kStageScalar, LW, true>)
+                        : (mode == kStageLinear ? col2im_stream_kernel<G, CC, WSUB, M_LIN, LW, false>
+                           : mode == kStageRuns ? col2im_stream_kernel<G, CC, WSUB, M_RUNS, LW, false>
+                                                : col2im_stream_kernel<G, CC, WSUB, kStageScalar, LW, false>);
     // Bands of image rows: as many workgroups as the chip holds at once, and
     // no more.  The kernel is bound by the loads each wavefront can keep in
     // flight, so resident wavefronts are what counts; a second, partial round
@@ -670,7 +724,7 @@ static int launch_col2im_stream(G g, const float* col, long B, int C, int H, int
     const long blocks = per_band * bands;
     CGT_ARG_CHECK(blocks < (1L << 31), "col2im: too many workgroups");
     kernel<<<dim3((unsigned)blocks), dim3(256), lds, st>>>(g, col, im, C, H, W, m, n, band, (int)bands,
-                                                           tiles_w, nchunks);
+                                                           tiles_w, nchunks, (int)out_off);
     CGT_LAUNCH_CHECK("col2im_stream_kernel");
     return CGT_AMD_OK;
 }

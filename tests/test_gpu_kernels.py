@@ -108,6 +108,10 @@ IM2COL_CASES = [
     ((2, 6, 9, 20), (5, 5), (2, 2), (1, 1)),       # 5x5, 32 lanes per row, partial chunk
     ((2, 12, 10, 10), (5, 5), (2, 2), (1, 1)),     # 5x5, 16 lanes per row, partial chunk
     ((4, 64, 15, 15), (5, 5), (2, 2), (1, 1)),     # CIFAR conv2 at full channel count
+    # col2im with a tile as wide as the image: finished rows leave through LDS in batches of 8 per channel
+    ((2, 10, 37, 45), (3, 3), (1, 1), (1, 1)),     # odd width: batches start at any alignment, partial chunk, partial top batch
+    ((2, 8, 19, 64), (3, 3), (0, 0), (1, 1)),      # full 64-wide tile, no padding
+    ((1, 4, 70, 33), (5, 5), (2, 2), (1, 1)),      # 5x5, 32 lanes per row, several bands
     # odd Z with every channel staged at once: the row's region is written as aligned 16-byte units
     ((5, 3, 23, 27), (11, 11), (0, 0), (4, 4)),    # Z = 363, regions of 1815 floats: every start alignment
     ((3, 5, 9, 11), (3, 3), (1, 1), (1, 1)),       # Z = 45, a region shorter than one pass

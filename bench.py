@@ -55,12 +55,12 @@ DEFAULT_WORKLOAD = "vgg_mid_conv3x3_128x56x56_b64"
 # WRITE_SIZE runs of this script (summaries and calibration in profiles/):
 # (workload, stage) -> bytes.  None where no counter run has been made.
 TRAFFIC = {
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_fwd_NT"): 1087300000,    # 2.0 * 486.0 MB fetched + 115.3 MB written
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_dgrad_NN"): 1088800000,  # 2.0 * 82.0 + 924.8
+    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_fwd_NT"): 1088700000,    # 2.0 * 486.7 MB fetched + 115.3 MB written
+    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_dgrad_NN"): 1095000000,  # 2.0 * 85.1 + 924.8
     ("vgg_mid_conv3x3_128x56x56_b64", "gemm_wgrad_TN"): 1128100000,  # 2.0 * 531.0 + 66.1 (split-K partials incl.)
-    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_fwd_NT"): 828900000,     # 2.0 * 340.1 + 148.7
-    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_dgrad_NN"): 811500000,   # 2.0 * 106.8 + 597.9 (rows of 363 floats)
-    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_wgrad_TN"): 1099100000,  # 2.0 * 524.4 + 50.3 (partials incl.)
+    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_fwd_NT"): 830300000,     # 2.0 * 340.8 + 148.7
+    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_dgrad_NN"): 801100000,   # 2.0 * 101.4 + 598.3 (rows of 363 floats)
+    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_wgrad_TN"): 1087100000,  # 2.0 * 518.3 + 50.5 (partials incl.)
 }
 
 
@@ -118,7 +118,7 @@ class LayerOnGpu(object):
         nelem = lambda a: int(np.prod(a.shape))  # noqa: E731
         st = []
         s = stream
-        st.append(Stage("im2col", "im2col_pipe_kernel", lambda: K.im2col(self.x, (r, c), pad, stride, out=self.col, stream=s),
+        st.append(Stage("im2col", "im2col_pipe_kernel or im2col_linear_kernel", lambda: K.im2col(self.x, (r, c), pad, stride, out=self.col, stream=s),
                         4 * (nelem(self.x) + nelem(self.col)), "hbm"))
         st.append(Stage("gemm_fwd_NT", "sgemm_kernel", lambda: K.mul22(self.col2, self.f_LZ, False, True, out=self.y_mnL, stream=s),
                         2 * Bmn * L * Z, "mfma"))
@@ -128,7 +128,7 @@ class LayerOnGpu(object):
         if cfg["lrn"]:
             size, alpha, beta, k = cfg["lrn"]
             self.top, self.scale = empty(self.y.shape), empty(self.y.shape)
-            st.append(Stage("lrn_fwd", "lrn_fwd_kernel", lambda: K.lrn_fwd(self.y, size, alpha, beta, k, out=(self.top, self.scale), stream=s),
+            st.append(Stage("lrn_fwd", "lrn_fwd_flat_kernel or lrn_fwd_kernel", lambda: K.lrn_fwd(self.y, size, alpha, beta, k, out=(self.top, self.scale), stream=s),
                             3 * 4 * nelem(self.y), "hbm"))
             act = self.top
         if cfg["pool"]:

@@ -118,7 +118,7 @@ class LayerOnGpu(object):
         nelem = lambda a: int(np.prod(a.shape))  # noqa: E731
         st = []
         s = stream
-        st.append(Stage("im2col", "im2col_pipe_kernel or im2col_linear_kernel", lambda: K.im2col(self.x, (r, c), pad, stride, out=self.col, stream=s),
+        st.append(Stage("im2col", "im2col_linear_kernel or im2col_pipe_kernel", lambda: K.im2col(self.x, (r, c), pad, stride, out=self.col, stream=s),
                         4 * (nelem(self.x) + nelem(self.col)), "hbm"))
         st.append(Stage("gemm_fwd_NT", "sgemm_kernel", lambda: K.mul22(self.col2, self.f_LZ, False, True, out=self.y_mnL, stream=s),
                         2 * Bmn * L * Z, "mfma"))

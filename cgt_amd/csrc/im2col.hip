@@ -224,42 +224,114 @@ __global__ __launch_bounds__(kIm2colThreads) void im2col_pipe_kernel(
     }
 }
 
-// Linear writer for rows that are not a whole number of 16-byte units (Z % 4 != 0,
-// e.g. 3 x 11 x 11 = 363).  With all channels staged at once, the workgroup's
-// output -- the n*Z floats of row (b, h) -- is ONE contiguous region.  It is
-// written as aligned 16-byte units wherever its first float falls: unit q holds
-// floats f = head + 4q .. +3 of the region, float f is pixel w = f / Z, element
-// z = f % Z, and since z = (c*kh + ho)*kw + wo the staged value sits at LDS row
-// z / kw, column w*sw + z % kw -- one division by a compile-time constant per
-// float.  (w, z) advance by a fixed step per pass, so nothing is divided by Z
-// inside the loop.  The up to three floats before the first and after the last
-// whole unit are written singly.
+// Linear writer.  With ALL channels staged at once, the output for a run of tw
+// pixels of row (b, h) -- tw*Z floats -- is ONE contiguous region of the column
+// buffer, and a workgroup writes it front to back as aligned 16-byte units
+// wherever its first float falls (Z % 4 != 0, e.g. 3 x 11 x 11 = 363, moves the
+// start from row to row): unit q holds floats f = head + 4q .. +3 of the region,
+// float f is pixel f / Z, element z = f % Z, and since z = (c*kh + ho)*kw + wo
+// the staged value sits at LDS row z / kw, column pixel*sw + z % kw.  Both the
+// staging and the writing advance by fixed steps with carries, so there is no
+// division inside a loop.  The up to three floats before the first and after the
+// last whole unit are written singly.  tw is the whole row when the staged rows
+// of all channels fit (AlexNet conv1), else the widest tile that fits (VGG:
+// 128 channels x 3 rows x 16 columns, regions of 14 pixels = 63 KB).
 template <class G, int NI>
 __global__ __launch_bounds__(kIm2colThreads) void im2col_linear_kernel(
-    G g, const float* __restrict__ im, float* __restrict__ col, int C, int H, int W, int m, int n) {
-    extern __shared__ float tile[];  // [C*kh][Wp]
+    G g, const float* __restrict__ im, float* __restrict__ col, int C, int H, int W, int m, int n,
+    int tw, int ntiles) {
+    extern __shared__ float tile[];  // [C*kh][twi]
     constexpr int KH = G::kKH, KW = G::kKW, SW = G::kSW;
     static_assert(KW >= 3, "a unit of four floats may carry only once out of the kernel column");
-    const int Wp = W + 2 * g.pw();
-    const int rowlen = KH * Wp;
-    const int buflen = C * rowlen;               // <= NI * 256
-    const long bid = xcd_remap(blockIdx.x, gridDim.x);
-    const int h = (int)(bid % m);
-    const long b = bid / m;
+    unsigned bid = (unsigned)xcd_remap(blockIdx.x, gridDim.x);       // 32-bit: 64-bit divisions cost hundreds of instructions
+    const int wt = (int)(bid % (unsigned)ntiles);                    // tiles of a row are neighbours: their regions are adjacent
+    bid /= (unsigned)ntiles;
+    const int h = (int)(bid % (unsigned)m);
+    const long b = bid / (unsigned)m;
+    const int w0 = wt * tw, nw = min(tw, n - w0);
+    const int Wp = (tw - 1) * SW + KW;           // staged columns: image columns x0 .. x0 + Wp - 1
+    const int x0 = w0 * SW - g.pw();
+    const int R = C * KH;
+    const int buflen = R * Wp;                   // <= NI * 256
     const int hbase = h * g.sh() - g.ph();
     const long plane = (long)H * W;
     const float* base = im + b * C * plane;
 
+    // Element e of the staging area is LDS row e / Wp (= channel * kh + kernel row), column e % Wp.
+    // A thread's elements are 256 apart: a fixed step in (channel, kernel row, column) with a carry
+    // out of the column and one out of the kernel row; the image offset follows by additions.
     float reg[NI];
     bool ok[NI];
+    if constexpr (NI >= 32) {
+        // The largest staging areas decode each element by division instead.  That is several times
+        // the arithmetic, and measures FASTER there (AlexNet conv1, 30 KB staged: 0.113 vs 0.122 ms):
+        // with cheap addresses a workgroup fires its 32 loads per lane in one burst, and the bursts
+        // of the resident workgroups crowd the stores of the others, which are what the kernel is
+        // bound by.  Small staging areas are latency-bound and prefer the additions (0.016 vs 0.022 ms
+        // on a 3 x 32 x 32 input).
+        const int rowlen = KH * Wp;
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-        const int e = threadIdx.x + i * kIm2colThreads;
-        const int c = e / rowlen, rem = e - c * rowlen;
-        const int ho = rem / Wp, x = rem - ho * Wp;
-        const int hp = hbase + ho, wp = x - g.pw();
-        ok[i] = e < buflen && hp >= 0 && hp < H && wp >= 0 && wp < W;
-        reg[i] = base[ok[i] ? (int)(c * plane + hp * W + wp) : 0];
+        for (int i = 0; i < NI; ++i) {
+            const int e = threadIdx.x + i * kIm2colThreads;
+            const int c = e / rowlen, rem = e - c * rowlen;
+            const int ho = rem / Wp, x = rem - ho * Wp;
+            const int hp = hbase + ho, wp = x0 + x;
+            ok[i] = e < buflen && hp >= 0 && hp < H && wp >= 0 && wp < W;
+            reg[i] = base[ok[i] ? (int)(c * plane + hp * W + wp) : 0];
+        }
+    } else
+    {
+        // four independent chains (elements i = k, k+4, k+8, ... for k = 0..3), so that the address
+        // arithmetic of one load does not wait for the previous one's
+        constexpr int NCH = 4;
+        static_assert(NI % NCH == 0, "staged elements per thread must split evenly over the chains");
+        const int up_x = W - Wp, up_ho = (int)plane - KH * W;
+        int x[NCH], c[NCH], ho[NCH], at[NCH];
+        auto advance = [&](int k, int dx, int dho, int dc, int dat) __attribute__((always_inline)) {
+            x[k] += dx;
+            ho[k] += dho;
+            c[k] += dc;
+            at[k] += dat;
+            if (x[k] >= Wp) {
+                x[k] -= Wp;
+                ++ho[k];
+                at[k] += up_x;
+            }
+            if (ho[k] >= KH) {
+                ho[k] -= KH;
+                ++c[k];
+                at[k] += up_ho;
+            }
+        };
+        {
+            const int row0 = (int)threadIdx.x / Wp;
+            x[0] = (int)threadIdx.x - row0 * Wp;
+            c[0] = row0 / KH;
+            ho[0] = row0 - c[0] * KH;
+            at[0] = c[0] * (int)plane + (hbase + ho[0]) * W + x0 + x[0];     // C*H*W < 2^31
+            const int drow = kIm2colThreads / Wp, dx = kIm2colThreads - drow * Wp;
+            const int dc = drow / KH, dho = drow - dc * KH;
+            const int dat = dc * (int)plane + dho * W + dx;
+#pragma unroll
+            for (int k = 1; k < NCH; ++k) {
+                x[k] = x[k - 1];
+                c[k] = c[k - 1];
+                ho[k] = ho[k - 1];
+                at[k] = at[k - 1];
+                advance(k, dx, dho, dc, dat);
+            }
+        }
+        const int drow = NCH * kIm2colThreads / Wp, dx = NCH * kIm2colThreads - drow * Wp;
+        const int dc = drow / KH, dho = drow - dc * KH;
+        const int dat = dc * (int)plane + dho * W + dx;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int k = i % NCH;
+            const int hp = hbase + ho[k], wp = x0 + x[k];
+            ok[i] = c[k] < C && hp >= 0 && hp < H && wp >= 0 && wp < W;
+            reg[i] = base[ok[i] ? at[k] : 0];
+            advance(k, dx, dho, dc, dat);
+        }
     }
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
@@ -269,8 +341,8 @@ __global__ __launch_bounds__(kIm2colThreads) void im2col_linear_kernel(
     __syncthreads();
 
     const int Z = C * KH * KW;
-    const int len = n * Z;                                   // floats in the region
-    const long start = (b * m + h) * (long)len;              // col is 16-byte aligned
+    const int len = nw * Z;                                  // floats in the region
+    const long start = ((b * m + h) * (long)n + w0) * Z;     // col is 16-byte aligned
     float* out = col + start;
     const int head = (int)((4 - (start & 3)) & 3);
     const int nunits = len > head ? (len - head) >> 2 : 0;
@@ -288,7 +360,6 @@ __global__ __launch_bounds__(kIm2colThreads) void im2col_linear_kernel(
     // the row (past the last one, R - 1) into the pixel.  Only the LDS offset is
     // kept up to date; the three floats after the first differ from it by j,
     // plus the same two carries.
-    const int R = C * KH;
     const int up_row = Wp - KW;                  // offset change when the kernel column wraps
     const int up_pix = SW - R * Wp;              // ... when the row wraps into the next pixel
     int f = head + 4 * (int)threadIdx.x;
@@ -798,13 +869,30 @@ static int launch_im2col(G g, const float* im, long B, int C, int H, int W, int 
         const bool small = (long)chunk * rowlen <= 12 * kIm2colThreads;
         dim3 grid((unsigned)blocks), block(kIm2colThreads);
         if constexpr (linear_writer_ok<G>()) {
-            // odd row length, all channels in one buffer: aligned 16-byte units over the linear region
-            if (!vec && nchunks == 1 && Z % 4 != 0 && reinterpret_cast<uintptr_t>(col) % 16 == 0 &&
-                (long)n * Z < (1L << 30) && (long)chunk * rowlen <= 32 * kIm2colThreads) {
-                if ((long)chunk * rowlen <= 12 * kIm2colThreads)
-                    im2col_linear_kernel<G, 12><<<grid, block, lds, st>>>(g, im, col, C, H, W, m, n);
+            // all channels staged at once, written as one linear region per tile of pixels: the
+            // whole row if it fits 32 KiB, else even tiles of at least 12 pixels within 24 KiB
+            // (VGG mid layer, 128 channels: 4 tiles of 14 pixels, 0.157 vs 0.174 ms for the chunked
+            // kernel; tiles of 8 are slower than it, their halo columns are a quarter of the loads)
+            const long R = (long)C * g.kh();
+            auto pixels_that_fit = [&](long budget) {
+                const long fit = budget / R;                                     // staged columns
+                return fit >= g.kw() ? std::min((long)n, (fit - g.kw()) / g.sw() + 1) : 0L;
+            };
+            long tw = pixels_that_fit(32L * kIm2colThreads);
+            if (tw < n) tw = pixels_that_fit(24L * kIm2colThreads);
+            if ((tw == n || tw >= 12) && reinterpret_cast<uintptr_t>(col) % 16 == 0 && tw * Z < (1L << 30)) {
+                const long ntiles = cdiv(n, tw);
+                tw = cdiv(n, ntiles);                                        // even tiles
+                const long staged = R * ((tw - 1) * g.sw() + g.kw());
+                const size_t lds_lin = (size_t)staged * sizeof(float);
+                dim3 lgrid((unsigned)(blocks * ntiles));
+                CGT_ARG_CHECK(blocks * ntiles < (1L << 31), "im2col: too many workgroups");
+                if (staged <= 12 * kIm2colThreads)
+                    im2col_linear_kernel<G, 12><<<lgrid, block, lds_lin, st>>>(g, im, col, C, H, W, m, n, (int)tw, (int)ntiles);
+                else if (staged <= 24 * kIm2colThreads)
+                    im2col_linear_kernel<G, 24><<<lgrid, block, lds_lin, st>>>(g, im, col, C, H, W, m, n, (int)tw, (int)ntiles);
                 else
-                    im2col_linear_kernel<G, 32><<<grid, block, lds, st>>>(g, im, col, C, H, W, m, n);
+                    im2col_linear_kernel<G, 32><<<lgrid, block, lds_lin, st>>>(g, im, col, C, H, W, m, n, (int)tw, (int)ntiles);
                 CGT_LAUNCH_CHECK("im2col_linear_kernel");
                 return CGT_AMD_OK;
             }

@@ -780,11 +780,10 @@ static int launch_col2im_stream(G g, const float* col, long B, int C, int H, int
                            : mode == kStageRuns ? col2im_stream_kernel<G, CC, WSUB, M_RUNS, LW, false>
                                                 : col2im_stream_kernel<G, CC, WSUB, kStageScalar, LW, false>);
     // Bands of image rows: as many workgroups as the chip holds at once, and
-    // no more.  The kernel is bound by the loads each wavefront can keep in
-    // flight, so resident wavefronts are what counts; a second, partial round
-    // of workgroups costs more than it gains (measured on the AlexNet layer:
-    // 2 bands 0.17 ms, 3 bands 0.21 ms), and each band re-reads kh - sh halo
-    // rows, so bands stay at least 2 kernel heights tall.
+    // no more.  A second, partial round of workgroups costs more than it gains
+    // (measured on the AlexNet layer: 1 or 2 bands 0.145 ms, 3 or 4 bands
+    // 0.153 ms), and each band re-reads kh - sh halo rows, so bands stay at
+    // least 2 kernel heights tall.
     int wg_per_cu = 0;
     CGT_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&wg_per_cu, kernel, 256, lds));
     const long resident = (long)std::max(wg_per_cu, 1) * kNumCU;

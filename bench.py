@@ -82,7 +82,7 @@ def make_inputs(cfg, batch=None, seed=0):
 class Stage(object):
     def __init__(self, name, kernel, fn, work, bound):
         self.name, self.kernel, self.fn, self.work, self.bound = name, kernel, fn, work, bound
-        self.ms = None
+        self.ms = self.ms_median = self.ms_min = self.ms_in_step = None
 
 
 class LayerOnGpu(object):
@@ -218,6 +218,26 @@ class LayerOnGpu(object):
                 self.stages[-1].fn()
                 self._wgrad_stream = main
                 self._join.record(side)
+
+    def time_stages_in_step(self, steps):
+        """Each stage's duration inside real steps: an event between every two stages of `steps`
+        consecutive steps (one stream).  A stage launched back to back with itself, as in
+        time_stages, finds its operands and its output buffer in the last-level cache when they
+        fit, and its stores can drain while the next copy runs; inside a step neither holds."""
+        from cgt_amd import capi
+        if self.overlap:
+            return
+        n = len(self.stages)
+        ev = [[capi.Event() for _ in range(n + 1)] for _ in range(steps)]
+        self.step()
+        for k in range(steps):
+            ev[k][0].record(self.stream)
+            for i, st in enumerate(self.stages):
+                st.fn()
+                ev[k][i + 1].record(self.stream)
+        capi.synchronize()
+        for i, st in enumerate(self.stages):
+            st.ms_in_step = sum(ev[k][i].elapsed_ms(ev[k][i + 1]) for k in range(steps)) / steps
 
     def time_stages(self, reps):
         from cgt_amd import capi
@@ -429,21 +449,41 @@ def main():
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
 
-    layer.time_stages(args.stage_reps)
+    # Two clocks per stage.  "ms_in_step": events between the stages of real steps (what a
+    # launch costs where it runs: after another kernel, operands wherever that left them) --
+    # the roofline figure uses this one.  "ms": the same launch repeated back to back, the
+    # kernel's own steady state (HBM kernels look better there than inside a step: repeated on
+    # the same buffers they find part of them in the 256 MB last-level cache; GEMMs look worse:
+    # the chip holds a lower clock under sustained matrix load).  --stage-reps 0 skips the second.
+    in_step_steps = max(5, min(args.steps, 20))
+    if args.stage_reps > 0 or is_gemm or args.glue:
+        layer.time_stages(max(args.stage_reps, 1))
+    if not is_gemm:
+        layer.time_stages_in_step(in_step_steps)
+
+    def clock(st):          # the stage's duration for the roofline: inside the step where measured
+        t = getattr(st, "ms_in_step", None)
+        return t if t is not None else st.ms
+
     stages = []
     gemm_flops = gemm_ms = 0.0
-    dominant = max((st for st in layer.stages if st.bound == "mfma"), key=lambda st: st.ms)
+    dominant = max((st for st in layer.stages if st.bound == "mfma"), key=clock)
     for st in layer.stages:
-        row = {"stage": st.name, "kernel": st.kernel, "ms": round(st.ms, 4), "ms_median": round(st.ms_median, 4),
-               "ms_min": round(st.ms_min, 4), "bound": st.bound}
-        if st.bound == "hbm":
-            gbs = st.work / (st.ms * 1e-3) / 1e9
-            row.update(bytes=st.work, GBps=round(gbs, 1), frac=round(gbs / HBM_PEAK_GBS, 4))
-        else:
-            tf = st.work / (st.ms * 1e-3) / 1e12
-            row.update(flops=st.work, TFLOPs=round(tf, 2), frac=round(tf / FP32_MFMA_PEAK_TFLOPS, 4))
+        row = {"stage": st.name, "kernel": st.kernel, "bound": st.bound}
+        peak = HBM_PEAK_GBS if st.bound == "hbm" else FP32_MFMA_PEAK_TFLOPS
+        unit, scale = ("GBps", 1e9) if st.bound == "hbm" else ("TFLOPs", 1e12)
+        row["bytes" if st.bound == "hbm" else "flops"] = st.work
+        if st.ms is not None:
+            rate = st.work / (st.ms * 1e-3) / scale
+            row.update({"ms": round(st.ms, 4), "ms_median": round(st.ms_median, 4), "ms_min": round(st.ms_min, 4),
+                        unit: round(rate, 2), "frac": round(rate / peak, 4)})
+        if getattr(st, "ms_in_step", None) is not None:
+            rate = st.work / (st.ms_in_step * 1e-3) / scale
+            row.update({"ms_in_step": round(st.ms_in_step, 4), unit + "_in_step": round(rate, 2),
+                        "frac_in_step": round(rate / peak, 4)})
+        if st.bound == "mfma":
             gemm_flops += st.work
-            gemm_ms += st.ms
+            gemm_ms += clock(st)
         stages.append(row)
     glue_stages = []
     for st in getattr(layer, "extra_stages", []):
@@ -467,10 +507,14 @@ def main():
         "frac_fp32_mfma_peak": round(value / FP32_MFMA_PEAK_TFLOPS, 4),
         # the dominant kernel: the slowest MFMA GEMM launch of a step
         "roofline": {"bound": "mfma", "kernel": dominant.kernel, "stage": dominant.name,
-                     "achieved": round(dominant.work / (dominant.ms * 1e-3) / 1e12, 2),
+                     "achieved": round(dominant.work / (clock(dominant) * 1e-3) / 1e12, 2),
                      "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(dominant.work / (dominant.ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4),
-                     "flops_per_launch": dominant.work, "avg_launch_ms": round(dominant.ms, 4),
+                     "frac": round(dominant.work / (clock(dominant) * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4),
+                     "flops_per_launch": dominant.work, "avg_launch_ms": round(clock(dominant), 4),
+                     "timing": ("HIP events around the launch inside %d consecutive steps" % in_step_steps
+                                if getattr(dominant, "ms_in_step", None) is not None else
+                                "HIP events around %d back-to-back launches" % max(args.stage_reps, 1)),
+                     "avg_launch_ms_back_to_back": None if dominant.ms is None else round(dominant.ms, 4),
                      "traffic": TRAFFIC.get((args.workload, dominant.name))},
         "gemm_all_launches": {"TFLOPs": round(gemm_tf, 2), "frac": round(gemm_tf / FP32_MFMA_PEAK_TFLOPS, 4)},
         "stages": stages,

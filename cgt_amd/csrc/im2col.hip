@@ -868,20 +868,20 @@ static int launch_im2col(G g, const float* im, long B, int C, int H, int W, int 
         const bool small = (long)chunk * rowlen <= 12 * kIm2colThreads;
         dim3 grid((unsigned)blocks), block(kIm2colThreads);
         if constexpr (linear_writer_ok<G>()) {
-            // all channels staged at once, written as one linear region per tile of pixels: the
-            // whole row if it fits 32 KiB, else even tiles of at least 12 pixels within 24 KiB
-            // (VGG mid layer, 128 channels: 4 tiles of 14 pixels, 0.157 vs 0.174 ms for the chunked
-            // kernel; tiles of 8 are slower than it, their halo columns are a quarter of the loads)
+            // all channels staged at once, written as one linear region: the whole row if it fits 32 KiB
             const long R = (long)C * g.kh();
             auto pixels_that_fit = [&](long budget) {
                 const long fit = budget / R;                                     // staged columns
                 return fit >= g.kw() ? std::min((long)n, (fit - g.kw()) / g.sw() + 1) : 0L;
             };
             long tw = pixels_that_fit(32L * kIm2colThreads);
-            if (tw < n) tw = pixels_that_fit(24L * kIm2colThreads);
-            if ((tw == n || tw >= 12) && reinterpret_cast<uintptr_t>(col) % 16 == 0 && tw * Z < (1L << 30)) {
-                const long ntiles = cdiv(n, tw);
-                tw = cdiv(n, ntiles);                                        // even tiles
+            // Tiles of a row (all channels staged, tw < n) are supported by the kernel and measure
+            // faster launched back to back (VGG mid layer, 4 tiles of 14 pixels: 0.157 vs 0.174 ms for
+            // the chunked kernel) but slower where they run, right after the previous step's
+            // weight-gradient GEMM (0.262 vs 0.211 ms; whole step 1.986 vs 1.937 ms), so only
+            // whole rows take this path.
+            if (tw == n && reinterpret_cast<uintptr_t>(col) % 16 == 0 && tw * Z < (1L << 30)) {
+                const long ntiles = 1;
                 const long staged = R * ((tw - 1) * g.sw() + g.kw());
                 const size_t lds_lin = (size_t)staged * sizeof(float);
                 dim3 lgrid((unsigned)(blocks * ntiles));

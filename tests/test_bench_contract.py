@@ -40,6 +40,11 @@ def test_default_workload_prints_the_contract_line():
     assert roof["bound"] in ("hbm", "mfma") and roof["unit"] in ("GB/s", "TFLOP/s")
     assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
     assert roof["peak"] == 157.3 and roof["traffic"] > 0
+    # the roofline figure is clocked inside real steps; every stage carries that clock and,
+    # with --stage-reps > 0, the back-to-back one as well
+    assert "inside" in roof["timing"] and roof["avg_launch_ms"] > 0
+    for row in out["stages"]:
+        assert row["ms_in_step"] > 0 and row["ms"] > 0 and 0 < row["frac_in_step"] < 1.2
     cpu = out["cpu_baseline"]
     assert cpu["kind"] in ("port", "reference") and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
     assert out["parity"]["ok"] is True

@@ -456,7 +456,7 @@ def main():
     # the same buffers they find part of them in the 256 MB last-level cache; GEMMs look worse:
     # the chip holds a lower clock under sustained matrix load).  --stage-reps 0 skips the second.
     in_step_steps = max(5, min(args.steps, 20))
-    if args.stage_reps > 0 or is_gemm or args.glue:
+    if args.stage_reps > 0 or is_gemm or args.glue or getattr(layer, "overlap", False):
         layer.time_stages(max(args.stage_reps, 1))
     if not is_gemm:
         layer.time_stages_in_step(in_step_steps)

@@ -224,33 +224,31 @@ __global__ __launch_bounds__(kIm2colThreads) void im2col_pipe_kernel(
     }
 }
 
-// Linear writer.  With ALL channels staged at once, the output for a run of tw
-// pixels of row (b, h) -- tw*Z floats -- is ONE contiguous region of the column
-// buffer, and a workgroup writes it front to back as aligned 16-byte units
-// wherever its first float falls (Z % 4 != 0, e.g. 3 x 11 x 11 = 363, moves the
-// start from row to row): unit q holds floats f = head + 4q .. +3 of the region,
-// float f is pixel f / Z, element z = f % Z, and since z = (c*kh + ho)*kw + wo
-// the staged value sits at LDS row z / kw, column pixel*sw + z % kw.  Both the
-// staging and the writing advance by fixed steps with carries, so there is no
-// division inside a loop.  The up to three floats before the first and after the
-// last whole unit are written singly.  tw is the whole row when the staged rows
-// of all channels fit (AlexNet conv1), else the widest tile that fits (VGG:
-// 128 channels x 3 rows x 16 columns, regions of 14 pixels = 63 KB).
+// Linear writer.  With ALL channels staged at once, the output of row (b, h) --
+// n*Z floats -- is ONE contiguous region of the column buffer, and a workgroup
+// writes it front to back as aligned 16-byte units wherever its first float
+// falls (Z % 4 != 0, e.g. 3 x 11 x 11 = 363, moves the start from row to row):
+// unit q holds floats f = head + 4q .. +3 of the region, float f is pixel f / Z,
+// element z = f % Z, and since z = (c*kh + ho)*kw + wo the staged value sits at
+// LDS row z / kw, column pixel*sw + z % kw.  Both the staging and the writing
+// advance by fixed steps with carries, so there is no division inside a loop.
+// The up to three floats before the first and after the last whole unit are
+// written singly.  (Splitting a row that does not fit into tiles of pixels, each
+// a region of its own, was tried on the VGG mid layer -- 4 tiles of 14 pixels,
+// 128 channels x 3 rows x 16 columns staged: 0.157 vs 0.174 ms for the chunked
+// kernel launched back to back, but 0.262 vs 0.211 ms where it runs, after the
+// previous step's weight-gradient GEMM -- and is not kept.)
 template <class G, int NI>
 __global__ __launch_bounds__(kIm2colThreads) void im2col_linear_kernel(
-    G g, const float* __restrict__ im, float* __restrict__ col, int C, int H, int W, int m, int n,
-    int tw, int ntiles) {
-    extern __shared__ float tile[];  // [C*kh][twi]
+    G g, const float* __restrict__ im, float* __restrict__ col, int C, int H, int W, int m, int n) {
+    extern __shared__ float tile[];  // [C*kh][Wp]
     constexpr int KH = G::kKH, KW = G::kKW, SW = G::kSW;
     static_assert(KW >= 3, "a unit of four floats may carry only once out of the kernel column");
-    unsigned bid = (unsigned)xcd_remap(blockIdx.x, gridDim.x);       // 32-bit: 64-bit divisions cost hundreds of instructions
-    const int wt = (int)(bid % (unsigned)ntiles);                    // tiles of a row are neighbours: their regions are adjacent
-    bid /= (unsigned)ntiles;
+    const unsigned bid = (unsigned)xcd_remap(blockIdx.x, gridDim.x);   // 32-bit: 64-bit divisions cost hundreds of instructions
     const int h = (int)(bid % (unsigned)m);
     const long b = bid / (unsigned)m;
-    const int w0 = wt * tw, nw = min(tw, n - w0);
-    const int Wp = (tw - 1) * SW + KW;           // staged columns: image columns x0 .. x0 + Wp - 1
-    const int x0 = w0 * SW - g.pw();
+    const int Wp = (n - 1) * SW + KW;            // staged columns: image columns x0 .. x0 + Wp - 1
+    const int x0 = -g.pw();
     const int R = C * KH;
     const int buflen = R * Wp;                   // <= NI * 256
     const int hbase = h * g.sh() - g.ph();
@@ -341,8 +339,8 @@ __global__ __launch_bounds__(kIm2colThreads) void im2col_linear_kernel(
     __syncthreads();
 
     const int Z = C * KH * KW;
-    const int len = nw * Z;                                  // floats in the region
-    const long start = ((b * m + h) * (long)n + w0) * Z;     // col is 16-byte aligned
+    const int len = n * Z;                                   // floats in the region
+    const long start = (b * m + h) * (long)len;              // col is 16-byte aligned
     float* out = col + start;
     const int head = (int)((4 - (start & 3)) & 3);
     const int nunits = len > head ? (len - head) >> 2 : 0;
@@ -868,30 +866,16 @@ static int launch_im2col(G g, const float* im, long B, int C, int H, int W, int 
         const bool small = (long)chunk * rowlen <= 12 * kIm2colThreads;
         dim3 grid((unsigned)blocks), block(kIm2colThreads);
         if constexpr (linear_writer_ok<G>()) {
-            // all channels staged at once, written as one linear region: the whole row if it fits 32 KiB
-            const long R = (long)C * g.kh();
-            auto pixels_that_fit = [&](long budget) {
-                const long fit = budget / R;                                     // staged columns
-                return fit >= g.kw() ? std::min((long)n, (fit - g.kw()) / g.sw() + 1) : 0L;
-            };
-            long tw = pixels_that_fit(32L * kIm2colThreads);
-            // Tiles of a row (all channels staged, tw < n) are supported by the kernel and measure
-            // faster launched back to back (VGG mid layer, 4 tiles of 14 pixels: 0.157 vs 0.174 ms for
-            // the chunked kernel) but slower where they run, right after the previous step's
-            // weight-gradient GEMM (0.262 vs 0.211 ms; whole step 1.986 vs 1.937 ms), so only
-            // whole rows take this path.
-            if (tw == n && reinterpret_cast<uintptr_t>(col) % 16 == 0 && tw * Z < (1L << 30)) {
-                const long ntiles = 1;
-                const long staged = R * ((tw - 1) * g.sw() + g.kw());
+            // all channels' rows staged at once (32 KiB), the output row written as one linear region
+            const long staged = (long)C * g.kh() * ((long)(n - 1) * g.sw() + g.kw());
+            if (staged <= 32L * kIm2colThreads && reinterpret_cast<uintptr_t>(col) % 16 == 0 && n * Z < (1L << 30)) {
                 const size_t lds_lin = (size_t)staged * sizeof(float);
-                dim3 lgrid((unsigned)(blocks * ntiles));
-                CGT_ARG_CHECK(blocks * ntiles < (1L << 31), "im2col: too many workgroups");
                 if (staged <= 12 * kIm2colThreads)
-                    im2col_linear_kernel<G, 12><<<lgrid, block, lds_lin, st>>>(g, im, col, C, H, W, m, n, (int)tw, (int)ntiles);
+                    im2col_linear_kernel<G, 12><<<grid, block, lds_lin, st>>>(g, im, col, C, H, W, m, n);
                 else if (staged <= 24 * kIm2colThreads)
-                    im2col_linear_kernel<G, 24><<<lgrid, block, lds_lin, st>>>(g, im, col, C, H, W, m, n, (int)tw, (int)ntiles);
+                    im2col_linear_kernel<G, 24><<<grid, block, lds_lin, st>>>(g, im, col, C, H, W, m, n);
                 else
-                    im2col_linear_kernel<G, 32><<<lgrid, block, lds_lin, st>>>(g, im, col, C, H, W, m, n, (int)tw, (int)ntiles);
+                    im2col_linear_kernel<G, 32><<<grid, block, lds_lin, st>>>(g, im, col, C, H, W, m, n);
                 CGT_LAUNCH_CHECK("im2col_linear_kernel");
                 return CGT_AMD_OK;
             }

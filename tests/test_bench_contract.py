@@ -48,3 +48,15 @@ def test_default_workload_prints_the_contract_line():
     cpu = out["cpu_baseline"]
     assert cpu["kind"] in ("port", "reference") and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
     assert out["parity"]["ok"] is True
+
+
+@pytest.mark.gpu
+def test_in_step_clock_alone():
+    # --stage-reps 0: only the in-step clock; the roofline figure still comes out
+    proc = _run(["--steps", "2", "--warmup", "1", "--stage-reps", "0", "--no-cpu", "--no-op-api",
+                 "--workload", "cifar_conv2_5x5_32x15x15_b128"], 600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    out = json.loads([ln for ln in proc.stdout.splitlines() if ln.strip()][0])
+    assert out["roofline"]["achieved"] > 0 and "inside" in out["roofline"]["timing"]
+    for row in out["stages"]:
+        assert row["ms_in_step"] > 0 and "ms" not in row

@@ -27,7 +27,10 @@ __host__ __device__ inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 // 5.9 TB/s with it and the 96 x 3025 transpose from 5.2 to 7.1 TB/s, while 4-byte stores
 // and runs that start anywhere (rows of 363 floats, planes of 3025) get SLOWER without
 // L2's write combining (AlexNet im2col -27 %, pool pullback -59 %), so only aligned
-// vector stores use it.
+// vector stores use it.  Those figures are for a kernel launched back to back with itself;
+// inside a conv layer's step, between other kernels, the gain is smaller on large outputs
+// (VGG im2col: none) and larger where the next kernel is bound by memory too (AlexNet
+// conv1 layer: 0.08 ms of 1.67 per step, mostly the LRN forward's two outputs).
 typedef float v4f __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void stream_store4(float* p, float a, float b, float c, float d) {
     v4f v = {a, b, c, d};

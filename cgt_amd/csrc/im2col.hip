@@ -237,7 +237,10 @@ __global__ __launch_bounds__(kIm2colThreads) void im2col_pipe_kernel(
 // a region of its own, was tried on the VGG mid layer -- 4 tiles of 14 pixels,
 // 128 channels x 3 rows x 16 columns staged: 0.157 vs 0.174 ms for the chunked
 // kernel launched back to back, but 0.262 vs 0.211 ms where it runs, after the
-// previous step's weight-gradient GEMM -- and is not kept.)
+// previous step's weight-gradient GEMM -- and is not kept; nor is a version of it that walks the
+// tiles of a row inside one workgroup with two staging buffers (0.184 ms back to back, 0.276 in
+// step): a tile reads the image in 64-byte pieces, which is cheap from the last-level cache, where a
+// kernel repeated on the same input finds it, and dear from HBM.)
 template <class G, int NI>
 __global__ __launch_bounds__(kIm2colThreads) void im2col_linear_kernel(
     G g, const float* __restrict__ im, float* __restrict__ col, int C, int H, int W, int m, int n) {

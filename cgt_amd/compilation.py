@@ -3,8 +3,8 @@
 Follows the reference's cgt/compilation.py:521-749: the op's code is wrapped
 with `#include "cgt_common.h"`, its includes and a `typedef struct $closure`
 generated from the closure triples; $function / $closure / $setup / $teardown
-are renamed with an md5 over (templated code, compiler flags, ABI version,
-extra sources); each source file is compiled (`c++` for "c++", `hipcc
+are renamed with an md5 over (templated code, compiler flags, ABI version, the
+text of the headers every closure includes, extra sources); each source file is compiled (`c++` for "c++", `hipcc
 --offload-arch=gfx950` for "hip" -- the reference's "cuda"/nvcc slot), linked
 into <cache>/<md5>.so, loaded with ctypes, and the closure struct is built as
 a ctypes.Structure.  A library that is already in the cache is not rebuilt.
@@ -21,6 +21,10 @@ from . import core, rt
 
 # bump when the object model in csrc/include/cgt_common.h changes layout
 CPP_ABI_VERSION = 1
+# headers every closure is compiled against: cgtArray's accessors are inline, so
+# their text is part of each cached library and therefore of its cache key
+_ABI_HEADERS = ("cgt_common.h", "cgt_amd.h")
+_abi_headers_hash = None
 
 _COMPILE_CONFIG = None
 _LIBRARIES = {}
@@ -53,6 +57,24 @@ def get_compile_info():
                                LINK_FLAGS=link_flags, CXX=_build.CXX, HIPCC=_build.HIPCC,
                                HIP_LINK_FLAGS="-L/opt/rocm/lib -lamdhip64")
     return _COMPILE_CONFIG
+
+
+def abi_headers_hash():
+    """md5 over the text of the headers the closures include."""
+    global _abi_headers_hash
+    if _abi_headers_hash is None:
+        h = hashlib.md5()
+        for name in _ABI_HEADERS:
+            for d in (_build.RT_INCLUDE, _build.INCLUDE):
+                path = os.path.join(d, name)
+                if os.path.exists(path):
+                    with open(path, "rb") as fh:
+                        h.update(fh.read())
+                    break
+            else:
+                raise RuntimeError("header %s not found" % name)
+        _abi_headers_hash = h.hexdigest()
+    return _abi_headers_hash
 
 
 def hash_seq(*strings):
@@ -155,7 +177,8 @@ class TranslationUnit(object):
 def nci2callable(nci):
     template_code = gen_templated_code(nci.includes, nci.closure_triples, nci.func_code)
     d = get_compile_info()
-    prefix = hash_seq(template_code, d["CPP_FLAGS"], str(CPP_ABI_VERSION), *(src.code for src in nci.extra_srcs))
+    prefix = hash_seq(template_code, d["CPP_FLAGS"], str(CPP_ABI_VERSION), abi_headers_hash(),
+                      *(src.code for src in nci.extra_srcs))
     names = dict(function=_funcname(prefix), closure=_closurename(prefix), setup=_setupname(prefix),
                  teardown=_teardownname(prefix))
     srcfiles = [core.SrcFile("c++", string.Template(template_code).substitute(names))]

@@ -506,7 +506,7 @@ class Mul22(Op):
                 long Kb = B->shape()[cl->tB ? 1 : 0];
                 cgt_check(K == Kb && A->shape()[cl->tA ? 1 : 0] == M && B->shape()[cl->tB ? 0 : 1] == N,
                     "shape mismatch at matrix-matrix multiplication");
-                if (K != Kb) return;
+                if (cgtGlobalStatus != cgtStatusOK) return;     // no launch on operands that do not fit
                 int rc = cgt_amd_sgemm(cl->tA, cl->tB, M, N, K, (const float*)A->data(), lda,
                     (const float*)B->data(), ldb, (float*)C->data(), ldc, cgt_get_stream());
                 cgt_check(rc == CGT_AMD_OK, "Mul22: %s", cgt_amd_last_error());
@@ -559,7 +559,8 @@ class BatchedMul22(Op):
                 long M = C->shape()[1];
                 long N = C->shape()[2];
                 long K = A->shape()[1+(cl->tA ? 0 : 1)];
-                cgt_check(B->shape()[0] == P && C->shape()[0] == P && B->shape()[1+(cl->tB ? 1 : 0)] == K,
+                cgt_check(B->shape()[0] == P && C->shape()[0] == P && B->shape()[1+(cl->tB ? 1 : 0)] == K &&
+                          A->shape()[1+(cl->tA ? 1 : 0)] == M && B->shape()[1+(cl->tB ? 0 : 1)] == N,
                     "shape mismatch at batched matrix multiplication");
                 if (cgtGlobalStatus != cgtStatusOK) return;
                 int rc = cgt_amd_sgemm_batched(cl->tA, cl->tB, P, M, N, K,
@@ -850,7 +851,9 @@ class ElwiseBinary(Op):
         code = r"""
             CGT_EXPORT_C void $function($closure* cl, cgtArray** reads, cgtArray* write) {
                 long n = reads[cl->scalar0 ? 1 : 0]->size();
-                cgt_check(write->size() == n, "Shape error in elementwise binary operation. You might be missing a call to cgt.broadcast(...)");
+                cgt_check(write->size() == n && (cl->scalar0 || cl->scalar1 || reads[1]->size() == n),
+                    "Shape error in elementwise binary operation. You might be missing a call to cgt.broadcast(...)");
+                if (cgtGlobalStatus != cgtStatusOK) return;     // no launch on operands that do not fit
                 int rc = cgt_amd_elwise_binary(cl->op, (int)reads[0]->dtype(), (int)reads[1]->dtype(), n,
                     reads[0]->data(), cl->scalar0, reads[1]->data(), cl->scalar1, write->data(), cgt_get_stream());
                 cgt_check(rc == CGT_AMD_OK, "ElwiseBinary: %s", cgt_amd_last_error());
@@ -924,8 +927,10 @@ class Repeat(Op):
                 for (int a = 0; a < nd; ++a) {
                     oshape[a] = write->shape()[a];
                     rep[a] = (cl->axes_mask >> a) & 1;
-                    cgt_check(!rep[a] || read->shape()[a] == 1, "Repeat: a repeated axis must have extent 1");
+                    cgt_check(rep[a] ? read->shape()[a] == 1 : read->shape()[a] == oshape[a],
+                        "Repeat: a repeated axis must have extent 1 and the others the output's extent");
                 }
+                if (cgtGlobalStatus != cgtStatusOK) return;
                 int rc = cgt_amd_repeat(read->data(), cgt_itemsize(read->dtype()), nd, oshape, rep,
                     write->data(), cgt_get_stream());
                 cgt_check(rc == CGT_AMD_OK, "Repeat: %s", cgt_amd_last_error());

@@ -15,6 +15,16 @@ void clear_error();
 
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 
+// Library-owned device workspaces (split-K partials, partial sums): one block per
+// (stream, user), grown on demand.  A block that is outgrown is NOT freed -- a HIP
+// graph recorded earlier may have its address baked in, and hipFree would stall the
+// stream -- it is retired and released with the stream (cgt_amd_stream_destroy).
+// Growth while the stream is being captured is refused (an allocation would break the
+// capture): returns nullptr with the message set.
+enum WorkspaceUser { kWsGemm = 0, kWsSum = 1, kWsUsers = 2 };
+float* stream_workspace(void* stream, WorkspaceUser user, size_t bytes, const char* what);
+void release_stream_workspaces(void* stream);
+
 constexpr int kWave = 64;    // CDNA wavefront width
 constexpr int kNumXCD = 8;   // MI355X: 8 accelerator dies, each with its own L2
 constexpr int kNumCU = 256;  // MI355X compute units

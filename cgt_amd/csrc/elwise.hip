@@ -12,9 +12,7 @@
 #include <algorithm>
 #include <cstdint>
 #include <cstring>
-#include <mutex>
 #include <type_traits>
-#include <unordered_map>
 
 namespace cgt_amd {
 
@@ -372,30 +370,9 @@ __global__ __launch_bounds__(256) void sum_generic_kernel(const float* __restric
     out[o] = acc;
 }
 
-// Workspace for partial sums, one per stream, grown on demand and kept.
-struct SumWorkspace {
-    float* ptr = nullptr;
-    size_t bytes = 0;
-};
-static std::mutex g_sum_mutex;
-static std::unordered_map<void*, SumWorkspace> g_sum_ws;
-
+// Workspace for partial sums: one per stream, owned by the library (see common.h).
 static float* sum_workspace(void* stream, size_t bytes) {
-    std::lock_guard<std::mutex> lock(g_sum_mutex);
-    SumWorkspace& w = g_sum_ws[stream];
-    if (w.bytes >= bytes) return w.ptr;
-    if (w.ptr) (void)hipFree(w.ptr);
-    w.ptr = nullptr;
-    w.bytes = 0;
-    void* p = nullptr;
-    const size_t want = std::max(bytes, (size_t)1 << 20);
-    if (hipMalloc(&p, want) != hipSuccess) {
-        (void)hipGetLastError();
-        return nullptr;
-    }
-    w.ptr = static_cast<float*>(p);
-    w.bytes = want;
-    return w.ptr;
+    return stream_workspace(stream, kWsSum, bytes, "sum");
 }
 
 // Merge neighbouring axes with the same flag; drops axes of extent 1.
@@ -555,10 +532,7 @@ CGT_API int cgt_amd_sum_f32(const float* x, int ndim, const long* shape, const i
             const long kblocks = cdiv(K, (long)kSumThreads);
             const int S0 = (int)std::max(1L, std::min(std::min(R0 / 4 + 1, 1024L), cdiv(target, kblocks)));
             float* ws = sum_workspace(stream, (size_t)S0 * K * sizeof(float));
-            if (!ws) {
-                set_error("sum: cannot allocate workspace");
-                return CGT_AMD_ERR_NOMEM;
-            }
+            if (!ws) return CGT_AMD_ERR_NOMEM;
             CGT_ARG_CHECK(kblocks * S0 < (1L << 31) && K < (1L << 31), "sum: too many workgroups");
             sum_cols_kernel<<<dim3((unsigned)(kblocks * S0)), dim3(kSumThreads), 0, st>>>(x, ws, R0, K, S0);
             CGT_LAUNCH_CHECK("sum_cols_kernel");
@@ -570,10 +544,7 @@ CGT_API int cgt_amd_sum_f32(const float* x, int ndim, const long* shape, const i
         const long S0 = std::max(1L, std::min(R0, cdiv(target, K * S1)));
         CGT_ARG_CHECK(K * S0 * S1 < (1L << 31) && S0 * S1 < (1L << 24), "sum: too many workgroups");
         float* ws = sum_workspace(stream, (size_t)(K * S0 * S1) * sizeof(float));
-        if (!ws) {
-            set_error("sum: cannot allocate workspace");
-            return CGT_AMD_ERR_NOMEM;
-        }
+        if (!ws) return CGT_AMD_ERR_NOMEM;
         const int vec = R1 % 4 == 0 && aligned_to(x, 16);
         sum_rkr_kernel<<<dim3((unsigned)(K * S0 * S1)), dim3(kSumThreads), 0, st>>>(x, ws, R0, K, R1, (int)S0, (int)S1, vec);
         CGT_LAUNCH_CHECK("sum_rkr_kernel");

@@ -49,9 +49,7 @@
 // about the same time.
 #include "common.h"
 #include <algorithm>
-#include <mutex>
 #include <type_traits>
-#include <unordered_map>
 
 namespace cgt_amd {
 
@@ -72,6 +70,10 @@ __device__ __forceinline__ int chunk_pos(int row, int chunk) { return chunk ^ ((
 // One 16-byte-per-lane load straight into LDS: lane l's data lands at lds_addr + 16*l.
 // Written as inline asm so that the compiler's wait-count insertion does not see it and
 // make every later LDS read wait for it; the loops wait with explicit s_waitcnt vmcnt.
+// m0 (the LDS base of the load) is written here and not listed as clobbered: the AMDGPU
+// backend reserves m0 -- it never keeps a value in it across other code, it sets it
+// immediately before each instruction of its own that reads it -- and rejects the listing
+// ("inline asm clobber list contains reserved registers: m0").
 __device__ __forceinline__ void load_to_lds16(const void* base, unsigned voff, unsigned lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(lds_addr), "v"(voff), "s"(base) : "memory");
@@ -676,29 +678,9 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     }
 }
 
-// Split-K workspaces, one per stream, grown on demand and kept.
-struct Workspace {
-    float* ptr = nullptr;
-    size_t bytes = 0;
-};
-static std::mutex g_ws_mutex;
-static std::unordered_map<void*, Workspace> g_ws;
-
+// Split-K / tail workspaces: one per stream, owned by the library (see common.h).
 static float* get_workspace(void* stream, size_t bytes) {
-    std::lock_guard<std::mutex> lock(g_ws_mutex);
-    Workspace& w = g_ws[stream];
-    if (w.bytes >= bytes) return w.ptr;
-    if (w.ptr) (void)hipFree(w.ptr);  // hipFree waits for work that may still read it
-    w.ptr = nullptr;
-    w.bytes = 0;
-    void* p = nullptr;
-    if (hipMalloc(&p, bytes) != hipSuccess) {
-        (void)hipGetLastError();
-        return nullptr;
-    }
-    w.ptr = static_cast<float*>(p);
-    w.bytes = bytes;
-    return w.ptr;
+    return stream_workspace(stream, kWsGemm, bytes, "sgemm");
 }
 
 static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
@@ -787,10 +769,7 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
         }
         if (a.splits > 1) {
             a.ws = get_workspace(stream, (size_t)a.splits * M * N * sizeof(float));
-            if (!a.ws) {
-                set_error("sgemm: cannot allocate split-K workspace");
-                return CGT_AMD_ERR_NOMEM;
-            }
+            if (!a.ws) return CGT_AMD_ERR_NOMEM;
         }
     }
     // tail split (single product, no split-K): tiles beyond the last full
@@ -817,10 +796,7 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
             a.tail_kchunk = (int)(cdiv(cdiv(K, best_s), KT) * KT);
             a.tail_splits = (int)cdiv(K, a.tail_kchunk);
             a.ws = get_workspace(stream, (size_t)tail_tiles * a.tail_splits * kShapes[shape].bm * kShapes[shape].bn * sizeof(float));
-            if (!a.ws) {
-                set_error("sgemm: cannot allocate tail workspace");
-                return CGT_AMD_ERR_NOMEM;
-            }
+            if (!a.ws) return CGT_AMD_ERR_NOMEM;
         }
     }
     const long wgs = a.splits > 1 ? tiles * a.splits : a.main_wgs + tail_tiles * a.tail_splits;

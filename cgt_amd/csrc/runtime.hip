@@ -2,6 +2,9 @@
 // events, error reporting.
 #include "common.h"
 #include <cstring>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
 
 namespace cgt_amd {
 
@@ -15,6 +18,48 @@ void set_error(const char* fmt, ...) {
 }
 
 void clear_error() { g_err[0] = 0; }
+
+struct StreamWorkspaces {
+    float* ptr[kWsUsers] = {nullptr, nullptr};
+    size_t bytes[kWsUsers] = {0, 0};
+    std::vector<void*> retired;
+};
+static std::mutex g_ws_mutex;
+static std::unordered_map<void*, StreamWorkspaces> g_ws;
+
+float* stream_workspace(void* stream, WorkspaceUser user, size_t bytes, const char* what) {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    StreamWorkspaces& w = g_ws[stream];
+    if (w.bytes[user] >= bytes) return w.ptr[user];
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(as_stream(stream), &cap) != hipSuccess) (void)hipGetLastError();
+    if (cap != hipStreamCaptureStatusNone) {
+        set_error("%s: the workspace would have to grow to %zu bytes while the stream is being captured; "
+                  "run the sequence once on this stream before capturing it", what, bytes);
+        return nullptr;
+    }
+    void* p = nullptr;
+    const size_t want = bytes < ((size_t)1 << 20) ? ((size_t)1 << 20) : bytes;
+    if (hipMalloc(&p, want) != hipSuccess) {
+        (void)hipGetLastError();
+        set_error("%s: cannot allocate a workspace of %zu bytes", what, want);
+        return nullptr;
+    }
+    if (w.ptr[user]) w.retired.push_back(w.ptr[user]);
+    w.ptr[user] = static_cast<float*>(p);
+    w.bytes[user] = want;
+    return w.ptr[user];
+}
+
+void release_stream_workspaces(void* stream) {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    auto it = g_ws.find(stream);
+    if (it == g_ws.end()) return;
+    for (int u = 0; u < kWsUsers; ++u)
+        if (it->second.ptr[u]) (void)hipFree(it->second.ptr[u]);
+    for (void* p : it->second.retired) (void)hipFree(p);
+    g_ws.erase(it);
+}
 
 __global__ void fill_u32_kernel(unsigned int* __restrict__ dst, unsigned int v, long n) {
     long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -119,7 +164,11 @@ CGT_API int cgt_amd_stream_create(void** stream) {
 }
 
 CGT_API int cgt_amd_stream_destroy(void* stream) {
-    if (stream) CGT_HIP_TRY(hipStreamDestroy(as_stream(stream)));
+    if (!stream) return CGT_AMD_OK;
+    // the stream's work may still use its workspaces: drain it before they go
+    CGT_HIP_TRY(hipStreamSynchronize(as_stream(stream)));
+    release_stream_workspaces(stream);
+    CGT_HIP_TRY(hipStreamDestroy(as_stream(stream)));
     return CGT_AMD_OK;
 }
 

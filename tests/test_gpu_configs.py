@@ -1,0 +1,136 @@
+"""The two small benchmark configurations, run exactly as they are stated --
+full batch, with the ReLU, RandomState(0), inputs drawn before weights --
+through the Op API on the GPU and compared stage by stage with the CPU oracle.
+
+  MNIST block   x = randn(64,1,28,28); W = 0.1*randn(32,1,3,3);
+                conv2d pad 1 -> x*(x>=0) -> max_pool 2x2 / stride 2 (13x13), forward.
+  CIFAR stack   x = rand(128,3,32,32); W1 = 0.01*randn(32,3,5,5);
+                W2 = 0.01*randn(64,32,5,5); conv p2 -> ReLU -> max_pool 3x3 / 2
+                (15x15) -> LRN(5, 1e-4, .75) -> conv p2; loss = sum of the
+                outputs; gradients wrt x, W1, W2.
+
+Graph shapes follow the reference's cgt/nn.py:44-45 (rectify), 87-111 (conv2d,
+max_pool_2d) and the gradient checks of cgt/tests/test_imgproc.py:40-97.
+
+Bars: the ReLU output, pooled values, int32 argmax and the pool pullback are
+bit-exact against the oracle applied to the same fp32 input; conv, LRN and the
+three gradients are within 1e-4 relative Frobenius error of the float64 oracle
+chain.  The argmax is a discrete choice, so the float64 chain takes the fp32
+mask (asserted bit-exact first); how often an independent float64 argmax would
+have chosen differently is bounded separately.
+"""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def cgt():
+    import cgt_amd
+    from cgt_amd import capi
+    capi.require_gpu()
+    return cgt_amd
+
+
+def relfro(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30)
+
+
+def _pool_values_from_mask(x, mask):
+    """x[n,c].flat[mask[n,c,ph,pw]]: pooled values of `x` under a given argmax."""
+    N, C, H, W = x.shape
+    flat = x.reshape(N, C, H * W)
+    return np.take_along_axis(flat, mask.reshape(N, C, -1).astype(np.int64), axis=2).reshape(mask.shape)
+
+
+def test_mnist_block_full_batch(cgt):
+    from cgt_amd import nn
+    rs = np.random.RandomState(0)
+    xval = rs.randn(64, 1, 28, 28).astype(np.float32)
+    wval = (0.1 * rs.randn(32, 1, 3, 3)).astype(np.float32)
+    x, W = cgt.constant(xval), cgt.constant(wval)
+    h = nn.conv2d(x, W, (3, 3), pad=(1, 1))
+    r = nn.rectify(h)
+    p = nn.max_pool_2d(r, (2, 2), (0, 0), (2, 2))
+    assert h.shape == (64, 32, 28, 28) and p.shape == (64, 32, 13, 13)
+    hv, rv = h.get(), r.get()
+    # conv against the float64 oracle
+    h64 = O.conv2d(xval.astype(np.float64), wval.astype(np.float64), (1, 1), (1, 1))
+    assert relfro(hv, h64) <= TOL
+    # im2col inside the conv is a copy: bit-exact
+    col = h.parents[0].parents[0].parents[0].parents[0]
+    assert col.shape == (64, 28, 28, 9)
+    assert np.array_equal(col.get(), O.im2col(xval, (3, 3), (1, 1), (1, 1)))
+    # ReLU as the reference spells it, on the same fp32 input: bit-exact (signs of zero included)
+    want_r = O.rectify(hv)
+    assert np.array_equal(rv.view(np.uint32), want_r.view(np.uint32))
+    assert (rv == 0).mean() > 0.2, "the ReLU must produce the ties the pool sees"
+    # pool values + int32 argmax on the ReLU output: bit-exact
+    top, mask = O.max_pool(rv, (2, 2), (0, 0), (2, 2))
+    gmask = p.parents[0].value[1].get()
+    assert gmask.dtype == np.int32 and np.array_equal(gmask, mask)
+    assert np.array_equal(p.get().view(np.uint32), top.view(np.uint32))
+    # whole block against the float64 chain (pooled values of a max are continuous in the input)
+    top64, _ = O.max_pool(O.rectify(h64), (2, 2), (0, 0), (2, 2))
+    assert relfro(p.get(), top64) <= TOL
+
+
+def test_cifar_stack_full_batch_forward_backward(cgt):
+    from cgt_amd import nn
+    d = np.float64
+    rs = np.random.RandomState(0)
+    xval = rs.rand(128, 3, 32, 32).astype(np.float32)
+    w1 = (0.01 * rs.randn(32, 3, 5, 5)).astype(np.float32)
+    w2 = (0.01 * rs.randn(64, 32, 5, 5)).astype(np.float32)
+    x, W1, W2 = cgt.constant(xval), cgt.constant(w1), cgt.constant(w2)
+    h1 = nn.conv2d(x, W1, (5, 5), pad=(2, 2))
+    r1 = nn.rectify(h1)
+    p1 = nn.max_pool_2d(r1, (3, 3), (0, 0), (2, 2))
+    n1 = nn.cross_channel_lrn(p1, 5, 1e-4, 0.75)
+    out = nn.conv2d(n1, W2, (5, 5), pad=(2, 2))
+    assert h1.shape == (128, 32, 32, 32) and p1.shape == (128, 32, 15, 15) and out.shape == (128, 64, 15, 15)
+    loss = cgt.sum(out)
+    gx, gW1, gW2 = cgt.grad(loss, [x, W1, W2])
+    assert gx.shape == xval.shape and gW1.shape == w1.shape and gW2.shape == w2.shape
+
+    # ---- forward, stage by stage
+    h1v, r1v, p1v = h1.get(), r1.get(), p1.get()
+    oh1 = O.conv2d(xval.astype(d), w1.astype(d), (2, 2), (1, 1))
+    assert relfro(h1v, oh1) <= TOL
+    assert np.array_equal(r1v.view(np.uint32), O.rectify(h1v).view(np.uint32))
+    assert (r1v == 0).mean() > 0.05, "the ReLU must produce the ties the pool sees"
+    top, mask = O.max_pool(r1v, (3, 3), (0, 0), (2, 2))
+    gmask = p1.parents[0].value[1].get()
+    assert np.array_equal(gmask, mask)
+    assert np.array_equal(p1v.view(np.uint32), top.view(np.uint32))
+    # LRN on the same fp32 input against the fp32 oracle (running-sum order differs: tolerance)
+    ltop, lscale = O.lrn_fwd(p1v, 5, 1e-4, 0.75)
+    gtop_scale = n1.parents[0].value
+    assert relfro(gtop_scale[0].get(), ltop) <= TOL and relfro(gtop_scale[1].get(), lscale) <= TOL
+
+    # ---- the float64 chain (argmax fixed to the fp32 one, see the module docstring)
+    or1 = O.rectify(oh1)
+    _, mask64 = O.max_pool(or1, (3, 3), (0, 0), (2, 2))
+    assert (mask64 != mask).mean() < 1e-4, "fp32 and float64 argmax should differ on near-ties only"
+    op1 = _pool_values_from_mask(or1, mask)
+    on1, oscale = O.lrn_fwd(op1, 5, 1e-4, 0.75)
+    oout = O.conv2d(on1, w2.astype(d), (2, 2), (1, 1))
+    assert relfro(n1.get(), on1) <= TOL
+    assert relfro(out.get(), oout) <= TOL
+    assert abs(float(loss.get()) - oout.sum()) <= TOL * np.abs(oout).sum()
+
+    # ---- backward: cotangent of sum(out) is ones
+    gn1, ogW2 = O.conv2d_pullback(on1, w2.astype(d), np.ones_like(oout), (2, 2), (1, 1))
+    gp1 = O.lrn_bwd(op1, on1, oscale, gn1, 5, 1e-4, 0.75)
+    gr1 = O.max_pool_pullback(or1.shape, mask, gp1)
+    gh1 = gr1 * (oh1 >= 0)                       # d/dx of x * (x >= 0)
+    ogx, ogW1 = O.conv2d_pullback(xval.astype(d), w1.astype(d), gh1, (2, 2), (1, 1))
+    assert relfro(gW2.get(), ogW2) <= TOL
+    assert relfro(gW1.get(), ogW1) <= TOL
+    assert relfro(gx.get(), ogx) <= TOL

@@ -128,6 +128,32 @@ def test_mul22_shape_mismatch_is_an_error(cgt):
         cgt.Result(cgt.Mul22(False, False), [A, B])
 
 
+def test_mul22_output_extent_mismatch_does_not_launch(cgt):
+    # the closure is handed a write array whose M (or N) does not fit A (or B): it must
+    # report the mismatch and launch nothing -- with extents taken from C the kernel
+    # would read A or B past their rows
+    from cgt_amd import core
+    from cgt_amd.capi import CgtAmdError
+    from cgt_amd.gpuarray import to_gpu
+    T2 = core.TensorType("f4", 2)
+    call = core.get_callable(core.Mul22(False, False), [T2, T2])
+    A, B = to_gpu(np.ones((3, 4), np.float32)), to_gpu(np.ones((4, 6), np.float32))
+    for cshape in [(7, 6), (3, 9)]:
+        sentinel = np.full(cshape, 123.0, np.float32)
+        C = to_gpu(sentinel)
+        with pytest.raises(CgtAmdError, match="shape mismatch"):
+            call.call([A, B], C)
+        assert np.array_equal(C.get(), sentinel)
+    bcall = core.get_callable(core.BatchedMul22(False, False), [core.TensorType("f4", 3)] * 2)
+    A3, B3 = to_gpu(np.ones((2, 3, 4), np.float32)), to_gpu(np.ones((2, 4, 6), np.float32))
+    for cshape in [(2, 7, 6), (2, 3, 9), (3, 3, 6)]:
+        sentinel = np.full(cshape, 123.0, np.float32)
+        C = to_gpu(sentinel)
+        with pytest.raises(CgtAmdError, match="shape mismatch"):
+            bcall.call([A3, B3], C)
+        assert np.array_equal(C.get(), sentinel)
+
+
 def test_batched_matmul(cgt):
     # cgt/tests/test_einsum.py, test_affine.py batchedmatmul: (2,3,5) x (2,5,7)
     rs = np.random.RandomState(0)

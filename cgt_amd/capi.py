@@ -52,6 +52,8 @@ PROTOTYPES = {
                             + [c_void_p, c_void_p]),
     "cgt_amd_sgemm": (c_int, [c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p,
                               c_long, c_void_p, c_long, c_void_p]),
+    "cgt_amd_sgemm_noalloc": (c_int, [c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p,
+                                      c_long, c_void_p, c_long, c_void_p]),
     "cgt_amd_sgemm_batched": (c_int, [c_int, c_int, c_long, c_long, c_long, c_long,
                                       c_void_p, c_long, c_long, c_void_p, c_long, c_long,
                                       c_void_p, c_long, c_long, c_void_p]),

@@ -49,6 +49,7 @@
 // about the same time.
 #include "common.h"
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 namespace cgt_amd {
@@ -683,6 +684,42 @@ static float* get_workspace(void* stream, size_t bytes) {
     return stream_workspace(stream, kWsGemm, bytes, "sgemm");
 }
 
+// Scratch of the entry point that allocates nothing (cgt_amd_sgemm_noalloc): the
+// split-K partials / tail pieces live in this file-scope device array instead of a
+// hipMalloc'ed workspace.  Every GPU the library runs on holds its own copy at its own
+// address until the process ends.  In host code `scratch` is only a handle for
+// hipGetSymbolAddress -- the device address is looked up once per device, with that
+// device current, and kept in g_scratch_ptr; kernels, like the workspace kernels above,
+// take that pointer as an argument.
+constexpr size_t kScratchBytes = (size_t)64 << 20;
+static __device__ __align__(256) float scratch[kScratchBytes / sizeof(float)];
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static float* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (nullptr + message on failure).
+static float* scratch_address() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        set_error("sgemm_noalloc: cannot identify the current device");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            (void)hipGetLastError();
+            set_error("sgemm_noalloc: hipGetSymbolAddress(scratch) failed on device %d: %s", dev,
+                      hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = static_cast<float*>(p);
+    }
+    return g_scratch_ptr[dev];
+}
+
 static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
 
 struct TileShape {
@@ -723,7 +760,7 @@ static void launch_trans(int tA, int tB, bool pipe, bool deep, int shape, dim3 g
 
 static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const float* A, long lda,
                          long sA, const float* B, long ldb, long sB, float* C, long ldc, long sC,
-                         void* stream) {
+                         void* stream, bool static_scratch = false) {
     CGT_ARG_CHECK(P >= 0 && M >= 0 && N >= 0 && K >= 0, "sgemm: negative size");
     if (P == 0 || M == 0 || N == 0) return CGT_AMD_OK;
     CGT_ARG_CHECK(A || K == 0, "sgemm: null A");
@@ -745,6 +782,21 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
             shape = i;
         }
     }
+    // where the partial products of a split go: the stream's workspace (grown on demand),
+    // or the static device array when the caller must not allocate
+    int ws_rc = CGT_AMD_ERR_NOMEM;
+    auto workspace = [&](size_t bytes) -> float* {
+        if (!static_scratch) return get_workspace(stream, bytes);
+        if (bytes > kScratchBytes) {
+            set_error("sgemm_noalloc: this product needs %zu bytes of split-K scratch, the static buffer holds %zu "
+                      "(use cgt_amd_sgemm, which allocates a workspace)", bytes, kScratchBytes);
+            ws_rc = CGT_AMD_ERR_ARG;
+            return nullptr;
+        }
+        float* p = scratch_address();
+        if (!p) ws_rc = CGT_AMD_ERR_HIP;
+        return p;
+    };
     GemmArgs a;
     a.A = A; a.B = B; a.C = C;
     a.lda = lda; a.ldb = ldb; a.ldc = ldc;
@@ -768,8 +820,8 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
             a.splits = (int)cdiv(K, a.kchunk);
         }
         if (a.splits > 1) {
-            a.ws = get_workspace(stream, (size_t)a.splits * M * N * sizeof(float));
-            if (!a.ws) return CGT_AMD_ERR_NOMEM;
+            a.ws = workspace((size_t)a.splits * M * N * sizeof(float));
+            if (!a.ws) return ws_rc;
         }
     }
     // tail split (single product, no split-K): tiles beyond the last full
@@ -795,8 +847,8 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
             a.main_wgs = (int)(tiles - r);
             a.tail_kchunk = (int)(cdiv(cdiv(K, best_s), KT) * KT);
             a.tail_splits = (int)cdiv(K, a.tail_kchunk);
-            a.ws = get_workspace(stream, (size_t)tail_tiles * a.tail_splits * kShapes[shape].bm * kShapes[shape].bn * sizeof(float));
-            if (!a.ws) return CGT_AMD_ERR_NOMEM;
+            a.ws = workspace((size_t)tail_tiles * a.tail_splits * kShapes[shape].bm * kShapes[shape].bn * sizeof(float));
+            if (!a.ws) return ws_rc;
         }
     }
     const long wgs = a.splits > 1 ? tiles * a.splits : a.main_wgs + tail_tiles * a.tail_splits;
@@ -838,6 +890,11 @@ using namespace cgt_amd;
 CGT_API int cgt_amd_sgemm(int tA, int tB, long M, long N, long K, const float* A, long lda,
                           const float* B, long ldb, float* C, long ldc, void* stream) {
     return gemm_dispatch(tA, tB, 1, M, N, K, A, lda, 0, B, ldb, 0, C, ldc, 0, stream);
+}
+
+CGT_API int cgt_amd_sgemm_noalloc(int tA, int tB, long M, long N, long K, const float* A, long lda,
+                                  const float* B, long ldb, float* C, long ldc, void* stream) {
+    return gemm_dispatch(tA, tB, 1, M, N, K, A, lda, 0, B, ldb, 0, C, ldc, 0, stream, true);
 }
 
 CGT_API int cgt_amd_sgemm_batched(int tA, int tB, long P, long M, long N, long K, const float* A,

@@ -246,6 +246,22 @@ int cgt_amd_sgemm(int tA, int tB, long M, long N, long K,
                   const float *A, long lda, const float *B, long ldb,
                   float *C, long ldc, void *stream);
 
+/* cgt_amd_sgemm for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  Same arguments, same kernels, same split
+ * plan and therefore bit-identical results; the split-K partials and tail
+ * pieces go to a 64 MiB device array that is part of the library's code object
+ * (one copy per GPU, held until the process ends) instead of a workspace that
+ * cgt_amd_sgemm grows with hipMalloc.  No hipMalloc / hipFree is ever called.
+ * A product whose plan needs more than 64 MiB of partials (e.g. a weight
+ * gradient with M*N*splits > 16 M floats) is refused with CGT_AMD_ERR_ARG and a
+ * message naming both sizes.  All calls on one GPU share the array: calls that
+ * overlap in time on different streams of the same GPU race on it -- issue them
+ * on one stream, or order them with events. */
+int cgt_amd_sgemm_noalloc(int tA, int tB, long M, long N, long K,
+                          const float *A, long lda, const float *B, long ldb,
+                          float *C, long ldc, void *stream);
+
 /* P independent products at A + p*strideA, B + p*strideB, C + p*strideC.
  * Replaces the cblas_sgemm loop of BatchedMul22 (cgt/core.py:2272-2285);
  * the reference has no GPU implementation of it.  A stride of 0 shares one

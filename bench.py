@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the CGT CNN hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--only] [--no-cpu]
 
 A step is one forward+backward pass of one configured layer over one batch of
 synthetic input, every buffer resident in HBM before the timed region:
@@ -12,10 +12,15 @@ synthetic input, every buffer resident in HBM before the timed region:
 Prints ONE JSON line: the headline conv2d fwd+bwd TFLOP/s over the whole
 step, a per-kernel table (HIP-event timed on the launch stream) with GB/s or
 TFLOP/s against the MI355X roofs, the roofline of the dominant kernel (the
-MFMA GEMM) and the CPU path timed on this box's host cores on a bounded
-sample.
+MFMA GEMM, its HBM traffic read from the counter summaries under profiles/)
+and the CPU path timed on this box's host cores on a bounded sample.  The
+headline workload is the VGG-style layer; the default run then measures the
+other configurations the same way (AlexNet conv1 with LRN and pool, the raw
+Mul22 / BatchedMul22 products, the CIFAR and MNIST first layers, whose GEMMs
+sit under the HBM roof and are reported against both roofs) under "workloads".
 """
 import argparse
+import gc
 import json
 import os
 import sys
@@ -34,10 +39,15 @@ WORKLOADS = {
     "vgg_mid_conv3x3_128x56x56_b64": dict(
         x=(64, 128, 56, 56), f=(128, 128, 3, 3), pad=(1, 1), stride=(1, 1),
         fscale="he", lrn=None, pool=((2, 2), (0, 0), (2, 2))),
-    # AlexNet conv1 -> LRN -> pool
+    # AlexNet conv1 -> LRN (k = 2, as the configuration states it; the reference's own LRN
+    # has k fixed at 1, the kernel and its cost are the same) -> pool
     "alexnet_conv1_11x11s4_3x227x227_b128": dict(
         x=(128, 3, 227, 227), f=(96, 3, 11, 11), pad=(0, 0), stride=(4, 4),
-        fscale=0.01, lrn=(5, 1e-4, 0.75, 1.0), pool=((3, 3), (0, 0), (2, 2))),
+        fscale=0.01, lrn=(5, 1e-4, 0.75, 2.0), pool=((3, 3), (0, 0), (2, 2))),
+    # first conv of the CIFAR stack: K = 75, N = 32 -- a GEMM under the HBM roof
+    "cifar_conv1_5x5_3x32x32_b128": dict(
+        x=(128, 3, 32, 32), f=(32, 3, 5, 5), pad=(2, 2), stride=(1, 1),
+        fscale=0.01, lrn=None, pool=((3, 3), (0, 0), (2, 2))),
     # second conv of the CIFAR stack (with its pool + LRN input side)
     "cifar_conv2_5x5_32x15x15_b128": dict(
         x=(128, 32, 15, 15), f=(64, 32, 5, 5), pad=(2, 2), stride=(1, 1),
@@ -51,17 +61,66 @@ WORKLOADS = {
 GEMM_WORKLOAD = "raw_gemm_4096_and_batched_64x512"
 DEFAULT_WORKLOAD = "vgg_mid_conv3x3_128x56x56_b64"
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs of this script (summaries and calibration in profiles/):
-# (workload, stage) -> bytes.  None where no counter run has been made.
-TRAFFIC = {
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_fwd_NT"): 1088700000,    # 2.0 * 486.7 MB fetched + 115.3 MB written
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_dgrad_NN"): 1095000000,  # 2.0 * 85.1 + 924.8
-    ("vgg_mid_conv3x3_128x56x56_b64", "gemm_wgrad_TN"): 1128100000,  # 2.0 * 531.0 + 66.1 (split-K partials incl.)
-    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_fwd_NT"): 830300000,     # 2.0 * 340.8 + 148.7
-    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_dgrad_NN"): 801100000,   # 2.0 * 101.4 + 598.3 (rows of 363 floats)
-    ("alexnet_conv1_11x11s4_3x227x227_b128", "gemm_wgrad_TN"): 1087100000,  # 2.0 * 518.3 + 50.5 (partials incl.)
+# The workloads the default run reports beside the headline one, under "workloads"
+EXTRA_WORKLOADS = ["alexnet_conv1_11x11s4_3x227x227_b128", GEMM_WORKLOAD, "cifar_conv1_5x5_3x32x32_b128",
+                   "mnist_conv3x3_1x28x28_b64"]
+
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries of this script, per workload
+PROFILE_PREFIX = {
+    "vgg_mid_conv3x3_128x56x56_b64": "vgg_mid_conv3x3_b64",
+    "alexnet_conv1_11x11s4_3x227x227_b128": "alexnet_conv1_b128",
 }
+
+
+def _pmc_rows(path):
+    """(scale, rows) of a counter summary: `scale` is the calibration factor its header
+    states ("factor: X"), rows are (kernel name, MB per launch) in the file's order, which is
+    the order of first launch inside a step."""
+    import re
+    scale, rows = None, []
+    with open(path) as fh:
+        for line in fh:
+            m = re.match(r"factor:\s*([0-9.]+)", line)
+            if m:
+                scale = float(m.group(1))
+                continue
+            parts = line.rstrip("\n").rsplit(None, 4)
+            if len(parts) == 5 and "kernel" in parts[0] and parts[0].strip() != "kernel":
+                try:
+                    rows.append((parts[0].strip(), float(parts[4])))
+                except ValueError:
+                    pass
+    return scale, rows
+
+
+def traffic_from_profiles(workload, profiles_dir=None):
+    """HBM bytes per launch of each GEMM stage of a step, read from the committed counter
+    summaries: stage -> calibrated FETCH_SIZE + WRITE_SIZE bytes of the sgemm launch and of
+    the reduce kernel that follows it (split-K / tail partials).  The summaries list kernels
+    in launch order, so the sgemm rows are, in order, the forward product, the data gradient
+    and the weight gradient.  {} when the workload has no summaries."""
+    prefix = PROFILE_PREFIX.get(workload)
+    profiles_dir = profiles_dir or os.path.join(ROOT, "profiles")
+    if prefix is None:
+        return {}
+    total = {}
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        path = os.path.join(profiles_dir, "%s_pmc_%s.txt" % (prefix, counter))
+        if not os.path.exists(path):
+            return {}
+        scale, rows = _pmc_rows(path)
+        if scale is None:
+            return {}
+        order = iter(["gemm_fwd_NT", "gemm_dgrad_NN", "gemm_wgrad_TN"])
+        stage = None
+        for name, mb in rows:
+            if "sgemm_kernel" in name:
+                stage = next(order, None)
+            elif "reduce_kernel" not in name:
+                stage = None if stage is None else "-"     # another kernel: later reduce rows are not this GEMM's
+            if stage not in (None, "-") and ("sgemm_kernel" in name or "reduce_kernel" in name):
+                total[stage] = total.get(stage, 0.0) + scale * mb * 1e6
+    return {k: int(round(v)) for k, v in total.items()}
 
 
 def make_inputs(cfg, batch=None, seed=0):
@@ -80,8 +139,9 @@ def make_inputs(cfg, batch=None, seed=0):
 
 
 class Stage(object):
-    def __init__(self, name, kernel, fn, work, bound):
+    def __init__(self, name, kernel, fn, work, bound, operand_bytes=None):
         self.name, self.kernel, self.fn, self.work, self.bound = name, kernel, fn, work, bound
+        self.operand_bytes = operand_bytes      # GEMM stages: 4 * (|A| + |B| + |C|), the compulsory traffic
         self.ms = self.ms_median = self.ms_min = self.ms_in_step = None
 
 
@@ -118,10 +178,11 @@ class LayerOnGpu(object):
         nelem = lambda a: int(np.prod(a.shape))  # noqa: E731
         st = []
         s = stream
+        gemm_bytes = 4 * (Bmn * Z + L * Z + Bmn * L)      # the three conv products touch the same three matrices
         st.append(Stage("im2col", "im2col_linear_kernel or im2col_pipe_kernel", lambda: K.im2col(self.x, (r, c), pad, stride, out=self.col, stream=s),
                         4 * (nelem(self.x) + nelem(self.col)), "hbm"))
         st.append(Stage("gemm_fwd_NT", "sgemm_kernel", lambda: K.mul22(self.col2, self.f_LZ, False, True, out=self.y_mnL, stream=s),
-                        2 * Bmn * L * Z, "mfma"))
+                        2 * Bmn * L * Z, "mfma", gemm_bytes))
         st.append(Stage("transpose_0312", "thin_transpose_kernel or batched_transpose_kernel",
                         lambda: K.transpose4(self.y_mnL.reshape(B, m, n, L), (0, 3, 1, 2), out=self.y, stream=s),
                         2 * 4 * nelem(self.y), "hbm"))
@@ -162,12 +223,12 @@ class LayerOnGpu(object):
         st.append(Stage("transpose_0231", "thin_transpose_kernel or batched_transpose_kernel", lambda: K.transpose4(self.gy, (0, 2, 3, 1), out=self.gc, stream=s),
                         2 * 4 * nelem(self.y), "hbm"))
         st.append(Stage("gemm_dgrad_NN", "sgemm_kernel", lambda: K.mul22(self.gc2, self.f_LZ, False, False, out=self.gcol, stream=s),
-                        2 * Bmn * L * Z, "mfma"))
+                        2 * Bmn * L * Z, "mfma", gemm_bytes))
         st.append(Stage("col2im", "col2im_stream_kernel",
                         lambda: K.col2im(self.gcol.reshape(B, m, n, Z), self.x.shape, (r, c), pad, stride, out=self.gx, stream=s),
                         4 * (nelem(self.x) + nelem(self.col)), "hbm"))
         st.append(Stage("gemm_wgrad_TN", "sgemm_kernel", lambda: K.mul22(self.gc2, self.col2, True, False, out=self.gf, stream=self._wgrad_stream),
-                        2 * Bmn * L * Z, "mfma"))
+                        2 * Bmn * L * Z, "mfma", gemm_bytes))
         self.stages = st
         self.conv_flops = 6 * Bmn * L * Z
         # The glue a SpatialConvolution training step adds around this layer
@@ -282,9 +343,10 @@ class GemmOnGpu(object):
         for tA, tB, name in [(False, False, "NN"), (False, True, "NT"), (True, False, "TN"), (True, True, "TT")]:
             st.append(Stage("mul22_%s_%d" % (name, n), "sgemm_kernel",
                             (lambda tA=tA, tB=tB: K.mul22(self.A, self.B, tA, tB, out=self.C, stream=s)),
-                            2 * n ** 3, "mfma"))
+                            2 * n ** 3, "mfma", 12 * n * n))
         st.append(Stage("batched_mul22_%dx%d" % (P, nb), "sgemm_kernel",
-                        lambda: K.batched_mul22(self.bA, self.bB, out=self.bC, stream=s), 2 * P * nb ** 3, "mfma"))
+                        lambda: K.batched_mul22(self.bA, self.bB, out=self.bC, stream=s), 2 * P * nb ** 3, "mfma",
+                        12 * P * nb * nb))
         self.stages = st
         self.overlap = False
         self.conv_flops = sum(x.work for x in st)
@@ -403,40 +465,18 @@ def cpu_gemm_baseline(n=2048):
                       % (n, reps, CB.blas_config(), threads, CB.cpu_model())}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS) + [GEMM_WORKLOAD])
-    ap.add_argument("--stage-reps", type=int, default=20)
-    ap.add_argument("--cpu-sample", type=int, default=16, help="images in the CPU baseline sample")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--overlap", action="store_true",
-                    help="issue the weight-gradient GEMM on a second stream beside col2im (default: one stream, "
-                         "which measures faster since the GEMM epilogues were trimmed)")
-    ap.add_argument("--no-overlap", action="store_true", help="accepted for older command lines: one stream is the default")
-    ap.add_argument("--glue", action="store_true",
-                    help="also time the conv-layer glue kernels (bias add, ReLU, their gradients, loss sum) on the "
-                         "layer's activation; they appear in `glue_stages`, outside the step")
-    ap.add_argument("--no-op-api", action="store_true", help="skip timing the same step through the Op API")
-    ap.add_argument("--no-check", action="store_true",
-                    help="skip the parity gate (profiling runs: keeps its small launches out of the kernel statistics)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (the hot path has no "
-                 "multi-GPU part: it would shard the batch axis)" % args.gpus)
-
+def measure(workload, args, primary):
+    """Run one workload: timed steps, both stage clocks, the stage table.  Returns the
+    fields of the JSON line that describe it (the caller adds the Op API and CPU legs)."""
     from cgt_amd import capi
-    capi.require_gpu()
-    is_gemm = args.workload == GEMM_WORKLOAD
+    is_gemm = workload == GEMM_WORKLOAD
     if is_gemm:
         cfg = {"x": [4096, 4096], "f": [4096, 4096], "pad": [], "stride": []}
         layer = GemmOnGpu()
         parity = {"ok": True, "skipped": True} if args.no_check else check_gemm_against_oracle()
     else:
-        cfg = WORKLOADS[args.workload]
-        layer = LayerOnGpu(cfg, overlap=args.overlap and not args.no_overlap, glue=args.glue)
+        cfg = WORKLOADS[workload]
+        layer = LayerOnGpu(cfg, overlap=primary and args.overlap and not args.no_overlap, glue=primary and args.glue)
         parity = {"ok": True, "skipped": True} if args.no_check else check_against_oracle(cfg)
 
     for _ in range(args.warmup):
@@ -456,8 +496,9 @@ def main():
     # the same buffers they find part of them in the 256 MB last-level cache; GEMMs look worse:
     # the chip holds a lower clock under sustained matrix load).  --stage-reps 0 skips the second.
     in_step_steps = max(5, min(args.steps, 20))
-    if args.stage_reps > 0 or is_gemm or args.glue or getattr(layer, "overlap", False):
-        layer.time_stages(max(args.stage_reps, 1))
+    stage_reps = args.stage_reps if primary or is_gemm else 0      # extra layers: the in-step clock only
+    if stage_reps > 0 or is_gemm or (primary and args.glue) or getattr(layer, "overlap", False):
+        layer.time_stages(max(stage_reps, 1))
     if not is_gemm:
         layer.time_stages_in_step(in_step_steps)
 
@@ -484,6 +525,14 @@ def main():
         if st.bound == "mfma":
             gemm_flops += st.work
             gemm_ms += clock(st)
+            # both roofs: a product with a short K (the CIFAR / MNIST first layers) moves more
+            # bytes per flop than the chip's 19.7 flop/byte balance and sits under the HBM roof
+            if getattr(st, "operand_bytes", None):
+                gbs = st.operand_bytes / (clock(st) * 1e-3) / 1e9
+                intensity = st.work / st.operand_bytes
+                row.update({"bytes": st.operand_bytes, "GBps_operands": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
+                            "flop_per_byte": round(intensity, 2),
+                            "roof": "hbm" if intensity < FP32_MFMA_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS else "mfma"})
         stages.append(row)
     glue_stages = []
     for st in getattr(layer, "extra_stages", []):
@@ -492,18 +541,19 @@ def main():
                             "bytes": st.work, "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4)})
     gemm_tf = gemm_flops / (gemm_ms * 1e-3) / 1e12
     value = layer.conv_flops / (ms_per_step * 1e-3) / 1e12
-
-    out = {
-        "metric": "conv2d fwd+bwd TFLOP/s (% fp32 MFMA peak); pool/LRN/im2col GB/s (% HBM)",
-        "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": args.workload, "x": list(cfg["x"]), "filters": list(cfg["f"]),
-                   "pad": list(cfg["pad"]), "stride": list(cfg["stride"]),
-                   "value_is": "conv GEMM flops (6*B*m*n*L*Z) / whole step time incl. im2col, col2im, "
-                               "transposes, pool and LRN stages",
-                   "schedule": ("one stream" if is_gemm or args.no_overlap or not args.overlap else
-                                "weight-gradient GEMM on a second stream beside col2im")},
+    traffic = traffic_from_profiles(workload).get(dominant.name)
+    config = {"workload": workload, "x": list(cfg["x"]), "filters": list(cfg["f"]),
+              "pad": list(cfg["pad"]), "stride": list(cfg["stride"]),
+              "value_is": "conv GEMM flops (6*B*m*n*L*Z) / whole step time incl. im2col, col2im, "
+                          "transposes, pool and LRN stages",
+              "schedule": ("one stream" if not getattr(layer, "overlap", False) else
+                           "weight-gradient GEMM on a second stream beside col2im")}
+    if is_gemm:
+        config["value_is"] = "flops of Mul22 4096^3 x {NN,NT,TN,TT} + BatchedMul22 64x512^3 / step time"
+    elif cfg.get("lrn"):
+        config["lrn"] = dict(zip(("size", "alpha", "beta", "k"), cfg["lrn"]))
+    res = {
+        "value": round(value, 3), "ms_per_step": round(ms_per_step, 4), "config": config,
         "frac_fp32_mfma_peak": round(value / FP32_MFMA_PEAK_TFLOPS, 4),
         # the dominant kernel: the slowest MFMA GEMM launch of a step
         "roofline": {"bound": "mfma", "kernel": dominant.kernel, "stage": dominant.name,
@@ -513,31 +563,83 @@ def main():
                      "flops_per_launch": dominant.work, "avg_launch_ms": round(clock(dominant), 4),
                      "timing": ("HIP events around the launch inside %d consecutive steps" % in_step_steps
                                 if getattr(dominant, "ms_in_step", None) is not None else
-                                "HIP events around %d back-to-back launches" % max(args.stage_reps, 1)),
+                                "HIP events around %d back-to-back launches" % max(stage_reps, 1)),
                      "avg_launch_ms_back_to_back": None if dominant.ms is None else round(dominant.ms, 4),
-                     "traffic": TRAFFIC.get((args.workload, dominant.name))},
+                     "traffic": traffic,
+                     "traffic_source": None if traffic is None else
+                     "profiles/%s_pmc_{FETCH,WRITE}_SIZE.txt, calibrated" % PROFILE_PREFIX[workload]},
         "gemm_all_launches": {"TFLOPs": round(gemm_tf, 2), "frac": round(gemm_tf / FP32_MFMA_PEAK_TFLOPS, 4)},
         "stages": stages,
         "glue_stages": glue_stages,
         "parity": parity,
-        "device": capi.device_name(),
     }
-    if is_gemm:
-        out["config"]["value_is"] = "flops of Mul22 4096^3 x {NN,NT,TN,TT} + BatchedMul22 64x512^3 / step time"
-    elif not args.no_op_api:
-        del layer        # the traced graph holds its own buffers
+    del layer, dominant, st
+    gc.collect()            # the stage closures and the layer reference each other
+    return res, cfg
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS) + [GEMM_WORKLOAD])
+    ap.add_argument("--stage-reps", type=int, default=20)
+    ap.add_argument("--cpu-sample", type=int, default=16, help="images in the CPU baseline sample")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--overlap", action="store_true",
+                    help="issue the weight-gradient GEMM on a second stream beside col2im (default: one stream, "
+                         "which measures faster since the GEMM epilogues were trimmed)")
+    ap.add_argument("--no-overlap", action="store_true", help="accepted for older command lines: one stream is the default")
+    ap.add_argument("--glue", action="store_true",
+                    help="also time the conv-layer glue kernels (bias add, ReLU, their gradients, loss sum) on the "
+                         "layer's activation; they appear in `glue_stages`, outside the step")
+    ap.add_argument("--no-op-api", action="store_true", help="skip timing the same step through the Op API")
+    ap.add_argument("--no-check", action="store_true",
+                    help="skip the parity gate (profiling runs: keeps its small launches out of the kernel statistics)")
+    ap.add_argument("--only", action="store_true",
+                    help="measure --workload alone (profiling runs); by default the headline workload is followed by "
+                         "the other configurations, reported under `workloads`")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (the hot path has no "
+                 "multi-GPU part: it would shard the batch axis)" % args.gpus)
+
+    from cgt_amd import capi
+    capi.require_gpu()
+    is_gemm = args.workload == GEMM_WORKLOAD
+    res, cfg = measure(args.workload, args, primary=True)
+    out = {
+        "metric": "conv2d fwd+bwd TFLOP/s (% fp32 MFMA peak); pool/LRN/im2col GB/s (% HBM)",
+        "value": res["value"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": res["ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+    }
+    out.update({k: v for k, v in res.items() if k not in ("value", "ms_per_step")})
+    out["device"] = capi.device_name()
+    parity_ok = res["parity"]["ok"]
+    if not is_gemm and not args.no_op_api:
         ms, n_instr = op_api_step_ms(cfg, args.steps, args.warmup)
-        out["op_api_step"] = {"ms_per_step": round(ms, 4), "TFLOPs": round(value * ms_per_step / ms, 3),
+        out["op_api_step"] = {"ms_per_step": round(ms, 4), "TFLOPs": round(res["value"] * res["ms_per_step"] / ms, 3),
                               "instructions": n_instr,
                               "what": "the same step through nn.conv2d / cross_channel_lrn / max_pool_2d + grad, compiled "
                                       "with cgt.function and replayed by the C++ interpreter (one stream)"}
+    # the other configurations, same measurement (their stage tables carry the in-step clock;
+    # the raw GEMMs, which have no step around them, the back-to-back one)
+    if not args.only and args.workload == DEFAULT_WORKLOAD:
+        out["workloads"] = {}
+        for name in EXTRA_WORKLOADS:
+            r, _ = measure(name, args, primary=False)
+            parity_ok = parity_ok and r["parity"]["ok"]
+            r["unit"] = "TFLOP/s"
+            out["workloads"][name] = r
     if not args.no_cpu and not is_gemm:
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample)
     elif not args.no_cpu:
         out["cpu_baseline"] = cpu_gemm_baseline()
     print(json.dumps(out))
-    if not parity["ok"]:
-        sys.exit("bench.py: parity gate failed: %r" % (parity,))
+    if not parity_ok:
+        sys.exit("bench.py: parity gate failed")
 
 
 if __name__ == "__main__":

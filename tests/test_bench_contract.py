@@ -22,6 +22,39 @@ def test_more_than_one_gpu_is_refused():
     assert "one GPU" in (proc.stdout + proc.stderr)
 
 
+def _traffic_by_hand(workload, stage):
+    """2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE megabytes of the stage's sgemm launch and the reduce
+    kernel behind it, read from the summaries with nothing but string splitting."""
+    prefix = {"vgg_mid_conv3x3_128x56x56_b64": "vgg_mid_conv3x3_b64"}[workload]
+    nth = ["gemm_fwd_NT", "gemm_dgrad_NN", "gemm_wgrad_TN"].index(stage)
+    total = 0.0
+    for counter, factor in (("FETCH_SIZE", 2.0), ("WRITE_SIZE", 1.0)):
+        lines = open(os.path.join(ROOT, "profiles", "%s_pmc_%s.txt" % (prefix, counter))).read().splitlines()
+        assert "factor: %s" % factor in lines
+        seen, take = -1, False
+        for ln in lines:
+            if "_kernel" not in ln or ln.startswith(("command", "kernel ")):
+                continue
+            if "sgemm_kernel" in ln:
+                seen += 1
+                take = seen == nth
+            elif "reduce_kernel" not in ln:
+                take = False
+            if take:
+                total += factor * float(ln.split()[-1]) * 1e6
+    return int(round(total))
+
+
+def test_traffic_is_read_from_the_profile_summaries():
+    import bench
+    t = bench.traffic_from_profiles("vgg_mid_conv3x3_128x56x56_b64")
+    assert set(t) == {"gemm_fwd_NT", "gemm_dgrad_NN", "gemm_wgrad_TN"}
+    for stage, v in t.items():
+        assert v == _traffic_by_hand("vgg_mid_conv3x3_128x56x56_b64", stage)
+        assert 1.0e9 < v < 1.3e9          # 1028 MB algorithmic per product of the VGG layer
+    assert bench.traffic_from_profiles("mnist_conv3x3_1x28x28_b64") == {}
+
+
 @pytest.mark.gpu
 def test_default_workload_prints_the_contract_line():
     proc = _run(["--steps", "2", "--warmup", "1", "--stage-reps", "2", "--cpu-sample", "2"], 600)
@@ -45,6 +78,22 @@ def test_default_workload_prints_the_contract_line():
     assert "inside" in roof["timing"] and roof["avg_launch_ms"] > 0
     for row in out["stages"]:
         assert row["ms_in_step"] > 0 and row["ms"] > 0 and 0 < row["frac_in_step"] < 1.2
+    # the traffic figure is what the committed counter summaries say, not a constant
+    import bench
+    assert roof["traffic"] == _traffic_by_hand(out["config"]["workload"], roof["stage"])
+    assert roof["traffic"] == bench.traffic_from_profiles(out["config"]["workload"])[roof["stage"]]
+    # the other configurations ride along: AlexNet conv1 (LRN both ways, k = 2), the raw products,
+    # and the first layers whose GEMMs are priced against both roofs
+    w = out["workloads"]
+    alex = w["alexnet_conv1_11x11s4_3x227x227_b128"]
+    assert alex["config"]["lrn"]["k"] == 2.0
+    names = [r["stage"] for r in alex["stages"]]
+    assert "lrn_fwd" in names and "lrn_bwd" in names and "max_pool_bwd" in names
+    assert all(r["ms_in_step"] > 0 for r in alex["stages"])
+    assert len(w["raw_gemm_4096_and_batched_64x512"]["stages"]) == 5
+    for name in ("cifar_conv1_5x5_3x32x32_b128", "mnist_conv3x3_1x28x28_b64"):
+        gemms = [r for r in w[name]["stages"] if r["bound"] == "mfma"]
+        assert len(gemms) == 3 and all(r["roof"] == "hbm" and r["frac_hbm"] > 0 and r["frac_in_step"] > 0 for r in gemms)
     cpu = out["cpu_baseline"]
     assert cpu["kind"] in ("port", "reference") and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
     assert out["parity"]["ok"] is True

@@ -73,13 +73,112 @@ class TupleType(object):
         return hash(self.eltypes)
 
 
+# ================================================================ symbolic extents
+
+class ShapeInt(int):
+    """An array extent that remembers how it was computed.
+
+    The reference derives every shape symbolically (Size ops and integer
+    arithmetic over them, cgt/core.py:1614-1640 and the shp_apply rules), so a
+    compiled function serves any batch size.  Nodes here are evaluated while
+    they are built, so an extent is a concrete python int -- this subclass --
+    that also carries its expression:
+        ("const", v) | ("size", node, axis) | (op, a, b) with op in + - * // ceildiv | ("neg", a)
+    `function` turns the expressions that depend on its arguments into
+    Size / integer-op instructions; everywhere else a ShapeInt is just an int.
+    """
+
+    def __new__(cls, value, expr=None):
+        self = int.__new__(cls, value)
+        self.expr = ("const", int(value)) if expr is None else expr
+        return self
+
+    @staticmethod
+    def _expr(v):
+        return v.expr if isinstance(v, ShapeInt) else ("const", int(v))
+
+    def _bin(self, other, op, value, swap=False):
+        if not isinstance(other, (int, np.integer)) or isinstance(other, bool):
+            return NotImplemented
+        a, b = (ShapeInt._expr(other), self.expr) if swap else (self.expr, ShapeInt._expr(other))
+        if a[0] == "const" and b[0] == "const":
+            return ShapeInt(value)
+        return ShapeInt(value, (op, a, b))
+
+    def __add__(self, o):
+        return self._bin(o, "+", int(self) + int(o)) if isinstance(o, (int, np.integer)) else NotImplemented
+
+    def __radd__(self, o):
+        return self._bin(o, "+", int(o) + int(self), True) if isinstance(o, (int, np.integer)) else NotImplemented
+
+    def __sub__(self, o):
+        return self._bin(o, "-", int(self) - int(o)) if isinstance(o, (int, np.integer)) else NotImplemented
+
+    def __rsub__(self, o):
+        return self._bin(o, "-", int(o) - int(self), True) if isinstance(o, (int, np.integer)) else NotImplemented
+
+    def __mul__(self, o):
+        return self._bin(o, "*", int(self) * int(o)) if isinstance(o, (int, np.integer)) else NotImplemented
+
+    def __rmul__(self, o):
+        return self._bin(o, "*", int(o) * int(self), True) if isinstance(o, (int, np.integer)) else NotImplemented
+
+    def __floordiv__(self, o):
+        return self._bin(o, "//", int(self) // int(o)) if isinstance(o, (int, np.integer)) else NotImplemented
+
+    def __rfloordiv__(self, o):
+        return self._bin(o, "//", int(o) // int(self), True) if isinstance(o, (int, np.integer)) else NotImplemented
+
+    def __neg__(self):
+        return ShapeInt(-int(self), None if self.expr[0] == "const" else ("neg", self.expr))
+
+    def is_constant(self):
+        return self.expr[0] == "const"
+
+    @staticmethod
+    def _lift(v):
+        return v if isinstance(v, ShapeInt) else ShapeInt(int(v))
+
+    def __reduce__(self):
+        return (int, (int(self),))
+
+
+def ceil_divide(x, y):
+    """max(0, iceil(x / y)), the pooled-extent rule (reference cgt/api.py:145-146 as
+    MaxPool.shp_apply uses it), symbolic when an operand is."""
+    v = max(0, -((-int(x)) // int(y)))
+    a, b = ShapeInt._expr(x), ShapeInt._expr(y)
+    if a[0] == "const" and b[0] == "const":
+        return ShapeInt(v)
+    return ShapeInt(v, ("ceildiv", a, b))
+
+
+def shape_depends_on(expr, out=None):
+    """The nodes whose extents a shape expression reads."""
+    out = [] if out is None else out
+    if expr[0] == "size":
+        out.append(expr[1])
+    elif expr[0] != "const":
+        for sub in expr[1:]:
+            shape_depends_on(sub, out)
+    return out
+
+
 # ================================================================ nodes
 
 class Node(object):
     """A value together with how it was made (op, parents)."""
 
-    def __init__(self, typ, op, parents, value, name=None):
+    def __init__(self, typ, op, parents, value, name=None, shape_sym=None, scalar_expr=None):
         self.typ, self.op, self.parents, self.value, self.name = typ, op, list(parents), value, name
+        # extents as ShapeInts (a tuple of such lists for a tuple-valued node); None: taken
+        # from the value, each extent then reads "size of this node along that axis"
+        self.shape_sym = shape_sym
+        # for an int64 scalar leaf that stands for an extent: the expression it came from
+        self.scalar_expr = scalar_expr
+        # a constant whose VALUE was computed from an extent (e.g. the 1/n of a mean): a
+        # compiled function that contains it is tied to the shapes it was traced with
+        self.shape_baked = False
 
     @property
     def ndim(self):
@@ -91,7 +190,12 @@ class Node(object):
 
     @property
     def shape(self):
-        return tuple(self.value.shape)
+        """Extents as ShapeInts (plain ints to every consumer that does not care)."""
+        if self.shape_sym is not None and not isinstance(self.typ, TupleType):
+            return tuple(self.shape_sym)
+        if isinstance(self.typ, TupleType):
+            raise TypeError("a tuple-valued node has no single shape")
+        return tuple(ShapeInt(d, ("size", self, i)) for i, d in enumerate(self.value.shape))
 
     @property
     def devtype(self):
@@ -182,6 +286,10 @@ def constant(value, devtype=None):
         return value
     if isinstance(value, GpuArray):
         return Node(_value_type(value), None, [], value)
+    if isinstance(value, ShapeInt):
+        # an extent used as an operand (Reshape / Col2Im / Repeat / Fill take their shape
+        # operands as int64 host scalars): the node remembers the expression
+        return Node(TensorType("i8", 0), None, [], np.array(int(value), np.int64), scalar_expr=value.expr)
     arr = np.asarray(value)
     if arr.dtype.kind == "f":
         if devtype == "cpu":
@@ -196,12 +304,19 @@ to_device = constant
 
 
 def shape(x):
-    """Shape as a list of python ints (the reference returns symbolic scalars)."""
-    return [int(s) for s in as_node(x).shape]
+    """Shape as a list of ShapeInts: python ints that remember the expression they came
+    from (the reference returns symbolic scalar nodes)."""
+    return list(as_node(x).shape)
 
 
 def size(x, axis):
     return shape(x)[axis]
+
+
+def scalar_extent(node):
+    """The extent an int64 scalar operand stands for, with its expression."""
+    node = as_node(node)
+    return ShapeInt(int(np.asarray(node.value)), node.scalar_expr)
 
 
 # ================================================================ Op base
@@ -244,6 +359,12 @@ class Op(object):
     def get_native_compile_info(self, input_types, devtype):
         """Returns NativeCompileInfo."""
         raise MethodNotDefined
+
+    def get_gpu_deref_mask(self, input_types):
+        """Which inputs the op's GPU closure dereferences on the device: the
+        gpu_deref_mask of its NativeCompileInfo (all of them if it declares none)."""
+        mask = self.get_native_compile_info(list(input_types), "gpu").gpu_deref_mask
+        return tuple(mask) if mask is not None else (True,) * len(input_types)
 
     def get_py_func(self, input_types):
         raise MethodNotDefined
@@ -353,20 +474,71 @@ def _alloc(typ, shp):
     return empty(tuple(int(s) for s in shp), np.dtype(typ.dtype))
 
 
+_DEREF_MASKS = {}
+
+
+def determine_device(op, parents):
+    """Device an op's result lives on (the rule of the reference's determine_devices,
+    cgt/compilation.py:45-80, for this build's ops): by-value views and Transport follow
+    their definition, every computing op is native_gpu; int64 scalars never reach here --
+    they are leaves and stay on the host."""
+    if isinstance(op, Transport):
+        return op.dev
+    if op.return_type == "byval":
+        return parents[0].devtype
+    return "gpu" if "native_gpu" in op.available_impls else "cpu"
+
+
+def add_transports(op, parents, devtype):
+    """The parents `op` will actually read: a parent that lives on another device than
+    the op is replaced by a Transport of it -- but only if the op dereferences that input
+    on its own device, which is what its gpu_deref_mask says (reference
+    cgt/compilation.py:285-304 ships EVERY cross-device parent and carries the note
+    "look at native compilation info, gpu deref mask"; core.py:748 declares the mask).
+    Shape operands and repeat counts (mask False) are read in place on the host.  One
+    Transport per (node, device), shared by all its consumers, as the reference's
+    dev2copy does."""
+    if isinstance(op, Transport) or devtype != "gpu":
+        return parents
+    key = (op.get_hash(), tuple(p.typ for p in parents))
+    if key not in _DEREF_MASKS:
+        _DEREF_MASKS[key] = op.get_gpu_deref_mask([p.typ for p in parents])
+    nci_mask = _DEREF_MASKS[key]
+    placed = []
+    for p, deref in zip(parents, nci_mask):
+        if deref and p.devtype != devtype and not isinstance(p.typ, TupleType):
+            copies = p.__dict__.setdefault("_transports", {})
+            if devtype not in copies:
+                copies[devtype] = Result(Transport(devtype), [p])
+            p = copies[devtype]
+        placed.append(p)
+    return placed
+
+
 def Result(op, parents):
     """Apply `op` to `parents` now and return the Node that holds the result.
-    (In the reference this only builds the graph node, core.py:511-517; the
-    Alloc + ReturnByRef pair that runs it comes from the compilation pipeline.)"""
+    (In the reference this only builds the graph node, core.py:511-517; device
+    placement, the Transports and the Alloc + ReturnByRef pair that runs it come
+    from the compilation pipeline.  Here placement happens as the node is built,
+    by the same rules, so that the traced graph `function` compiles already has
+    its Transport nodes.)"""
     parents = [as_node(p) for p in parents]
+    parents = add_transports(op, parents, determine_device(op, parents))
     input_types = [p.typ for p in parents]
     typ = op.typ_apply(input_types)
-    if "python" in op.available_impls and (op.return_type == "byval" or "native_gpu" not in op.available_impls):
+    shp = op.shp_apply(parents)
+    if "python" in op.available_impls and (op.return_type == "byval" or "native_gpu" not in op.available_impls
+                                           or isinstance(op, Transport)):
         value = op.get_py_func(input_types)([p.value for p in parents])
     else:
-        out = _alloc(typ, op.shp_apply(parents))
+        out = _alloc(typ, shp)
         get_callable(op, input_types, "gpu").call([p.value for p in parents], out)
         value = out
-    return Node(typ, op, parents, value)
+    if isinstance(typ, TupleType):
+        shape_sym = tuple([ShapeInt._lift(d) for d in s] for s in shp)
+    else:
+        shape_sym = [ShapeInt._lift(d) for d in shp]
+    return Node(typ, op, parents, value, shape_sym=shape_sym)
 
 
 class TupleIndex(Op):
@@ -388,6 +560,9 @@ class TupleIndex(Op):
 
     def typ_apply(self, input_types):
         return input_types[0][self.idx]
+
+    def shp_apply(self, inputs):
+        return list(inputs[0].shape_sym[self.idx])
 
     def get_py_func(self, input_types):
         return lambda reads: reads[0][self.idx]
@@ -647,6 +822,9 @@ class Reshape(Op):
     def typ_apply(self, input_types):
         return TensorType(input_types[0].dtype, len(input_types) - 1)
 
+    def shp_apply(self, inputs):
+        return [scalar_extent(s) for s in inputs[1:]]
+
     def get_py_func(self, input_types):
         def f(reads):
             return reads[0].reshape(tuple(int(np.asarray(s)) for s in reads[1:]))
@@ -657,15 +835,32 @@ class Reshape(Op):
 
 
 class Transport(Op):
-    """Copy between host and device (reference core.py:1596-1612: cgt_copy_object)."""
-    available_impls = ("python",)
+    """Copy to another device (reference core.py:1596-1612: cgt_copy_object).  Evaluated
+    in python while nodes are built; a compiled `function` replays the native closure
+    into an array Alloc'ed on the target device."""
+    available_impls = ("python", "native_cpu", "native_gpu")
 
     def __init__(self, dev):
         assert dev in ("cpu", "gpu")
         self.dev = dev
 
+    def get_hash(self):
+        return "Transport"          # one closure serves both directions
+
     def typ_apply(self, input_types):
         return input_types[0]
+
+    def shp_apply(self, inputs):
+        return shape(inputs[0])
+
+    def get_native_compile_info(self, _input_types, _devtype):
+        # only ever placed between two different devices (there are no no-op transports)
+        code = r"""
+            CGT_EXPORT_C void $function(void* cldata, cgtObject** reads, cgtObject* write) {
+                cgt_copy_object(write, reads[0]);
+            }
+            """
+        return NativeCompileInfo(code)
 
     def get_py_func(self, input_types):
         def f(reads):
@@ -675,12 +870,15 @@ class Transport(Op):
             return v.get() if isinstance(v, GpuArray) else v
         return f
 
+    def __repr__(self):
+        return "Transport{%s}" % self.dev
+
     def pullback(self, inputs, _out, gout):
         return [Result(Transport(as_node(inputs[0]).devtype), [gout])]
 
 
 def reshape(x, shp):
-    return Result(Reshape(), [x] + [int(s) for s in shp])
+    return Result(Reshape(), [x] + list(shp))
 
 
 def transpose(x, axes):
@@ -902,7 +1100,7 @@ class Repeat(Op):
         for ax, rep in zip(self.axes, inputs[1:]):
             if out[ax] != 1:
                 raise ValueError("Repeat: axis %d has extent %d, not 1" % (ax, out[ax]))
-            out[ax] = int(np.asarray(as_node(rep).value))
+            out[ax] = scalar_extent(rep)
         return out
 
     def typ_apply(self, input_types):
@@ -1004,7 +1202,7 @@ class Fill(Op):
         raise MethodNotDefined("Fill is not differentiable")
 
     def shp_apply(self, inputs):
-        return [int(np.asarray(as_node(i).value)) for i in inputs]
+        return [scalar_extent(i) for i in inputs]
 
     def typ_apply(self, input_types):
         assert all(t.dtype == "i8" and t.ndim == 0 for t in input_types), \
@@ -1097,12 +1295,17 @@ def mean(x, axis=None, keepdims=False):
     n = 1
     for ax in axes:
         n *= size(x, ax)
-    return sum(x, axis=axes, keepdims=keepdims) / float(n)
+    divisor = constant(np.float32(n))
+    # the divisor's VALUE comes from extents: a function compiled from this graph serves
+    # other shapes only if those extents do not depend on its arguments
+    divisor.shape_baked = not ShapeInt._lift(n).is_constant()
+    divisor.baked_expr = ShapeInt._lift(n).expr
+    return sum(x, axis=axes, keepdims=keepdims) / divisor
 
 
 def fill(val, shp):
     """Array of shape `shp` filled with the scalar `val` (reference cgt/api.py:246-258)."""
-    return Result(Fill(val), [int(s) for s in shp])
+    return Result(Fill(val), list(shp))
 
 
 def zeros(shp):

@@ -44,7 +44,10 @@ void cgt_memcpy(cgtDevtype dest, cgtDevtype src, void* dest_ptr, void* src_ptr, 
         memcpy(dest_ptr, src_ptr, (size_t)nbytes);
         return;
     }
-    int rc = cgt_amd_memcpy((int)dest, (int)src, dest_ptr, src_ptr, nbytes);
+    // device to device: ordered on the stream the closures launch on, no host wait
+    int rc = (dest == cgtGPU && src == cgtGPU)
+                 ? cgt_amd_memcpy_async((int)dest, (int)src, dest_ptr, src_ptr, nbytes, cgt_get_stream())
+                 : cgt_amd_memcpy((int)dest, (int)src, dest_ptr, src_ptr, nbytes);
     cgt_check(rc == CGT_AMD_OK, "cgt_memcpy: %s", cgt_amd_last_error());
 }
 
@@ -114,7 +117,7 @@ struct MemLocation {
     cgtDevtype devtype;
 };
 
-enum InstrKind { LoadArgumentKind = 0, AllocKind, BuildTupKind, ReturnByRefKind, ReturnByValKind };
+enum InstrKind { LoadArgumentKind = 0, AllocKind, BuildTupKind, ReturnByRefKind, ReturnByValKind, ArgTransportKind };
 
 struct Instruction {
     InstrKind kind;
@@ -122,8 +125,13 @@ struct Instruction {
     MemLocation write;
     // LoadArgument
     int arg_index;
-    // Alloc: shape comes from the int64 host scalars in `reads`
+    // Alloc: shape comes from the int64 host scalars in `reads`.  `backing` is the largest
+    // buffer this instruction has allocated so far: a later run with a shape that fits it
+    // gets a view of it instead of a new allocation.
     cgtDtype dtype;
+    IRC<cgtObject> backing;   // owns the memory
+    IRC<cgtObject> current;   // what the last run put into the write slot: `backing` or a view of it
+    long backing_bytes;
     // ReturnByRef / ReturnByVal
     void* fptr;
     void* closure;
@@ -153,11 +161,26 @@ struct Interpreter {
                         return fail("Alloc: shape operands must be int64 host scalars");
                     shape[i] = sz->at<long>(0);
                 }
-                cgtArray* cur = static_cast<cgtArray*>(storage[in.write.index].get());
-                bool same = cur && cur->kind() == cgtObject::ArrayKind && cur->ndim() == ndim &&
-                            cur->dtype() == in.dtype && cur->devtype() == in.write.devtype;
-                for (int i = 0; same && i < ndim; ++i) same = cur->shape()[i] == shape[i];
-                if (!same) storage[in.write.index] = new cgtArray(ndim, shape.data(), in.dtype, in.write.devtype);
+                for (int i = 0; i < ndim; ++i)
+                    if (shape[i] < 0) return fail("Alloc: negative extent");
+                storage[in.write.index] = place(in, ndim, shape.data(), in.dtype);
+                return cgtGlobalStatus == cgtStatusOK;
+            }
+            case ArgTransportKind: {
+                // an argument on its way to the device its consumers run on: passed through
+                // untouched when it is already there, else copied (cgt_copy_object, the body
+                // of the reference's Transport op) into a buffer this instruction keeps
+                cgtObject* src = storage[in.reads[0].index].get();
+                if (!src || !cgt_is_array(src)) return fail("Transport: the argument is not an array");
+                cgtArray* a = static_cast<cgtArray*>(src);
+                if (a->devtype() == in.write.devtype) {
+                    storage[in.write.index] = src;
+                    return true;
+                }
+                cgtArray* dst = place(in, a->ndim(), a->shape(), a->dtype());
+                if (cgtGlobalStatus != cgtStatusOK) return false;
+                storage[in.write.index] = dst;
+                cgt_copy_object(dst, a);
                 return cgtGlobalStatus == cgtStatusOK;
             }
             case BuildTupKind: {
@@ -182,6 +205,30 @@ struct Interpreter {
             }
         }
         return fail("unknown instruction kind");
+    }
+
+    // The array an allocating instruction hands out for this run: the one of the last run
+    // while the shape is unchanged, a view of the instruction's buffer while the shape fits
+    // it, a new buffer otherwise (the old one is dropped; cgt_free waits for work that
+    // still uses it).
+    cgtArray* place(Instruction& in, int ndim, const long* shape, cgtDtype dtype) {
+        cgtArray* cur = static_cast<cgtArray*>(in.current.get());
+        bool same = cur && cur->ndim() == ndim && cur->dtype() == dtype;
+        for (int i = 0; same && i < ndim; ++i) same = cur->shape()[i] == shape[i];
+        if (same) return cur;
+        long need = cgt_itemsize(dtype);
+        for (int i = 0; i < ndim; ++i) need *= shape[i];
+        cgtArray* out;
+        if (in.backing && need <= in.backing_bytes) {
+            cgtArray* b = static_cast<cgtArray*>(in.backing.get());
+            out = new cgtArray(ndim, shape, dtype, in.write.devtype, b->data(), false);
+        } else {
+            out = new cgtArray(ndim, shape, dtype, in.write.devtype);
+            in.backing = out;
+            in.backing_bytes = need;
+        }
+        in.current = out;
+        return out;
     }
 
     bool fail(const char* msg) {
@@ -302,6 +349,12 @@ CGT_EXPORT int cgt_rt_interp_add_alloc(void* h, int dtype, const long* ridx, con
     return push(static_cast<Interpreter*>(h), in, ridx, rdev, nr, widx, wdev);
 }
 
+CGT_EXPORT int cgt_rt_interp_add_arg_transport(void* h, long ridx, int rdev, long widx, int wdev) {
+    Instruction in = Instruction();
+    in.kind = ArgTransportKind;
+    return push(static_cast<Interpreter*>(h), in, &ridx, &rdev, 1, widx, wdev);
+}
+
 CGT_EXPORT int cgt_rt_interp_add_build_tup(void* h, const long* ridx, const int* rdev, int nr, long widx, int wdev) {
     Instruction in = Instruction();
     in.kind = BuildTupKind;
@@ -322,6 +375,55 @@ CGT_EXPORT int cgt_rt_interp_add_return_byval(void* h, void* fptr, void* closure
     in.fptr = fptr;
     in.closure = closure;
     return push(static_cast<Interpreter*>(h), in, ridx, rdev, nr, widx, wdev);
+}
+
+// ---- shape arithmetic: by-value closures the interpreter fires through ReturnByVal, so that
+// Alloc and the ops' shape operands follow the shapes of the arguments at every run (the
+// reference computes them with its Size op and integer elementwise ops, cgt/core.py:1614-1640)
+
+struct cgt_rt_size_closure { int axis; };
+struct cgt_rt_intop_closure { int op; };
+
+static cgtArray* new_i8_scalar(long v) {
+    long shape1[1] = {1};
+    cgtArray* a = new cgtArray(0, shape1, cgt_i8, cgtCPU);
+    a->at<long>(0) = v;
+    return a;
+}
+
+// extent of axis `axis` of reads[0] as an int64 host scalar
+CGT_EXPORT cgtObject* cgt_rt_op_size(void* cl, cgtObject** reads) {
+    const int axis = static_cast<cgt_rt_size_closure*>(cl)->axis;
+    cgtArray* a = static_cast<cgtArray*>(reads[0]);
+    cgt_check(cgt_is_array(reads[0]) && axis >= 0 && axis < a->ndim(), "Size: axis %d of a %d-d array", axis, a->ndim());
+    if (cgtGlobalStatus != cgtStatusOK) return new_i8_scalar(0);
+    return new_i8_scalar(a->shape()[axis]);
+}
+
+// integer arithmetic on int64 host scalars: 0 add, 1 sub, 2 mul, 3 floor division,
+// 4 max(0, ceil(x / y)) (the pooling size rule), 5 negate (one operand)
+CGT_EXPORT cgtObject* cgt_rt_op_intop(void* cl, cgtObject** reads) {
+    const int op = static_cast<cgt_rt_intop_closure*>(cl)->op;
+    const long x = static_cast<cgtArray*>(reads[0])->at<long>(0);
+    const long y = op == 5 ? 1 : static_cast<cgtArray*>(reads[1])->at<long>(0);
+    long r = 0;
+    cgt_check(!((op == 3 || op == 4) && y == 0), "integer division by zero in a shape expression");
+    if (cgtGlobalStatus != cgtStatusOK) return new_i8_scalar(0);
+    switch (op) {
+        case 0: r = x + y; break;
+        case 1: r = x - y; break;
+        case 2: r = x * y; break;
+        case 3: r = x / y - ((x % y != 0) && ((x < 0) != (y < 0)) ? 1 : 0); break;   // floor, like python //
+        case 4: {
+            long f = x / y - ((x % y != 0) && ((x < 0) != (y < 0)) ? 1 : 0);
+            long c = f + (x % y != 0 ? 1 : 0);
+            r = c > 0 ? c : 0;
+            break;
+        }
+        case 5: r = -x; break;
+        default: cgt_check(false, "unknown integer op %d", op);
+    }
+    return new_i8_scalar(r);
 }
 
 // Pre-load a constant (e.g. a shape scalar or a parameter) into a slot.

@@ -137,6 +137,23 @@ CGT_API int cgt_amd_memcpy(int dest_devtype, int src_devtype, void* dest, const 
     return CGT_AMD_OK;
 }
 
+CGT_API int cgt_amd_memcpy_async(int dest_devtype, int src_devtype, void* dest, const void* src,
+                                 long nbytes, void* stream) {
+    CGT_ARG_CHECK(nbytes >= 0, "memcpy_async: negative size");
+    if (nbytes == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(dest && src, "memcpy_async: null pointer");
+    hipMemcpyKind kind;
+    if (src_devtype == CGT_AMD_CPU && dest_devtype == CGT_AMD_GPU) kind = hipMemcpyHostToDevice;
+    else if (src_devtype == CGT_AMD_GPU && dest_devtype == CGT_AMD_CPU) kind = hipMemcpyDeviceToHost;
+    else if (src_devtype == CGT_AMD_GPU && dest_devtype == CGT_AMD_GPU) kind = hipMemcpyDeviceToDevice;
+    else {
+        set_error("memcpy_async: invalid devtypes %d <- %d", dest_devtype, src_devtype);
+        return CGT_AMD_ERR_ARG;
+    }
+    CGT_HIP_TRY(hipMemcpyAsync(dest, src, (size_t)nbytes, kind, as_stream(stream)));
+    return CGT_AMD_OK;
+}
+
 CGT_API int cgt_amd_fill_u32(void* dst, unsigned int value, long count, void* stream) {
     CGT_ARG_CHECK(count >= 0, "fill: negative count");
     if (count == 0) return CGT_AMD_OK;

@@ -52,6 +52,7 @@ PROTOTYPES = {
     "cgt_rt_interp_free": (None, [c_void_p]),
     "cgt_rt_interp_add_load_argument": (c_int, [c_void_p, c_int, c_long, c_int]),
     "cgt_rt_interp_add_alloc": (c_int, [c_void_p, c_int, LONGP, INTP, c_int, c_long, c_int]),
+    "cgt_rt_interp_add_arg_transport": (c_int, [c_void_p, c_long, c_int, c_long, c_int]),
     "cgt_rt_interp_add_build_tup": (c_int, [c_void_p, LONGP, INTP, c_int, c_long, c_int]),
     "cgt_rt_interp_add_return_byref": (c_int, [c_void_p, c_void_p, c_void_p, LONGP, INTP, c_int, c_long, c_int]),
     "cgt_rt_interp_add_return_byval": (c_int, [c_void_p, c_void_p, c_void_p, LONGP, INTP, c_int, c_long, c_int]),
@@ -181,6 +182,9 @@ class Interpreter(object):
     def alloc(self, dtype, shape_locs, wloc):
         idx, dev, n = self._locs(shape_locs)
         return self._ok(self._L.cgt_rt_interp_add_alloc(self.handle, np.dtype(dtype).num, idx, dev, n, wloc[0], wloc[1]), "Alloc")
+
+    def arg_transport(self, rloc, wloc):
+        return self._ok(self._L.cgt_rt_interp_add_arg_transport(self.handle, rloc[0], rloc[1], wloc[0], wloc[1]), "ArgTransport")
 
     def build_tup(self, read_locs, wloc):
         idx, dev, n = self._locs(read_locs)

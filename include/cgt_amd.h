@@ -62,6 +62,14 @@ int cgt_amd_free(void *ptr);
  * branch of cgt_memcpy (src/cgt_common.cpp:138-153). */
 int cgt_amd_memcpy(int dest_devtype, int src_devtype, void *dest, const void *src, long nbytes);
 
+/* The same copy issued to `stream` without waiting for it: device-to-device
+ * copies are ordered with the kernels of that stream (the interpreter's
+ * Transport between two device buffers and the write-back of a parameter
+ * update use it); a copy that touches pageable host memory may still block the
+ * caller until the host side has been staged. */
+int cgt_amd_memcpy_async(int dest_devtype, int src_devtype, void *dest, const void *src, long nbytes,
+                         void *stream);
+
 /* Asynchronous fill of `count` 32-bit words with `value` (a fill kernel, safe
  * to capture in a HIP graph). */
 int cgt_amd_fill_u32(void *dst, unsigned int value, long count, void *stream);

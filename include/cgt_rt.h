@@ -55,12 +55,26 @@ int cgt_rt_copy_object(void *to, void *from);   /* host <-> device as needed */
 int cgt_rt_apply_byref(void *fptr, void *closure, void **reads, int n_reads, void *write);
 void *cgt_rt_apply_byval(void *fptr, void *closure, void **reads, int n_reads);
 
+/* by-value closures for shape arithmetic (fire them with ReturnByVal): the result is a
+ * new int64 host scalar.  cgt_rt_op_size: closure = { int axis }, reads[0] = any array.
+ * cgt_rt_op_intop: closure = { int op }, reads = int64 host scalars; op 0 add, 1 sub,
+ * 2 mul, 3 floor division, 4 max(0, ceil(x / y)), 5 negate. */
+void *cgt_rt_op_size(void *closure, void **reads);
+void *cgt_rt_op_intop(void *closure, void **reads);
+
 /* sequential interpreter over storage slots (LoadArgument / Alloc / BuildTup /
- * ReturnByRef / ReturnByVal); add_* return the instruction index or -1 */
+ * ReturnByRef / ReturnByVal, plus the argument transport below); add_* return the
+ * instruction index or -1.  Alloc reads its shape from int64 host scalars in slots at
+ * every run; it hands out the same array while the shape is unchanged and a view of its
+ * buffer while the shape fits it. */
 void *cgt_rt_interp_new(long n_slots);
 void cgt_rt_interp_free(void *interp);
 int cgt_rt_interp_add_load_argument(void *interp, int arg_index, long widx, int wdev);
 int cgt_rt_interp_add_alloc(void *interp, int dtype, const long *ridx, const int *rdev, int nr, long widx, int wdev);
+/* the array in slot ridx on its way to device wdev: the slot's object itself when it is
+ * already there (a device array handed in as an argument: no copy), else a copy
+ * (cgt_copy_object) in a buffer the instruction keeps and reuses */
+int cgt_rt_interp_add_arg_transport(void *interp, long ridx, int rdev, long widx, int wdev);
 int cgt_rt_interp_add_build_tup(void *interp, const long *ridx, const int *rdev, int nr, long widx, int wdev);
 int cgt_rt_interp_add_return_byref(void *interp, void *fptr, void *closure, const long *ridx, const int *rdev, int nr, long widx, int wdev);
 int cgt_rt_interp_add_return_byval(void *interp, void *fptr, void *closure, const long *ridx, const int *rdev, int nr, long widx, int wdev);

@@ -76,7 +76,7 @@ def test_function_device_outputs_reuse_buffers_and_check_shapes(cgt):
     assert (y2.ptr, p2.ptr) == ptrs
     assert np.allclose(y2.get(), 2 * y.get(), rtol=1e-5, atol=1e-5)
     with pytest.raises(ValueError):
-        f(x0[:1], fl)
+        f(x0[0], fl)                                    # wrong rank
     with pytest.raises(TypeError):
         f(x0)
     single = cgt.function([xn, fn], y)
@@ -150,6 +150,176 @@ def test_function_with_sgd_updates_trains_in_place(cgt):
     assert losses[-1] < losses[0]
     assert np.linalg.norm(layer.weight.get() - w64) <= 1e-4 * np.linalg.norm(w64)
     assert np.linalg.norm(layer.bias.get() - b64) <= 1e-4 * np.linalg.norm(b64)
+
+
+def test_function_is_shape_generic(cgt):
+    # compiled at batch 4, called at batch 7 and at batch 4 again: extents that depend on the
+    # argument are recomputed by Size / integer-op instructions, Alloc follows them
+    # (src/execution.cpp:251-264), and every output has the bits of a fresh evaluation
+    from cgt_amd import nn
+    rs = np.random.RandomState(5)
+    w = (rs.randn(16, 8, 3, 3) / 8).astype(np.float32)
+    b = (0.1 * rs.randn(1, 16, 1, 1)).astype(np.float32)
+    layer = nn.SpatialConvolution(8, 16, (3, 3), (1, 1), weight_init=w, bias_init=b)
+
+    def graph(xn):
+        act = nn.rectify(layer(xn))
+        act = nn.cross_channel_lrn(act, 5, 1e-3, 0.75)
+        pooled = nn.max_pool_2d(act, (3, 3), (0, 0), (2, 2))
+        loss = cgt.sum(pooled * pooled)
+        gx, gw, gb = cgt.grad(loss, [xn, layer.weight, layer.bias])
+        return [pooled, loss, gx, gw, gb]
+
+    x4 = rs.randn(4, 8, 17, 17).astype(np.float32)
+    xn = cgt.constant(x4)
+    f = cgt.function([xn], graph(xn), device_outputs=True)
+    assert f.shape_generic and f.n_shape_instructions > 0
+    ptrs = {}
+    for batch in (4, 7, 4, 4, 2):
+        xb = rs.randn(batch, 8, 17, 17).astype(np.float32)
+        got = f(xb)
+        want = graph(cgt.constant(xb))
+        for g, node in zip(got, want):
+            assert g.shape == node.shape
+            assert np.array_equal(g.get().view(np.uint32), node.get().view(np.uint32)), batch
+        ptrs.setdefault(batch, []).append([g.ptr for g in got])
+    # the buffers that grew for batch 7 serve the smaller batches after it: no new allocation
+    assert ptrs[4][1] == ptrs[7][0] and ptrs[4][2] == ptrs[7][0] and ptrs[2][0] == ptrs[7][0]
+    # spatial extents are symbolic too
+    xs = rs.randn(3, 8, 21, 13).astype(np.float32)
+    for g, node in zip(f(xs), graph(cgt.constant(xs))):
+        assert np.array_equal(g.get().view(np.uint32), node.get().view(np.uint32))
+
+
+def test_function_with_a_baked_extent_keeps_the_traced_shapes(cgt):
+    # mean() divides by a constant computed from the extents: such a function must refuse
+    # other shapes instead of dividing by the wrong count
+    x0 = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
+    xn = cgt.constant(x0)
+    f = cgt.function([xn], cgt.mean(xn * xn))
+    assert not f.shape_generic
+    assert abs(float(f(x0)) - (x0 * x0).mean()) <= 1e-4 * (x0 * x0).mean()
+    with pytest.raises(ValueError):
+        f(x0[:1])
+    # an extent of a weight (not an argument) is a constant: still generic in the argument
+    wn = cgt.constant(np.ones((3, 4), np.float32))
+    g = cgt.function([xn], cgt.sum(xn * 2.0) * cgt.mean(wn))
+    assert g.shape_generic
+    assert abs(float(g(x0[:1])) - 2 * x0[:1].sum()) <= 1e-3
+
+
+def test_function_transports_follow_the_gpu_deref_mask(cgt):
+    # conv2d + bias + grad built from HOST leaves: the placement rule (reference
+    # cgt/compilation.py:45-80, 285-304, with the gpu_deref_mask of core.py:748 honoured) puts
+    # one Transport in front of x and one in front of W; Col2Im's four int64 scalars, the
+    # Reshape operands and Repeat's counts are read in place on the host
+    from cgt_amd import core, nn, rt
+    rs = np.random.RandomState(6)
+    x0 = rs.randn(3, 4, 9, 9).astype(np.float32)
+    w0 = (rs.randn(6, 4, 3, 3) / 6).astype(np.float32)
+    b0 = (0.1 * rs.randn(1, 6, 1, 1)).astype(np.float32)
+
+    def graph(xn, wn, bn):
+        y = core.broadcast("+", nn.conv2d(xn, wn, (3, 3), (1, 1)), bn, "xxxx,1x11")
+        gy = cgt.constant(np.cos(np.arange(y.get().size, dtype=np.float32)).reshape(y.get().shape))
+        gx, gw, gb = cgt.grad(y, [xn, wn, bn], goutput=gy)
+        return [y, gx, gw, gb]
+
+    xh, wh = cgt.constant(x0, devtype="cpu"), cgt.constant(w0, devtype="cpu")
+    bn = cgt.constant(b0)
+    assert xh.devtype == "cpu" and wh.devtype == "cpu"
+    outs_h = graph(xh, wh, bn)
+    outs_d = graph(cgt.constant(x0), cgt.constant(w0), bn)
+    for a, b in zip(outs_h, outs_d):                     # node by node: same bits as the all-device graph
+        assert np.array_equal(a.get().view(np.uint32), b.get().view(np.uint32))
+    # the gradient of a host leaf comes back to the host (the pullback of a Transport is the
+    # reverse Transport); y and the bias gradient stay on the device
+    assert [o.devtype for o in outs_h] == ["gpu", "cpu", "cpu", "gpu"]
+    f = cgt.function([xh, wh], outs_h)
+    assert f.n_transports == 4 and f.n_arg_transports == 0
+    steps = f.plan_steps()
+    transports = [s for s in steps if s[0] == "byref" and s[4] == "transport"]
+    assert sorted((s[2][0][1], s[3][1]) for s in transports) == [(rt.CPU, rt.GPU)] * 2 + [(rt.GPU, rt.CPU)] * 2
+    seen = set()
+    for s in steps:
+        if s[0] != "byref" or s[4] != "op":
+            continue
+        name = s[1].op_str
+        devs = [loc[1] for loc in s[2]]
+        if name.startswith("Col2Im"):
+            assert devs == [rt.GPU] + [rt.CPU] * 4
+            seen.add("col2im")
+        elif name.startswith("Repeat"):
+            assert devs[0] == rt.GPU and all(d == rt.CPU for d in devs[1:])
+            seen.add("repeat")
+        else:
+            assert all(d == rt.GPU for d in devs), name
+    assert seen == {"col2im", "repeat"}
+    x1 = rs.randn(*x0.shape).astype(np.float32)
+    want = graph(cgt.constant(x1), cgt.constant(w0), bn)
+    for got, node in zip(f(x1, w0), want):
+        assert np.array_equal(got.view(np.uint32), node.get().view(np.uint32))
+    # an input that lives on the device may be handed over as a device array (no copy) or as a
+    # numpy array: LoadArgument + an argument transport inside the instruction list make the
+    # copy, not python, and both ways share the function's buffers
+    xd, wd = cgt.constant(x0), cgt.constant(w0)
+    fd = cgt.function([xd, wd], graph(xd, wd, bn), device_outputs=True)
+    assert fd.n_transports == 0 and fd.n_arg_transports == 2
+    got_h = fd(x1, w0)
+    ptrs = [g.ptr for g in got_h]
+    for got, node in zip(got_h, want):
+        assert np.array_equal(got.get().view(np.uint32), node.get().view(np.uint32))
+    x1_dev = cgt.to_gpu(x1 * 0.5)
+    got_d = fd(x1_dev, w0)
+    assert [g.ptr for g in got_d] == ptrs
+    want_half = graph(cgt.constant(x1 * 0.5), cgt.constant(w0), bn)
+    for got, node in zip(got_d, want_half):
+        assert np.array_equal(got.get().view(np.uint32), node.get().view(np.uint32))
+    assert np.array_equal(x1_dev.get(), x1 * 0.5)        # the caller's device array is only read
+    for got, node in zip(fd(x1, w0), want):               # host again: the staging buffer, not the caller's array
+        assert np.array_equal(got.get().view(np.uint32), node.get().view(np.uint32))
+    assert np.array_equal(x1_dev.get(), x1 * 0.5)
+
+
+def test_function_momentum_updates_read_the_new_value(cgt):
+    # v := 0.9 v - lr g ; p := p + v_new.  The second update reads the NEW velocity, and the
+    # function also returns an expression of the updated parameter: every reader of an update's
+    # right-hand side must see the new value, every reader of the parameter the old one
+    rs = np.random.RandomState(7)
+    x = rs.randn(5, 6).astype(np.float32)
+    p0 = rs.randn(6, 3).astype(np.float32)
+    v0 = (0.1 * rs.randn(6, 3)).astype(np.float32)
+    lr, mu = 0.05, 0.9
+    xn = cgt.constant(x)
+    p, v = cgt.constant(p0), cgt.constant(v0)
+    y = cgt.dot(xn, p)
+    loss = cgt.sum(y * y)
+    g, = cgt.grad(loss, [p])
+    v_new = v * mu - g * lr
+    p_new = p + v_new
+    probe = cgt.sum(p_new * p_new)               # an output computed from the updated parameter
+    step = cgt.function([xn], [loss, probe], updates=[(v, v_new), (p, p_new)])
+    pptr, vptr = p.value.ptr, v.value.ptr
+    p64, v64, x64 = p0.astype(np.float64), v0.astype(np.float64), x.astype(np.float64)
+    for _ in range(4):
+        got_loss, got_probe = step(x)
+        y64 = x64 @ p64
+        g64 = 2 * x64.T @ y64
+        v64 = mu * v64 - lr * g64
+        want_loss = (y64 * y64).sum()
+        p64 = p64 + v64
+        assert abs(float(got_loss) - want_loss) <= 1e-4 * want_loss
+        assert abs(float(got_probe) - (p64 * p64).sum()) <= 1e-4 * (p64 * p64).sum()
+        assert np.linalg.norm(p.get() - p64) <= 1e-4 * np.linalg.norm(p64)
+        assert np.linalg.norm(v.get() - v64) <= 1e-4 * np.linalg.norm(v64)
+    assert (p.value.ptr, v.value.ptr) == (pptr, vptr)
+    kinds = [s[4] for s in step.plan_steps() if s[0] == "byref"]
+    assert kinds[-1] == "update-copy" or kinds[-2] == "update-copy"
+    # two parameters whose updates read each other's OLD value
+    a, b = cgt.constant(np.float32([[1.0, 2.0]])), cgt.constant(np.float32([[10.0, 20.0]]))
+    swap = cgt.function([], [], updates=[(a, b * 1.0), (b, a * 1.0)])
+    swap()
+    assert np.array_equal(a.get(), [[10.0, 20.0]]) and np.array_equal(b.get(), [[1.0, 2.0]])
 
 
 def test_function_as_hip_graph_matches_eager_on_every_replay(cgt):

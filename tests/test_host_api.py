@@ -220,6 +220,53 @@ def test_interpreter_alloc_reuse_and_byref():
         it.alloc(np.int64, [], (99, cpu))
 
 
+def test_shape_int_keeps_its_expression():
+    from cgt_amd.core import ShapeInt, ceil_divide, shape_depends_on
+    leaf = object()
+    H = ShapeInt(28, ("size", leaf, 2))
+    m = (H + 2 * 1 - 3) // 1 + 1
+    assert m == 28 and isinstance(m, ShapeInt) and shape_depends_on(m.expr) == [leaf]
+    p = ceil_divide(m + 2 * 0 - 2, 2)
+    assert p == 13 and p.expr[0] == "ceildiv"
+    assert (ShapeInt(3) * 4).is_constant() and (3 * H).expr == ("*", ("const", 3), ("size", leaf, 2))
+    assert (-H).expr == ("neg", ("size", leaf, 2)) and (10 - H) == -18 and (H - 10).expr[0] == "-"
+    assert int(H) + 1 == 29 and type(int(H)) is int and [0] * ShapeInt(2) == [0, 0]
+    from cgt_amd.function import _eval_expr
+    assert _eval_expr(("ceildiv", ("const", -3), ("const", 2))) == 0
+    assert _eval_expr(("//", ("const", -3), ("const", 2))) == -2
+
+
+def test_interpreter_shape_instructions_and_alloc_capacity():
+    # Size / integer-op closures of the runtime computing an Alloc's shape from the argument
+    # at every run; a buffer that has grown serves the smaller shapes after it
+    from cgt_amd.function import _IntOpClosure, _RtCallable, _SizeClosure
+    it = rt.Interpreter(8)
+    cpu = rt.CPU
+    it.load_argument(0, (0, cpu))
+    it.set_slot(1, 3)
+    it.set_slot(2, 2)
+    it.return_byval(_RtCallable("cgt_rt_op_size", _SizeClosure(0)), [(0, cpu)], (3, cpu))
+    it.return_byval(_RtCallable("cgt_rt_op_intop", _IntOpClosure(2)), [(3, cpu), (1, cpu)], (4, cpu))     # 3 * n
+    it.return_byval(_RtCallable("cgt_rt_op_intop", _IntOpClosure(4)), [(3, cpu), (2, cpu)], (5, cpu))     # ceil(n / 2)
+    it.return_byval(_RtCallable("cgt_rt_op_intop", _IntOpClosure(3)), [(3, cpu), (2, cpu)], (6, cpu))     # n // 2
+    it.alloc(np.float32, [(4, cpu), (5, cpu)], (7, cpu))
+    L = rt.lib()
+
+    def run(n):
+        it.run([np.zeros((n, 2), np.int64)])
+        h = L.cgt_rt_interp_get_slot(it.handle, 7)
+        shp = L.cgt_rt_array_shape(h)
+        return (shp[0], shp[1]), L.cgt_rt_array_data(h), int(it.get_array(6))
+    s5, p5, f5 = run(5)
+    assert s5 == (15, 3) and f5 == 2
+    s5b, p5b, _ = run(5)
+    assert p5b == p5
+    s9, p9, f9 = run(9)
+    assert s9 == (27, 5) and f9 == 4
+    s4, p4, _ = run(4)
+    assert s4 == (12, 2) and p4 == p9, "a shape that fits the grown buffer must not allocate"
+
+
 # ---------------------------------------------------------------- conv-layer glue ops (host logic only)
 
 def test_elwise_binary_type_rules():

@@ -25,7 +25,7 @@ CXX = os.environ.get("CXX", "g++")
 CPP_FLAGS = ["-fvisibility=hidden", "-std=c++11", "-fPIC", "-O3", "-DNDEBUG"]
 INCLUDE = os.path.join(ROOT, "include")
 
-SOURCES = ["runtime.hip", "im2col.hip", "pool.hip", "lrn.hip", "gemm.hip", "glue.hip", "elwise.hip"]
+SOURCES = ["runtime.hip", "im2col.hip", "pool.hip", "lrn.hip", "gemm.hip", "glue.hip", "elwise.hip", "conv.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"

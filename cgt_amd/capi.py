@@ -43,6 +43,7 @@ PROTOTYPES = {
     "cgt_amd_im2col_f32": (c_int, [c_void_p] + [c_long] * 4 + [c_int] * 6 + [c_void_p, c_void_p]),
     "cgt_amd_col2im_f32": (c_int, [c_void_p] + [c_long] * 4 + [c_int] * 6 + [c_void_p, c_void_p]),
     "cgt_amd_pool_outsize": (c_long, [c_long, c_int, c_int, c_int]),
+    "cgt_amd_pool_staged_planes": (c_int, [c_int, c_long, c_long, c_long, c_long]),
     "cgt_amd_max_pool_f32": (c_int, [c_void_p] + [c_long] * 4 + [c_int] * 6 + [c_long] * 2
                              + [c_void_p, c_void_p, c_void_p]),
     "cgt_amd_max_pool_pullback_f32": (c_int, [c_void_p, c_void_p] + [c_long] * 4 + [c_int] * 6
@@ -58,6 +59,12 @@ PROTOTYPES = {
     "cgt_amd_sgemm_batched": (c_int, [c_int, c_int, c_long, c_long, c_long, c_long,
                                       c_void_p, c_long, c_long, c_void_p, c_long, c_long,
                                       c_void_p, c_long, c_long, c_void_p]),
+    "cgt_amd_conv_same_supported": (c_int, [c_long, c_long] + [c_int] * 6),
+    "cgt_amd_conv_same_padded_size": (c_long, [c_long, c_long, c_long, c_int, c_int]),
+    "cgt_amd_conv_same_pad_f32": (c_int, [c_void_p, c_long, c_long, c_long, c_int, c_int, c_void_p, c_void_p]),
+    "cgt_amd_conv_same_fwd_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int] + [c_long] * 5 + [c_int, c_int, c_void_p, c_void_p]),
+    "cgt_amd_conv_same_bwd_data_f32": (c_int, [c_void_p, c_void_p] + [c_long] * 5 + [c_int, c_int, c_void_p, c_void_p]),
+    "cgt_amd_conv_same_bwd_filter_f32": (c_int, [c_void_p, c_void_p] + [c_long] * 5 + [c_int, c_int, c_void_p, c_void_p]),
     "cgt_amd_elwise_unary_f32": (c_int, [c_int, c_long, c_void_p, c_void_p, c_void_p]),
     "cgt_amd_elwise_binary": (c_int, [c_int, c_int, c_int, c_long, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p]),
     "cgt_amd_repeat": (c_int, [c_void_p, c_int, c_int, ctypes.POINTER(c_long), ctypes.POINTER(c_int), c_void_p, c_void_p]),

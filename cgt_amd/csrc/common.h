@@ -21,9 +21,24 @@ inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 // stream -- it is retired and released with the stream (cgt_amd_stream_destroy).
 // Growth while the stream is being captured is refused (an allocation would break the
 // capture): returns nullptr with the message set.
-enum WorkspaceUser { kWsGemm = 0, kWsSum = 1, kWsUsers = 2 };
+enum WorkspaceUser { kWsGemm = 0, kWsSum = 1, kWsConvRows = 2, kWsConvFilter = 3, kWsUsers = 4 };
 float* stream_workspace(void* stream, WorkspaceUser user, size_t bytes, const char* what);
 void release_stream_workspaces(void* stream);
+
+// GEMM over an operand read straight from a zero-padded image (gemm.hip): the products of
+// a stride-1 convolution with pad = (kernel - 1) / 2, without a column buffer.
+//   mode 1: rows[B * tpi * 128][N] = sum over (tap, c) of img[b][c][q + tapoff] * Wk[n][tap*C + c]
+//           (q = row within the image's tpi * 128 rows of the padded grid)
+//   mode 2: out[M][taps * C] = sum over (b, q) of A[b][m][q] * img[b][c][q + tapoff]
+struct ConvGemm {
+    int mode;
+    long B, C, plane;      // images, channels of `img`, floats per padded plane
+    int wp, kh, kw;        // padded width, kernel
+    long tpi, spi;         // mode 1: row tiles (of 128) per image; mode 2: K slices (of 16) per image
+};
+int sgemm_conv(const ConvGemm& cv, long M, long N, const float* A, const float* B, float* C, long ldc, void* stream);
+// 1 if sgemm_conv has a tile shape for these extents (mode 1: N filters; mode 2: M filters, C channels)
+bool sgemm_conv_supported(int mode, long filters, long channels);
 
 constexpr int kWave = 64;    // CDNA wavefront width
 constexpr int kNumXCD = 8;   // MI355X: 8 accelerator dies, each with its own L2

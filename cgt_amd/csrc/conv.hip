@@ -1,0 +1,263 @@
+// Stride-1 "same" convolution (pad = (kernel - 1) / 2, odd kernels) without a column
+// buffer: forward, data gradient and weight gradient as GEMMs whose image operand is read
+// straight from a zero-padded copy of the image (sgemm_conv in gemm.hip).
+//
+// Padded layout: [B * C planes][plane floats] + a zeroed tail, plane = (H + 2p)(W + 2q)
+// rounded up past 16 zero floats; pixel (h, w) of a plane sits at (h + p) * Wp + (w + q).
+// A row of the forward GEMM is a pixel of the padded grid, q = h * Wp + w (the Wp - W
+// positions at the end of each grid row are junk rows that nobody reads back), so that
+// "tap (ho, wo) of pixel q" is the plain offset q + ho * Wp + wo: every operand tile is a
+// contiguous run per channel, loaded straight into LDS like any GEMM tile.
+//
+//   forward        rows[b][q][l]   = sum_{tap,c} xpad[b][c][q + tapoff] * f[l][c][tap]
+//   data gradient  rows[b][q][c]   = sum_{tap,l} gypad[b][l][q + tapoff] * f[l][c][flipped tap]
+//   weight grad    gf[l][tap][c]   = sum_{b,q}   gypad[b][l][q + center] * xpad[b][c][q + tapoff]
+// (the padding columns of gypad are zero, so the junk positions of q contribute nothing).
+#include "common.h"
+#include <algorithm>
+
+namespace cgt_amd {
+
+struct SameGeom {
+    long B, C, H, W, L;
+    int kh, kw, ph, pw;
+    long Hp, Wp, plane, tail;
+    long tpi;      // 128-row tiles per image in the forward / data-gradient GEMM
+    long spi;      // 16-pixel K slices per image in the weight-gradient GEMM
+    long total(long planes) const { return planes * plane + tail; }
+};
+
+static bool make_geom(SameGeom& g, long B, long C, long H, long W, long L, int kh, int kw) {
+    if (kh < 1 || kw < 1 || kh % 2 == 0 || kw % 2 == 0) return false;
+    g.B = B; g.C = C; g.H = H; g.W = W; g.L = L;
+    g.kh = kh; g.kw = kw; g.ph = (kh - 1) / 2; g.pw = (kw - 1) / 2;
+    g.Hp = H + 2 * g.ph; g.Wp = W + 2 * g.pw;
+    g.plane = (g.Hp * g.Wp + 16 + 15) / 16 * 16;
+    g.tail = (256 + (long)kh * g.Wp + 3) / 4 * 4;
+    g.tpi = cdiv(H * g.Wp, 128);
+    g.spi = cdiv(H * g.Wp, 16);
+    return true;
+}
+
+// dst plane: zero everywhere except the H x W interior.  A thread writes 4 consecutive
+// floats of a plane (plane % 4 == 0: one aligned 16-byte store) and gathers them from the
+// source rows; both sides are contiguous runs per image row.
+__global__ __launch_bounds__(256) void pad_planes_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                         long planes, int H, int W, int Wp, int ph, int pw,
+                                                         int plane, int units_per_plane, long total_units,
+                                                         long tail_units) {
+    const float rWp = 1.0f / (float)Wp;
+    for (long u = (long)blockIdx.x * 256 + threadIdx.x; u < total_units + tail_units; u += (long)gridDim.x * 256) {
+        float o[4] = {0.f, 0.f, 0.f, 0.f};
+        if (u < total_units) {
+            const long pl = u / units_per_plane;
+            const int e0 = (int)(u - pl * units_per_plane) * 4;
+            const float* sp = src + pl * (long)H * W;
+            // row of e0 by reciprocal multiplication (plane < 2^21 is checked on the host), fixed up exactly
+            int hp = (int)(((float)e0 + 0.5f) * rWp);
+            int wp = e0 - hp * Wp;
+            if (wp < 0) { --hp; wp += Wp; }
+            if (wp >= Wp) { ++hp; wp -= Wp; }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int h = hp - ph, w = wp - pw;
+                if (h >= 0 && h < H && w >= 0 && w < W) o[j] = sp[h * W + w];
+                if (++wp == Wp) { wp = 0; ++hp; }
+            }
+        }
+        stream_store4(dst + u * 4, o[0], o[1], o[2], o[3]);
+    }
+}
+
+// rows [B][rows_per_image][L] (row q = h * Wp + w) -> out [B][L][H][W] (+ optional
+// per-channel bias and ReLU, applied as x * (x >= 0)).  A workgroup takes 64 consecutive
+// output positions of one image and all L channels: the rows it needs are one contiguous
+// block of the input (64 positions + the junk rows between them), copied to LDS with
+// 16-byte loads; each channel then leaves as a run of 64 floats.
+constexpr int kR2NPos = 64;
+__global__ __launch_bounds__(256) void rows_to_nchw_kernel(const float* __restrict__ rows, float* __restrict__ out,
+                                                           const float* __restrict__ bias, int relu,
+                                                           int HW, int W, int Wp, int L, long rows_per_image,
+                                                           int tiles, int npos) {
+    extern __shared__ float tile[];          // [max_rows][L | 1]
+    const int LD = L | 1;
+    const int bid = blockIdx.x;
+    const int b = bid / tiles, t = bid - b * tiles;
+    const int p0 = t * npos;
+    const int np = min(npos, HW - p0);
+    const int h0 = p0 / W, w0 = p0 - h0 * W;
+    const int q0 = h0 * Wp + w0;
+    const int pl = p0 + np - 1, hl = pl / W;
+    const int q1 = hl * Wp + (pl - hl * W);          // last row needed
+    const int nrows = q1 - q0 + 1;                   // <= max_rows
+    const float* blk = rows + ((long)b * rows_per_image + q0) * L;
+    const int n = nrows * L;                          // L % 4 == 0
+    const float rL = 1.0f / (float)L;
+    for (int i0 = threadIdx.x * 4; i0 < n; i0 += 1024 * 4) {
+        v4f v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const v4f*>(blk + min(i0 + u * 1024, n - 4));
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int i = i0 + u * 1024;
+            if (i < n) {
+                int r = (int)((float)i * rL);
+                int c = i - r * L;
+                if (c < 0) { --r; c += L; }
+                if (c >= L) { ++r; c -= L; }
+                float* d = tile + r * LD + c;
+                d[0] = v[u].x; d[1] = v[u].y; d[2] = v[u].z; d[3] = v[u].w;
+            }
+        }
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane < np) {
+        const int p = p0 + lane, h = p / W, w = p - h * W;
+        const int r = h * Wp + w - q0;
+        float* dst = out + (long)b * L * HW + p;
+        for (int c = wave; c < L; c += 4) {
+            float v = tile[r * LD + c];
+            if (bias) v += bias[c];
+            if (relu) v = v * (v >= 0.0f ? 1.0f : 0.0f);
+            dst[(long)c * HW] = v;
+        }
+    }
+}
+
+// filters [L][C][kh][kw] -> [C][(kh-1-ho, kw-1-wo) taps][L]: the filter bank of the data
+// gradient seen as a forward convolution of the cotangent
+__global__ __launch_bounds__(256) void flip_filters_kernel(const float* __restrict__ f, float* __restrict__ out,
+                                                           int L, int C, int kh, int kw) {
+    const int taps = kh * kw;
+    const long total = (long)L * C * taps;
+    for (long o = (long)blockIdx.x * 256 + threadIdx.x; o < total; o += (long)gridDim.x * 256) {
+        const int l = (int)(o % L);
+        const long r = o / L;
+        const int tap = (int)(r % taps), c = (int)(r / taps);
+        const int ho = tap / kw, wo = tap - ho * kw;
+        out[o] = f[(((long)l * C + c) * kh + (kh - 1 - ho)) * kw + (kw - 1 - wo)];
+    }
+}
+
+static int rows_to_nchw(const SameGeom& g, const float* rows, long Lout, const float* bias, int relu, float* out,
+                        hipStream_t st) {
+    const long HW = g.H * g.W;
+    // positions per workgroup: 64, fewer for narrow images whose junk rows would not fit LDS
+    int npos = kR2NPos;
+    auto rows_needed = [&](int n) { return std::min((long)n + (n / g.W + 2) * (g.Wp - g.W), g.H * g.Wp); };
+    while (npos > 1 && rows_needed(npos) * (Lout | 1) * (long)sizeof(float) > 48 * 1024) npos /= 2;
+    const size_t lds = (size_t)rows_needed(npos) * (Lout | 1) * sizeof(float);
+    const long tiles = cdiv(HW, (long)npos);
+    CGT_ARG_CHECK(lds <= 64 * 1024 && g.B * tiles < (1L << 31), "conv_same: output tile does not fit LDS");
+    rows_to_nchw_kernel<<<dim3((unsigned)(g.B * tiles)), dim3(256), lds, st>>>(
+        rows, out, bias, relu, (int)HW, (int)g.W, (int)g.Wp, (int)Lout, g.tpi * 128, (int)tiles, npos);
+    CGT_LAUNCH_CHECK("rows_to_nchw_kernel");
+    return CGT_AMD_OK;
+}
+
+static int check_same(const char* what, SameGeom& g, long B, long C, long H, long W, long L, int kh, int kw) {
+    CGT_ARG_CHECK(B >= 0 && C > 0 && H > 0 && W > 0 && L > 0, "%s: bad shape", what);
+    CGT_ARG_CHECK(make_geom(g, B, C, H, W, L, kh, kw), "%s: the kernel must be odd x odd (pad = (kernel - 1) / 2)", what);
+    CGT_ARG_CHECK(g.plane < (1L << 21), "%s: image plane too large for this path", what);
+    return CGT_AMD_OK;
+}
+
+}  // namespace cgt_amd
+
+using namespace cgt_amd;
+
+CGT_API int cgt_amd_conv_same_supported(long C, long L, int kh, int kw, int ph, int pw, int sh, int sw) {
+    if (sh != 1 || sw != 1 || kh % 2 == 0 || kw % 2 == 0 || ph != (kh - 1) / 2 || pw != (kw - 1) / 2) return 0;
+    if (L > 128 || L % 4 != 0 || C > 128 || C % 4 != 0) return 0;   // rows -> NCHW keeps all channels of 64 pixels in LDS
+    // forward: C channels in, L filters; data gradient: L channels in, C "filters"; weight gradient: both
+    return sgemm_conv_supported(1, L, C) && sgemm_conv_supported(1, C, L) && sgemm_conv_supported(2, L, C) ? 1 : 0;
+}
+
+CGT_API long cgt_amd_conv_same_padded_size(long planes, long H, long W, int kh, int kw) {
+    SameGeom g;
+    if (planes < 0 || H <= 0 || W <= 0 || !make_geom(g, 1, 1, H, W, 1, kh, kw)) return -1;
+    return g.total(planes);
+}
+
+CGT_API int cgt_amd_conv_same_pad_f32(const float* x, long planes, long H, long W, int kh, int kw, float* xpad,
+                                      void* stream) {
+    SameGeom g;
+    int rc = check_same("conv_same_pad", g, 1, 1, H, W, 1, kh, kw);
+    if (rc) return rc;
+    CGT_ARG_CHECK(planes >= 0 && (x || planes == 0) && xpad, "conv_same_pad: null pointer");
+    CGT_ARG_CHECK(reinterpret_cast<uintptr_t>(xpad) % 16 == 0, "conv_same_pad: the padded buffer must be 16-byte aligned");
+    const long upp = g.plane / 4, units = planes * upp, tail_units = g.tail / 4;
+    const long blocks = std::min(cdiv(units + tail_units, 256L), 1L << 16);
+    pad_planes_kernel<<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(
+        x, xpad, planes, (int)H, (int)W, (int)g.Wp, g.ph, g.pw, (int)g.plane, (int)upp, units, tail_units);
+    CGT_LAUNCH_CHECK("pad_planes_kernel");
+    return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_conv_same_fwd_f32(const float* xpad, const float* f, const float* bias, int relu, long B, long C,
+                                      long H, long W, long L, int kh, int kw, float* y, void* stream) {
+    SameGeom g;
+    int rc = check_same("conv_same_fwd", g, B, C, H, W, L, kh, kw);
+    if (rc) return rc;
+    if (B == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(xpad && f && y, "conv_same_fwd: null pointer");
+    CGT_ARG_CHECK(cgt_amd_conv_same_supported(C, L, kh, kw, g.ph, g.pw, 1, 1), "conv_same_fwd: unsupported extents C=%ld L=%ld", C, L);
+    const long taps = (long)kh * kw;
+    float* wk = stream_workspace(stream, kWsConvFilter, (size_t)L * C * taps * sizeof(float), "conv_same_fwd");
+    float* rows = stream_workspace(stream, kWsConvRows, (size_t)B * g.tpi * 128 * std::max(L, C) * sizeof(float), "conv_same_fwd");
+    if (!wk || !rows) return CGT_AMD_ERR_NOMEM;
+    // filters [L][C][kh][kw] -> [L][tap][C]: the K axis of the product is (tap, channel)
+    const long fs[4] = {L, C, kh, kw};
+    const int ax[4] = {0, 2, 3, 1};
+    rc = cgt_amd_transpose4_f32(f, fs, ax, wk, stream);
+    if (rc) return rc;
+    ConvGemm cv = {1, B, C, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi};
+    rc = sgemm_conv(cv, B * g.tpi * 128, L, xpad, wk, rows, L, stream);
+    if (rc) return rc;
+    return rows_to_nchw(g, rows, L, bias, relu, y, as_stream(stream));
+}
+
+CGT_API int cgt_amd_conv_same_bwd_data_f32(const float* gypad, const float* f, long B, long C, long H, long W, long L,
+                                           int kh, int kw, float* gx, void* stream) {
+    SameGeom g;
+    int rc = check_same("conv_same_bwd_data", g, B, C, H, W, L, kh, kw);
+    if (rc) return rc;
+    if (B == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(gypad && f && gx, "conv_same_bwd_data: null pointer");
+    CGT_ARG_CHECK(cgt_amd_conv_same_supported(C, L, kh, kw, g.ph, g.pw, 1, 1), "conv_same_bwd_data: unsupported extents C=%ld L=%ld", C, L);
+    const long taps = (long)kh * kw;
+    float* wk = stream_workspace(stream, kWsConvFilter, (size_t)L * C * taps * sizeof(float), "conv_same_bwd_data");
+    float* rows = stream_workspace(stream, kWsConvRows, (size_t)B * g.tpi * 128 * std::max(L, C) * sizeof(float), "conv_same_bwd_data");
+    if (!wk || !rows) return CGT_AMD_ERR_NOMEM;
+    flip_filters_kernel<<<dim3((unsigned)std::min(cdiv(L * C * taps, 256L), 4096L)), dim3(256), 0, as_stream(stream)>>>(
+        f, wk, (int)L, (int)C, kh, kw);
+    CGT_LAUNCH_CHECK("flip_filters_kernel");
+    // a forward convolution of the cotangent: L channels in, C "filters" [C][tap][L]
+    ConvGemm cv = {1, B, L, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi};
+    rc = sgemm_conv(cv, B * g.tpi * 128, C, gypad, wk, rows, C, stream);
+    if (rc) return rc;
+    return rows_to_nchw(g, rows, C, nullptr, 0, gx, as_stream(stream));
+}
+
+CGT_API int cgt_amd_conv_same_bwd_filter_f32(const float* gypad, const float* xpad, long B, long C, long H, long W,
+                                             long L, int kh, int kw, float* gf, void* stream) {
+    SameGeom g;
+    int rc = check_same("conv_same_bwd_filter", g, B, C, H, W, L, kh, kw);
+    if (rc) return rc;
+    CGT_ARG_CHECK(gf, "conv_same_bwd_filter: null pointer");
+    const long taps = (long)kh * kw;
+    if (B == 0) return cgt_amd_fill_u32(gf, 0u, L * C * taps, stream);
+    CGT_ARG_CHECK(gypad && xpad, "conv_same_bwd_filter: null pointer");
+    CGT_ARG_CHECK(cgt_amd_conv_same_supported(C, L, kh, kw, g.ph, g.pw, 1, 1), "conv_same_bwd_filter: unsupported extents C=%ld L=%ld", C, L);
+    float* wk = stream_workspace(stream, kWsConvFilter, (size_t)L * C * taps * sizeof(float), "conv_same_bwd_filter");
+    if (!wk) return CGT_AMD_ERR_NOMEM;
+    // pixel q of the padded grid <-> cotangent at q + (ph * Wp + pw): its padding is zero, so junk pixels add nothing
+    ConvGemm cv = {2, B, C, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi};
+    rc = sgemm_conv(cv, L, taps * C, gypad + g.ph * g.Wp + g.pw, xpad, wk, taps * C, stream);
+    if (rc) return rc;
+    // [L][tap][C] -> [L][C][kh][kw]
+    const long ws[4] = {L, kh, kw, C};
+    const int ax[4] = {0, 3, 1, 2};
+    return cgt_amd_transpose4_f32(wk, ws, ax, gf, stream);
+}

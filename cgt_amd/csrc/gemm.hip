@@ -98,6 +98,16 @@ struct GemmArgs {
     // [piece][BM][BN]; tail_reduce_kernel adds them up in order.
     int main_wgs, tail_splits, tail_kchunk;
     int wide;          // a leading dimension too large for 32-bit tile offsets: tested loads everywhere
+    // Implicit convolution (stride 1, pad = (kernel-1)/2): an operand is read straight
+    // from the zero-padded image [B][C][plane] instead of a column buffer.  The K axis
+    // is ordered (tap, channel), so a slice of 16 is one tap and 16 consecutive channels.
+    //   mode 1 (forward / data gradient): A[row][k] = img[b][c][q + tapoff], rows are the
+    //     pixels q = h*Wp + w of the padded grid, cv_tpi tiles of rows per image;
+    //   mode 2 (weight gradient): the K axis runs over those pixels, cv_spi slices per
+    //     image; A[l][q] and B[tap*C + c][q] are both q-contiguous.
+    int conv;
+    int cv_wp, cv_kw, cv_cpb, cv_tpi, cv_spi, cv_c;   // padded width, kernel width, C/16, tiles / slices per image, C
+    long cv_plane, cv_imgA, cv_imgB;                  // plane stride and per-image strides (floats)
 };
 
 // One ROWS x KT operand tile, moved with 16-byte accesses.
@@ -239,9 +249,11 @@ __device__ __forceinline__ int xcd_remap(int id, int n) {
 // WGM x WGN wavefronts, each TM x TN blocks of 32x32.
 // PIPE selects the software-pipelined main loop (k-contiguous operands only).
 // DEEP (plain loop only) keeps two K slices of global loads in flight instead of one.
-template <bool AKC, bool BKC, bool PIPE, int WGM, int WGN, int TM, int TN, bool DEEP = false>
+template <bool AKC, bool BKC, bool PIPE, int WGM, int WGN, int TM, int TN, bool DEEP = false, int CONV = 0>
 __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmArgs a) {
     static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
+    static_assert(CONV == 0 || (!PIPE && !DEEP && BKC && AKC == (CONV == 2)),
+                  "implicit convolution: plain loop; mode 1 reads A row-contiguous, mode 2 k-contiguous");
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
     typedef OperandTile<AKC, BM> TileA;
     typedef OperandTile<BKC, BN> TileB;
@@ -349,11 +361,63 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
     // whole (an edge tile in N still streams A untested) and the tested ones
     // otherwise; a ragged last K slice is tested for both.
     constexpr int kFast = 0, kMixed = 1;
-    const bool wholeA = m0 + BM <= a.M && !a.wide, wholeB = n0 + BN <= a.N && !a.wide;
-    const bool ragged_k = (kend - kbeg) % KT != 0;
+    const bool wholeA = CONV != 0 || (m0 + BM <= a.M && !a.wide), wholeB = CONV != 0 || (n0 + BN <= a.N && !a.wide);
+    const bool ragged_k = CONV == 0 && (kend - kbeg) % KT != 0;
     const char* originA = reinterpret_cast<const char*>(A + (AKC ? (long)m0 * a.lda + kbeg : (long)kbeg * a.lda + m0));
     const char* originB = reinterpret_cast<const char*>(B + (BKC ? (long)n0 * a.ldb + kbeg : (long)kbeg * a.ldb + n0));
     const long stepA = (AKC ? (long)KT : (long)KT * a.lda) * 4, stepB = (BKC ? (long)KT : (long)KT * a.ldb) * 4;
+    // Implicit convolution: where the slices of the image operand(s) start.  Slices are
+    // issued in ascending order, one call of conv_next() each, so the walk is a handful
+    // of scalar adds and compares per slice (everything here is wave-uniform).
+    const char* cvA = nullptr;
+    const char* cvB = nullptr;
+    int cv_i = 0, cv_j = 0;        // mode 1: channel block, kernel column; mode 2: slice within the image
+    if constexpr (CONV == 1) {
+        const int s0 = kbeg / KT;
+        const int tap = s0 / a.cv_cpb;
+        cv_i = s0 - tap * a.cv_cpb;
+        const int ho = tap / a.cv_kw;
+        cv_j = tap - ho * a.cv_kw;
+        const int img = tm / a.cv_tpi, t = tm - img * a.cv_tpi;
+        cvA = reinterpret_cast<const char*>(A + (long)img * a.cv_imgA + (long)t * BM + (long)ho * a.cv_wp + cv_j +
+                                            (long)cv_i * KT * a.cv_plane);
+    } else if constexpr (CONV == 2) {
+        const int s0 = kbeg / KT;
+        const int img = s0 / a.cv_spi;
+        cv_i = s0 - img * a.cv_spi;
+        const int tap = n0 / a.cv_c, c0 = n0 - tap * a.cv_c;
+        const int ho = tap / a.cv_kw, wo = tap - ho * a.cv_kw;
+        cvA = reinterpret_cast<const char*>(A + (long)img * a.cv_imgA + (long)m0 * a.cv_plane + (long)cv_i * KT);
+        cvB = reinterpret_cast<const char*>(B + (long)img * a.cv_imgB + (long)c0 * a.cv_plane + (long)ho * a.cv_wp + wo +
+                                            (long)cv_i * KT);
+    }
+    // origins of the next slice to be issued, then step to the one after it
+    auto conv_next = [&](const char*& oa, const char*& ob) {
+        if constexpr (CONV == 1) {
+            oa = cvA;
+            ob = originB;
+            originB += stepB;
+            cvA += (long)KT * a.cv_plane * 4;
+            if (++cv_i == a.cv_cpb) {             // next tap: back to channel 0, one pixel to the right
+                cv_i = 0;
+                cvA += 4 - (long)a.cv_cpb * KT * a.cv_plane * 4;
+                if (++cv_j == a.cv_kw) {          // next kernel row
+                    cv_j = 0;
+                    cvA += (long)(a.cv_wp - a.cv_kw) * 4;
+                }
+            }
+        } else if constexpr (CONV == 2) {
+            oa = cvA;
+            ob = cvB;
+            cvA += KT * 4;
+            cvB += KT * 4;
+            if (++cv_i == a.cv_spi) {             // next image
+                cv_i = 0;
+                cvA += (a.cv_imgA - (long)a.cv_spi * KT) * 4;
+                cvB += (a.cv_imgB - (long)a.cv_spi * KT) * 4;
+            }
+        }
+    };
     auto load_slice = [&](auto mode, TileA& ra, TileB& rb, int slice) {
         constexpr int MODE = decltype(mode)::value;
         if (MODE == kFast) {
@@ -457,16 +521,30 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                 // iteration kt-1, which every wavefront left through the barrier.
                 const int wave_u = __builtin_amdgcn_readfirstlane(wave);
                 if (nk > 0) {
-                    ta.load_direct(originA, ta.goff, As[0], wave_u);
-                    tb.load_direct(originB, tb.goff, Bs[0], wave_u);
+                    if constexpr (CONV != 0) {
+                        const char *oa, *ob;
+                        conv_next(oa, ob);
+                        ta.load_direct(oa, ta.goff, As[0], wave_u);
+                        tb.load_direct(ob, tb.goff, Bs[0], wave_u);
+                    } else {
+                        ta.load_direct(originA, ta.goff, As[0], wave_u);
+                        tb.load_direct(originB, tb.goff, Bs[0], wave_u);
+                    }
                 }
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 __syncthreads();
                 for (int kt = 0; kt < nk; ++kt) {
                     const int cur = kt & 1;
                     if (kt + 1 < nk) {
-                        ta.load_direct(originA + (kt + 1) * stepA, ta.goff, As[cur ^ 1], wave_u);
-                        tb.load_direct(originB + (kt + 1) * stepB, tb.goff, Bs[cur ^ 1], wave_u);
+                        if constexpr (CONV != 0) {
+                            const char *oa, *ob;
+                            conv_next(oa, ob);
+                            ta.load_direct(oa, ta.goff, As[cur ^ 1], wave_u);
+                            tb.load_direct(ob, tb.goff, Bs[cur ^ 1], wave_u);
+                        } else {
+                            ta.load_direct(originA + (kt + 1) * stepA, ta.goff, As[cur ^ 1], wave_u);
+                            tb.load_direct(originB + (kt + 1) * stepB, tb.goff, Bs[cur ^ 1], wave_u);
+                        }
                     }
 #pragma unroll
                     for (int kk = 0; kk < KT / 8; ++kk) {
@@ -517,10 +595,14 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
             }
         }
     };
-    if (wholeA) ta.init_offsets(a.lda);
-    if (wholeB) tb.init_offsets(a.ldb);
-    if (wholeA && wholeB && !ragged_k) main_loop(std::integral_constant<int, kFast>{});
-    else main_loop(std::integral_constant<int, kMixed>{});
+    if (wholeA) ta.init_offsets(CONV != 0 ? a.cv_plane : a.lda);
+    if (wholeB) tb.init_offsets(CONV == 2 ? a.cv_plane : a.ldb);
+    if constexpr (CONV != 0) {
+        main_loop(std::integral_constant<int, kFast>{});      // the host sends whole tiles and whole slices only
+    } else {
+        if (wholeA && wholeB && !ragged_k) main_loop(std::integral_constant<int, kFast>{});
+        else main_loop(std::integral_constant<int, kMixed>{});
+    }
 
     // accumulator element e of a 32x32 block: row 8*(e/4) + 4*half + e%4, column l32.
     // Destination: C, this split's partial matrix, or (tail pieces) a tile-local
@@ -742,6 +824,39 @@ static void launch_shape(int shape, dim3 grid, hipStream_t st, const GemmArgs& a
     }
 }
 
+// implicit-convolution variants: 128-row tiles, N tile of 128 / 64 / 32
+static void launch_conv(int mode, int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
+    dim3 block(kGemmThreads);
+    if (mode == 1) {
+        switch (shape) {
+            case 0: sgemm_kernel<false, true, false, 2, 2, 2, 2, false, 1><<<grid, block, 0, st>>>(a); break;
+            case 2: sgemm_kernel<false, true, false, 4, 1, 1, 2, false, 1><<<grid, block, 0, st>>>(a); break;
+            default: sgemm_kernel<false, true, false, 4, 1, 1, 1, false, 1><<<grid, block, 0, st>>>(a); break;
+        }
+    } else {
+        switch (shape) {
+            case 0: sgemm_kernel<true, true, false, 2, 2, 2, 2, false, 2><<<grid, block, 0, st>>>(a); break;
+            case 2: sgemm_kernel<true, true, false, 4, 1, 1, 2, false, 2><<<grid, block, 0, st>>>(a); break;
+            default: sgemm_kernel<true, true, false, 4, 1, 1, 1, false, 2><<<grid, block, 0, st>>>(a); break;
+        }
+    }
+}
+
+// tile shape (index into kShapes) of an implicit-convolution product, -1 if none fits:
+// tiles must be whole -- 128 rows, and an N tile that divides the filter count (mode 1) or
+// the channel count, so that a tile of the (tap, channel) axis lies in one tap (mode 2)
+static int conv_shape(int mode, long filters, long channels) {
+    const long n = mode == 1 ? filters : channels;
+    if (mode == 2 && filters % 128 != 0) return -1;
+    if (channels % KT != 0) return -1;
+    if (n % 128 == 0) return 0;
+    if (n == 64) return 2;
+    if (n == 32) return 3;
+    return -1;
+}
+
+bool sgemm_conv_supported(int mode, long filters, long channels) { return conv_shape(mode, filters, channels) >= 0; }
+
 static void launch_trans(int tA, int tB, bool pipe, bool deep, int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
     dim3 block(kGemmThreads);
     if (deep) {     // 128x128 tiles, plain loop, not NT (there the second register set spills)
@@ -760,7 +875,7 @@ static void launch_trans(int tA, int tB, bool pipe, bool deep, int shape, dim3 g
 
 static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const float* A, long lda,
                          long sA, const float* B, long ldb, long sB, float* C, long ldc, long sC,
-                         void* stream, bool static_scratch = false) {
+                         void* stream, bool static_scratch = false, const ConvGemm* cv = nullptr) {
     CGT_ARG_CHECK(P >= 0 && M >= 0 && N >= 0 && K >= 0, "sgemm: negative size");
     if (P == 0 || M == 0 || N == 0) return CGT_AMD_OK;
     CGT_ARG_CHECK(A || K == 0, "sgemm: null A");
@@ -769,7 +884,7 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     CGT_ARG_CHECK(M < (1L << 31) - 128 && N < (1L << 31) - 128 && K < (1L << 31) - KT && P < 65536,
                   "sgemm: size too large");
     CGT_ARG_CHECK(ldc < (1L << 27) || M <= 4, "sgemm: ldc >= 2^27 with more than 4 rows is not supported");
-    CGT_ARG_CHECK(lda >= (tA ? M : K) && ldb >= (tB ? K : N) && ldc >= N,
+    CGT_ARG_CHECK(cv || (lda >= (tA ? M : K) && ldb >= (tB ? K : N) && ldc >= N),
                   "sgemm: leading dimension too small (lda=%ld ldb=%ld ldc=%ld)", lda, ldb, ldc);
     // tile shape: least padded work, ties to the earlier (larger) shape
     int shape = 0;
@@ -797,7 +912,21 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
         if (!p) ws_rc = CGT_AMD_ERR_HIP;
         return p;
     };
+    if (cv) {
+        shape = conv_shape(cv->mode, cv->mode == 1 ? N : M, cv->C);
+        CGT_ARG_CHECK(shape >= 0, "sgemm_conv: no tile shape for these extents");
+        CGT_ARG_CHECK(cv->plane < (1L << 24), "sgemm_conv: padded plane too large");
+    }
     GemmArgs a;
+    a.conv = cv ? cv->mode : 0;
+    if (cv) {
+        a.cv_wp = cv->wp; a.cv_kw = cv->kw; a.cv_cpb = (int)(cv->C / KT); a.cv_c = (int)cv->C;
+        a.cv_tpi = (int)cv->tpi; a.cv_spi = (int)cv->spi;
+        a.cv_plane = cv->plane;
+        // mode 1: A is the image; mode 2: A is the (shifted) padded cotangent with M planes per image, B the image
+        a.cv_imgA = (cv->mode == 1 ? cv->C : M) * cv->plane;
+        a.cv_imgB = cv->C * cv->plane;
+    }
     a.A = A; a.B = B; a.C = C;
     a.lda = lda; a.ldb = ldb; a.ldc = ldc;
     a.sA = sA; a.sB = sB; a.sC = sC;
@@ -809,7 +938,7 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     a.splits = 1;
     a.kchunk = (int)(cdiv(std::max(K, 1L), KT) * KT);
     a.ws = nullptr;
-    a.wide = (lda >= (1L << 23) || ldb >= (1L << 23)) ? 1 : 0;
+    a.wide = (!cv && (lda >= (1L << 23) || ldb >= (1L << 23))) ? 1 : 0;
     if (P == 1 && tiles < 512 && K >= 64 * KT) {
         long want = std::max(1L, 1024 / tiles);
         want = std::min(want, K / (8 * KT));                    // at least 8 slices per split
@@ -860,12 +989,13 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     // to work through, not when the whole product is one round of resident
     // workgroups (4096^3: 1024 tiles = 4 per CU), and not for a ragged K, where its
     // tiles would all take the register-staged variant (K = 363: plain loop +3 %).
-    const bool pipe = tiles * P >= 5L * kNumCU && K % KT == 0;
+    const bool pipe = !cv && tiles * P >= 5L * kNumCU && K % KT == 0;
     // two slices of loads in flight: one round of resident workgroups (they start together
     // and load in bursts) with a long K range each
     const long slices = cdiv(a.splits > 1 ? (long)a.kchunk : K, KT);
-    const bool deep = shape == 0 && !(!tA && tB) && wgs <= 4L * kNumCU && slices >= 32;
-    launch_trans(tA, tB, pipe, deep, shape, grid, st, a);
+    const bool deep = !cv && shape == 0 && !(!tA && tB) && wgs <= 4L * kNumCU && slices >= 32;
+    if (cv) launch_conv(cv->mode, shape, grid, st, a);
+    else launch_trans(tA, tB, pipe, deep, shape, grid, st, a);
     CGT_LAUNCH_CHECK("sgemm_kernel");
     if (a.splits > 1) {
         const long MN = M * N;
@@ -881,6 +1011,15 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
         CGT_LAUNCH_CHECK("tail_reduce_kernel");
     }
     return CGT_AMD_OK;
+}
+
+int sgemm_conv(const ConvGemm& cv, long M, long N, const float* A, const float* B, float* C, long ldc,
+               void* stream) {
+    const long taps = (long)cv.kh * cv.kw;
+    if (cv.mode == 1)   // A = image (row-contiguous operand), B = filters [N][taps * C]
+        return gemm_dispatch(1, 1, 1, M, N, taps * cv.C, A, M, 0, B, taps * cv.C, 0, C, ldc, 0, stream, false, &cv);
+    // A = cotangent planes [B][M][plane], B = image; K runs over (image, pixel slice)
+    return gemm_dispatch(0, 1, 1, M, N, cv.B * cv.spi * KT, A, cv.plane, 0, B, cv.plane, 0, C, ldc, 0, stream, false, &cv);
 }
 
 }  // namespace cgt_amd

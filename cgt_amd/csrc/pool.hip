@@ -290,12 +290,34 @@ CGT_API long cgt_amd_pool_outsize(long H, int k, int pad, int stride) {
 
 namespace cgt_amd {
 
+// The staged kernels split flat indices with fastdiv, which is exact below 2^21: they are
+// taken only while a workgroup's input and output index ranges stay below that; otherwise
+// the direct kernels (64-bit integer division) run.
+constexpr long kFastdivLimit = 1L << 21;
+
+// planes per workgroup of the staged forward kernel, 0: use the direct kernel
+static int pool_fwd_planes_per_wg(long H, long W, long PH, long PW) {
+    const long plane_bytes = H * W * (long)sizeof(float);
+    if (plane_bytes > 48 * 1024) return 0;
+    long ppw = std::max(1L, (16 * 1024) / std::max(1L, plane_bytes));
+    ppw = std::min(ppw, (kFastdivLimit - 1) / std::max(1L, PH * PW));   // pad >= kernel: more outputs than inputs
+    return ppw * H * W < kFastdivLimit && ppw >= 1 ? (int)ppw : 0;
+}
+
+// planes per workgroup of the staged generic pullback kernel, 0: use the direct kernel
+static int pool_bwd_planes_per_wg(long H, long W, long PH, long PW) {
+    const long out_bytes = PH * PW * 2 * (long)sizeof(float);  // top_diff + mask per plane
+    if (out_bytes > 48 * 1024) return 0;
+    long ppw = std::max(1L, (16 * 1024) / std::max(1L, out_bytes));
+    ppw = std::min(ppw, (kFastdivLimit - 1) / std::max(1L, H * W));     // large strides: huge planes, few outputs
+    return ppw >= 1 && ppw * PH * PW < kFastdivLimit ? (int)ppw : 0;
+}
+
 template <class G>
 static int launch_pool_fwd(G g, const float* bottom, long nplanes, long H, long W, long PH, long PW,
                            float* top, int* mask, hipStream_t st) {
     const long plane_bytes = H * W * (long)sizeof(float);
-    if (plane_bytes <= 48 * 1024) {
-        int ppw = (int)std::max(1L, (16 * 1024) / std::max(1L, plane_bytes));
+    if (int ppw = pool_fwd_planes_per_wg(H, W, PH, PW)) {
         const long blocks = cdiv(nplanes, ppw);
         max_pool_fwd_kernel<G><<<dim3((unsigned)blocks), dim3(kPoolThreads), (size_t)ppw * plane_bytes, st>>>(
             g, bottom, top, mask, nplanes, (int)H, (int)W, (int)PH, (int)PW, ppw);
@@ -328,8 +350,7 @@ static int launch_pool_bwd(G g, const int* mask, const float* top_diff, long npl
         }
     }
     const long out_bytes = PH * PW * 2 * (long)sizeof(float);  // top_diff + mask per plane
-    if (out_bytes <= 48 * 1024) {
-        int ppw = (int)std::max(1L, (16 * 1024) / out_bytes);
+    if (int ppw = pool_bwd_planes_per_wg(H, W, PH, PW)) {
         const long blocks = cdiv(nplanes, ppw);
         max_pool_bwd_kernel<G><<<dim3((unsigned)blocks), dim3(kPoolThreads), (size_t)ppw * out_bytes, st>>>(
             g, mask, top_diff, bottom_diff, nplanes, (int)H, (int)W, (int)PH, (int)PW, ppw);
@@ -345,6 +366,10 @@ static int launch_pool_bwd(G g, const int* mask, const float* top_diff, long npl
 }
 
 }  // namespace cgt_amd
+
+CGT_API int cgt_amd_pool_staged_planes(int backward, long H, long W, long PH, long PW) {
+    return backward ? pool_bwd_planes_per_wg(H, W, PH, PW) : pool_fwd_planes_per_wg(H, W, PH, PW);
+}
 
 CGT_API int cgt_amd_max_pool_f32(const float* bottom, long N, long C, long H, long W, int kh,
                                  int kw, int ph, int pw, int sh, int sw, long PH, long PW,

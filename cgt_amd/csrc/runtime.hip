@@ -20,8 +20,8 @@ void set_error(const char* fmt, ...) {
 void clear_error() { g_err[0] = 0; }
 
 struct StreamWorkspaces {
-    float* ptr[kWsUsers] = {nullptr, nullptr};
-    size_t bytes[kWsUsers] = {0, 0};
+    float* ptr[kWsUsers] = {};
+    size_t bytes[kWsUsers] = {};
     std::vector<void*> retired;
 };
 static std::mutex g_ws_mutex;

@@ -272,3 +272,58 @@ def conv2d_pullback(x, f, gy, pad=(0, 0), stride=(1, 1), col=None, stream=None):
     gx = col2im(gcol.reshape(B, m, n, Z), x.shape, (r, c), pad, stride, stream=stream)
     gf = mul22(gc, col.reshape(B * m * n, Z), True, False, stream=stream).reshape(f.shape)
     return gx, gf
+
+
+# ---------------------------------------------------------------- convolution without a column buffer
+
+def conv_same_supported(C, L, kernel, pad, stride):
+    """Whether the im2col-free path covers a layer (stride 1, odd kernel, pad = (kernel-1)/2,
+    channel / filter counts its GEMM tiles fit)."""
+    return bool(capi.lib().cgt_amd_conv_same_supported(int(C), int(L), *_geom(kernel, pad, stride)))
+
+
+def conv_same_padded_size(planes, H, W, kernel):
+    n = capi.lib().cgt_amd_conv_same_padded_size(int(planes), int(H), int(W), int(kernel[0]), int(kernel[1]))
+    if n < 0:
+        raise ValueError("conv_same: bad geometry")
+    return n
+
+
+def conv_same_pad(x, kernel, out=None, stream=None):
+    """Zero-padded copy of x [B,C,H,W] in the layout the im2col-free products read (a flat array)."""
+    _f32(x)
+    B, C, H, W = x.shape
+    res = _out(out, (conv_same_padded_size(B * C, H, W, kernel),))
+    capi.check(capi.lib().cgt_amd_conv_same_pad_f32(x.ptr, B * C, H, W, int(kernel[0]), int(kernel[1]), res.ptr, stream))
+    return res
+
+
+def conv_same_fwd(xpad, f, xshape, bias=None, relu=False, out=None, stream=None):
+    """conv2d (stride 1, same padding) from the padded input; optional fused bias add and rectify."""
+    _f32(xpad, f)
+    B, C, H, W = xshape
+    L, C2, kh, kw = f.shape
+    if C2 != C:
+        raise ValueError("filter channels %d != input channels %d" % (C2, C))
+    y = _out(out, (B, L, H, W))
+    capi.check(capi.lib().cgt_amd_conv_same_fwd_f32(xpad.ptr, f.ptr, None if bias is None else bias.ptr, int(bool(relu)),
+                                                    B, C, H, W, L, kh, kw, y.ptr, stream))
+    return y
+
+
+def conv_same_bwd_data(gypad, f, xshape, out=None, stream=None):
+    _f32(gypad, f)
+    B, C, H, W = xshape
+    L, _, kh, kw = f.shape
+    gx = _out(out, (B, C, H, W))
+    capi.check(capi.lib().cgt_amd_conv_same_bwd_data_f32(gypad.ptr, f.ptr, B, C, H, W, L, kh, kw, gx.ptr, stream))
+    return gx
+
+
+def conv_same_bwd_filter(gypad, xpad, xshape, fshape, out=None, stream=None):
+    _f32(gypad, xpad)
+    B, C, H, W = xshape
+    L, _, kh, kw = fshape
+    gf = _out(out, tuple(fshape))
+    capi.check(capi.lib().cgt_amd_conv_same_bwd_filter_f32(gypad.ptr, xpad.ptr, B, C, H, W, L, kh, kw, gf.ptr, stream))
+    return gf

@@ -196,6 +196,13 @@ int cgt_amd_col2im_f32(const float *col, long B, long C, long H, long W,
  * (cgt/nn_ops/max_pool_2d.py:40-41).  Returns 0 when the window does not fit. */
 long cgt_amd_pool_outsize(long H, int k, int pad, int stride);
 
+/* Host-side query, no launch: planes per workgroup the LDS-staged pooling kernel
+ * (backward != 0: the generic pullback kernel) would take for planes of H x W
+ * pooled to PH x PW, or 0 when the launcher falls back to the direct kernel --
+ * planes that do not fit LDS, or index ranges beyond what the staged kernels'
+ * reciprocal-multiply index split handles exactly (2^21). */
+int cgt_amd_pool_staged_planes(int backward, long H, long W, long PH, long PW);
+
 /* Max pooling with argmax.  bottom [N,C,H,W] -> top, mask [N,C,PH,PW].
  * Window rows/cols outside the image are skipped; the first maximum in
  * (h, w) scan order wins (strict >, starting from -FLT_MAX); mask holds
@@ -278,6 +285,52 @@ int cgt_amd_sgemm_batched(int tA, int tB, long P, long M, long N, long K,
                           const float *A, long lda, long strideA,
                           const float *B, long ldb, long strideB,
                           float *C, long ldc, long strideC, void *stream);
+
+/* ---------------------------------------------------------------- convolution without a column buffer
+ *
+ * conv2d with stride 1 and pad = (kernel - 1) / 2 (odd kernels), forward and
+ * both gradients, as GEMMs that read the image operand straight from a
+ * zero-padded copy of the image: no im2col / col2im pass and no [B,m,n,Z]
+ * column buffer.  They take the place, for the geometries they cover, of the
+ * reference's fused GPU convolution ops CudnnConvForward / BackwardData /
+ * BackwardFilter (cgt/nn_ops/cudnn_ops.py:58-143, include/cudnn_support.h:
+ * 135-215), and compute what nn.conv2d's im2col -> Mul22 composition computes
+ * (cgt/nn.py:95-100) to GEMM accuracy; the sums run over (tap, channel) instead
+ * of (channel, tap), so results agree with that composition to rounding, not
+ * bit for bit.
+ *
+ * Padded layout: `planes` planes of cgt_amd_conv_same_padded_size(1,...) -
+ * tail floats each, pixel (h, w) at (h + ph) * (W + 2 pw) + (w + pw), zeros
+ * elsewhere, plus a zeroed tail; cgt_amd_conv_same_pad_f32 writes all of it. */
+
+/* 1 if the three entry points below cover this layer: stride 1, odd kernel,
+ * pad = (kernel - 1) / 2, C and L in {32, 64, 128}, L = 128 for the weight
+ * gradient's tiles.  Otherwise use im2col + cgt_amd_sgemm + col2im. */
+int cgt_amd_conv_same_supported(long C, long L, int kh, int kw, int ph, int pw, int sh, int sw);
+
+/* Floats in the padded copy of `planes` planes of H x W (tail included); -1 on bad arguments. */
+long cgt_amd_conv_same_padded_size(long planes, long H, long W, int kh, int kw);
+
+/* x [planes][H][W] -> xpad (padded layout above; 16-byte aligned). */
+int cgt_amd_conv_same_pad_f32(const float *x, long planes, long H, long W, int kh, int kw,
+                              float *xpad, void *stream);
+
+/* y [B,L,H,W] = conv(x, f), f [L,C,kh,kw], from the padded x.  `bias` (L floats,
+ * may be NULL) is added per channel and, if relu != 0, the result is replaced by
+ * v * (v >= 0) -- the bias add and rectify of SpatialConvolution + nn.rectify
+ * (cgt/nn.py:44-45, 231-233) applied while the result is written, with the same
+ * fp32 operations as the separate ops.  Uses workspaces owned by the library. */
+int cgt_amd_conv_same_fwd_f32(const float *xpad, const float *f, const float *bias, int relu,
+                              long B, long C, long H, long W, long L, int kh, int kw,
+                              float *y, void *stream);
+
+/* gx [B,C,H,W] from the padded cotangent gypad (L planes per image). */
+int cgt_amd_conv_same_bwd_data_f32(const float *gypad, const float *f, long B, long C, long H, long W,
+                                   long L, int kh, int kw, float *gx, void *stream);
+
+/* gf [L,C,kh,kw] from the padded cotangent and the padded input. */
+int cgt_amd_conv_same_bwd_filter_f32(const float *gypad, const float *xpad, long B, long C, long H,
+                                     long W, long L, int kh, int kw, float *gf, void *stream);
 
 /* ---------------------------------------------------------------- conv glue */
 

@@ -45,6 +45,26 @@ def test_no_compute_needed_for_host_only_entry_points():
     assert capi.device_count() >= 0
 
 
+def test_staged_pool_kernels_stay_inside_their_index_range():
+    # the LDS-staged kernels split flat indices by reciprocal multiplication, exact below 2^21:
+    # the launcher must fall back to the direct kernels beyond that
+    from cgt_amd import capi
+    lib = capi.lib()
+    limit = 1 << 21
+    cases = [(55, 55, 26, 26), (56, 56, 27, 27), (2100, 2100, 65, 65), (1, 1, 1001, 1001), (3, 3, 700, 700),
+             (110, 110, 54, 54), (4000, 3, 124, 1), (1, 1, 1, 1), (40000, 40000, 10, 10)]
+    for H, W, PH, PW in cases:
+        for backward in (0, 1):
+            ppw = lib.cgt_amd_pool_staged_planes(backward, H, W, PH, PW)
+            assert ppw >= 0
+            if ppw:
+                assert ppw * H * W < limit and ppw * PH * PW < limit, (backward, H, W, PH, PW, ppw)
+                assert (PH * PW * 8 if backward else H * W * 4) <= 48 * 1024
+    assert lib.cgt_amd_pool_staged_planes(0, 55, 55, 26, 26) >= 1       # the AlexNet planes stay staged
+    assert lib.cgt_amd_pool_staged_planes(1, 2100, 2100, 65, 65) == 0   # 4.4 M cells per plane: direct kernel
+    assert lib.cgt_amd_pool_staged_planes(0, 1, 1, 1001, 1001) in (0, 1, 2)
+
+
 def test_argument_errors_are_reported_not_fatal():
     # argument validation happens on the host before any launch
     from cgt_amd import capi

@@ -209,6 +209,8 @@ def prebuild_standard_ops():
     info = nn_ops.im2col.Im2ColInfo(3, 3, 1, 1, 1, 1)
     pinfo = nn_ops.max_pool_2d.PoolInfo(2, 2, 0, 0, 2, 2)
     linfo = nn_ops.cross_channel_lrn.LRNInfo(5, 1e-4, 0.75)
+    cinfo = nn_ops.conv_same.ConvSameInfo(3, 3)
+    T1 = core.TensorType("f4", 1)
     todo = [
         (nn_ops.im2col.Im2Col(info), [T4]),
         (nn_ops.im2col.Col2Im(info), [T4, S, S, S, S]),
@@ -219,6 +221,11 @@ def prebuild_standard_ops():
         (core.Mul22(False, True), [T2, T2]),
         (core.BatchedMul22(False, False), [T3, T3]),
         (core.Transpose((0, 3, 1, 2)), [T4]),
+        (nn_ops.conv_same.ConvPad(cinfo), [T4]),
+        (nn_ops.conv_same.ConvForward(cinfo), [T4, T1, T4]),
+        (nn_ops.conv_same.ConvBackwardData(cinfo), [T1, T4, T4]),
+        (nn_ops.conv_same.ConvBackwardFilter(cinfo), [T1, T1, T4, T4]),
+        (core.Transport("gpu"), [T4]),
         # conv-layer glue: the closure code is generic over element type and
         # rank, so one library per op class serves every use
         (core.ElwiseUnary("exp"), [T4]),

@@ -195,6 +195,68 @@ CGT_API int cgt_amd_conv_same_pad_f32(const float* x, long planes, long H, long 
     return CGT_AMD_OK;
 }
 
+// ---- the pieces (each one kernel plus, for the products, the GEMM's own reduce kernel)
+
+CGT_API int cgt_amd_conv_same_filter_f32(const float* f, long L, long C, int kh, int kw, int flipped, float* fk,
+                                         void* stream) {
+    CGT_ARG_CHECK(L > 0 && C > 0 && kh > 0 && kw > 0 && f && fk, "conv_same_filter: bad arguments");
+    if (!flipped) {     // [L][C][kh][kw] -> [L][tap][C]: the K axis of the product is (tap, channel)
+        const long fs[4] = {L, C, kh, kw};
+        const int ax[4] = {0, 2, 3, 1};
+        return cgt_amd_transpose4_f32(f, fs, ax, fk, stream);
+    }
+    const long total = L * C * kh * kw;
+    flip_filters_kernel<<<dim3((unsigned)std::min(cdiv(total, 256L), 4096L)), dim3(256), 0, as_stream(stream)>>>(
+        f, fk, (int)L, (int)C, kh, kw);
+    CGT_LAUNCH_CHECK("flip_filters_kernel");
+    return CGT_AMD_OK;
+}
+
+CGT_API long cgt_amd_conv_same_rows_size(long B, long H, long W, long N, int kh, int kw) {
+    SameGeom g;
+    if (B < 0 || N <= 0 || H <= 0 || W <= 0 || !make_geom(g, B, 1, H, W, N, kh, kw)) return -1;
+    return B * g.tpi * 128 * N;
+}
+
+CGT_API int cgt_amd_conv_same_rows_f32(const float* imgpad, const float* fk, long B, long Cin, long H, long W,
+                                       long N, int kh, int kw, float* rows, void* stream) {
+    SameGeom g;
+    int rc = check_same("conv_same_rows", g, B, Cin, H, W, N, kh, kw);
+    if (rc) return rc;
+    if (B == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(imgpad && fk && rows, "conv_same_rows: null pointer");
+    CGT_ARG_CHECK(sgemm_conv_supported(1, N, Cin), "conv_same_rows: unsupported extents (%ld channels, %ld filters)", Cin, N);
+    ConvGemm cv = {1, B, Cin, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi};
+    return sgemm_conv(cv, B * g.tpi * 128, N, imgpad, fk, rows, N, stream);
+}
+
+CGT_API int cgt_amd_conv_same_rows_to_nchw_f32(const float* rows, const float* bias, int relu, long B, long N,
+                                               long H, long W, int kh, int kw, float* out, void* stream) {
+    SameGeom g;
+    int rc = check_same("conv_same_rows_to_nchw", g, B, 1, H, W, N, kh, kw);
+    if (rc) return rc;
+    if (B == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(rows && out && N % 4 == 0 && N <= 128, "conv_same_rows_to_nchw: bad arguments");
+    return rows_to_nchw(g, rows, N, bias, relu, out, as_stream(stream));
+}
+
+CGT_API int cgt_amd_conv_same_wgrad_f32(const float* gypad, const float* xpad, long B, long C, long H, long W,
+                                        long L, int kh, int kw, float* gfk, void* stream) {
+    SameGeom g;
+    int rc = check_same("conv_same_wgrad", g, B, C, H, W, L, kh, kw);
+    if (rc) return rc;
+    CGT_ARG_CHECK(gfk, "conv_same_wgrad: null pointer");
+    const long taps = (long)kh * kw;
+    if (B == 0) return cgt_amd_fill_u32(gfk, 0u, L * C * taps, stream);
+    CGT_ARG_CHECK(gypad && xpad, "conv_same_wgrad: null pointer");
+    CGT_ARG_CHECK(sgemm_conv_supported(2, L, C), "conv_same_wgrad: unsupported extents (%ld channels, %ld filters)", C, L);
+    // pixel q of the padded grid <-> cotangent at q + (ph * Wp + pw): its padding is zero, so junk pixels add nothing
+    ConvGemm cv = {2, B, C, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi};
+    return sgemm_conv(cv, L, taps * C, gypad + g.ph * g.Wp + g.pw, xpad, gfk, taps * C, stream);
+}
+
+// ---- the three products of a layer, composed from the pieces with library-owned workspaces
+
 CGT_API int cgt_amd_conv_same_fwd_f32(const float* xpad, const float* f, const float* bias, int relu, long B, long C,
                                       long H, long W, long L, int kh, int kw, float* y, void* stream) {
     SameGeom g;
@@ -207,14 +269,8 @@ CGT_API int cgt_amd_conv_same_fwd_f32(const float* xpad, const float* f, const f
     float* wk = stream_workspace(stream, kWsConvFilter, (size_t)L * C * taps * sizeof(float), "conv_same_fwd");
     float* rows = stream_workspace(stream, kWsConvRows, (size_t)B * g.tpi * 128 * std::max(L, C) * sizeof(float), "conv_same_fwd");
     if (!wk || !rows) return CGT_AMD_ERR_NOMEM;
-    // filters [L][C][kh][kw] -> [L][tap][C]: the K axis of the product is (tap, channel)
-    const long fs[4] = {L, C, kh, kw};
-    const int ax[4] = {0, 2, 3, 1};
-    rc = cgt_amd_transpose4_f32(f, fs, ax, wk, stream);
-    if (rc) return rc;
-    ConvGemm cv = {1, B, C, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi};
-    rc = sgemm_conv(cv, B * g.tpi * 128, L, xpad, wk, rows, L, stream);
-    if (rc) return rc;
+    if ((rc = cgt_amd_conv_same_filter_f32(f, L, C, kh, kw, 0, wk, stream))) return rc;
+    if ((rc = cgt_amd_conv_same_rows_f32(xpad, wk, B, C, H, W, L, kh, kw, rows, stream))) return rc;
     return rows_to_nchw(g, rows, L, bias, relu, y, as_stream(stream));
 }
 
@@ -230,13 +286,9 @@ CGT_API int cgt_amd_conv_same_bwd_data_f32(const float* gypad, const float* f, l
     float* wk = stream_workspace(stream, kWsConvFilter, (size_t)L * C * taps * sizeof(float), "conv_same_bwd_data");
     float* rows = stream_workspace(stream, kWsConvRows, (size_t)B * g.tpi * 128 * std::max(L, C) * sizeof(float), "conv_same_bwd_data");
     if (!wk || !rows) return CGT_AMD_ERR_NOMEM;
-    flip_filters_kernel<<<dim3((unsigned)std::min(cdiv(L * C * taps, 256L), 4096L)), dim3(256), 0, as_stream(stream)>>>(
-        f, wk, (int)L, (int)C, kh, kw);
-    CGT_LAUNCH_CHECK("flip_filters_kernel");
-    // a forward convolution of the cotangent: L channels in, C "filters" [C][tap][L]
-    ConvGemm cv = {1, B, L, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi};
-    rc = sgemm_conv(cv, B * g.tpi * 128, C, gypad, wk, rows, C, stream);
-    if (rc) return rc;
+    // a forward convolution of the cotangent: L channels in, C "filters" [C][flipped tap][L]
+    if ((rc = cgt_amd_conv_same_filter_f32(f, L, C, kh, kw, 1, wk, stream))) return rc;
+    if ((rc = cgt_amd_conv_same_rows_f32(gypad, wk, B, L, H, W, C, kh, kw, rows, stream))) return rc;
     return rows_to_nchw(g, rows, C, nullptr, 0, gx, as_stream(stream));
 }
 
@@ -248,14 +300,10 @@ CGT_API int cgt_amd_conv_same_bwd_filter_f32(const float* gypad, const float* xp
     CGT_ARG_CHECK(gf, "conv_same_bwd_filter: null pointer");
     const long taps = (long)kh * kw;
     if (B == 0) return cgt_amd_fill_u32(gf, 0u, L * C * taps, stream);
-    CGT_ARG_CHECK(gypad && xpad, "conv_same_bwd_filter: null pointer");
     CGT_ARG_CHECK(cgt_amd_conv_same_supported(C, L, kh, kw, g.ph, g.pw, 1, 1), "conv_same_bwd_filter: unsupported extents C=%ld L=%ld", C, L);
     float* wk = stream_workspace(stream, kWsConvFilter, (size_t)L * C * taps * sizeof(float), "conv_same_bwd_filter");
     if (!wk) return CGT_AMD_ERR_NOMEM;
-    // pixel q of the padded grid <-> cotangent at q + (ph * Wp + pw): its padding is zero, so junk pixels add nothing
-    ConvGemm cv = {2, B, C, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi};
-    rc = sgemm_conv(cv, L, taps * C, gypad + g.ph * g.Wp + g.pw, xpad, wk, taps * C, stream);
-    if (rc) return rc;
+    if ((rc = cgt_amd_conv_same_wgrad_f32(gypad, xpad, B, C, H, W, L, kh, kw, wk, stream))) return rc;
     // [L][tap][C] -> [L][C][kh][kw]
     const long ws[4] = {L, kh, kw, C};
     const int ax[4] = {0, 3, 1, 2};

@@ -2,19 +2,40 @@
 
 conv2d keeps the reference's CPU-path composition
     im2col -> reshape -> Mul22(False, True) -> reshape -> transpose{0,3,1,2}
-with every op running on the GPU (the reference's devtype == "gpu" branch
-calls cuDNN instead, which this build replaces).
+with every op running on the GPU.  Where the reference's devtype == "gpu"
+branch switches to fused convolution ops (cuDNN, cgt/nn.py:88-93), this build
+switches to its own fused ops for the layers they cover -- stride 1, pad =
+(kernel - 1) / 2, channel and filter counts their GEMM tiles fit (nn_ops/
+conv_same.py) -- which need no column buffer; conv_algo("im2col") keeps the
+composition for every layer.
 """
 from . import core
+from .nn_ops import conv_same
 from .nn_ops.cross_channel_lrn import cross_channel_lrn  # noqa: F401
 from .nn_ops.im2col import im2col
 from .nn_ops.max_pool_2d import MaxPool, PoolInfo
+
+
+_CONV_ALGO = "auto"
+
+
+def conv_algo(name=None):
+    """Select how conv2d is built: "auto" (fused ops where they apply) or "im2col"
+    (always the im2col -> Mul22 composition).  Returns the previous setting."""
+    global _CONV_ALGO
+    old = _CONV_ALGO
+    if name is not None:
+        assert name in ("auto", "im2col")
+        _CONV_ALGO = name
+    return old
 
 
 def conv2d(x_BKRC, f_LKrc, kernelshape, pad=(0, 0), stride=(1, 1)):
     x_BKRC, f_LKrc = core.as_node(x_BKRC), core.as_node(f_LKrc)
     L, K, r, c = f_LKrc.shape
     assert tuple(kernelshape) == (r, c), "kernelshape must match the filter's last two axes"
+    if _CONV_ALGO == "auto" and conv_same.supported(x_BKRC, f_LKrc, kernelshape, pad, stride):
+        return conv_same.conv_same(x_BKRC, f_LKrc, kernelshape)
     col_BmnZ = im2col(x_BKRC, kernelshape, pad, stride)
     f_LZ = f_LKrc.reshape([L, K * r * c])
     B, m, n, Z = col_BmnZ.shape

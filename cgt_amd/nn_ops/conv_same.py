@@ -1,0 +1,191 @@
+"""Fused convolution ops for stride 1 and pad = (kernel - 1) / 2: forward, data
+gradient and weight gradient without a column buffer.
+
+They stand where the reference's GPU branch of nn.conv2d puts its fused ops --
+CudnnConvForward with its pullback made of CudnnConvBackwardData /
+CudnnConvBackwardFilter (cgt/nn_ops/cudnn_ops.py:58-143, cgt/nn.py:88-93) --
+with this library's own kernels behind them instead of cuDNN.  The image
+operand of each product is the zero-padded copy made by ConvPad, which the
+forward op and both gradients share.
+"""
+import ctypes
+from collections import namedtuple
+
+from .. import core
+
+ConvSameInfo = namedtuple("ConvSameInfo", ["kernel_h", "kernel_w"])
+
+
+def info2closure(info):
+    return [("kernel_h", ctypes.c_int, info.kernel_h), ("kernel_w", ctypes.c_int, info.kernel_w)]
+
+
+def padded_size(planes, H, W, info):
+    """Floats in the padded copy of `planes` planes (cgt_amd_conv_same_padded_size), as a
+    shape expression."""
+    Hp, Wp = H + 2 * ((info.kernel_h - 1) // 2), W + 2 * ((info.kernel_w - 1) // 2)
+    plane = (Hp * Wp + 16 + 15) // 16 * 16
+    tail = (256 + info.kernel_h * Wp + 3) // 4 * 4
+    return planes * plane + tail
+
+
+class ConvPad(core.Op):
+    """x [B,C,H,W] -> flat zero-padded copy, the layout the products read."""
+    available_impls = ("native_gpu",)
+
+    def __init__(self, info):
+        self.info = info
+
+    def get_diff(self, _):
+        return [False]          # gradients reach x through ConvForward's own pullback
+
+    def shp_apply(self, inputs):
+        B, C, H, W = core.shape(inputs[0])
+        return [padded_size(B * C, H, W, self.info)]
+
+    def typ_apply(self, input_types):
+        assert input_types[0].ndim == 4 and input_types[0].dtype == "f4"
+        return core.TensorType("f4", 1)
+
+    def get_native_compile_info(self, input_types, devtype):
+        assert devtype == "gpu"
+        code = r"""
+            CGT_EXPORT_C void $function($closure* cl, cgtArray** reads, cgtArray* write) {
+                cgtArray* x = reads[0];
+                const long* s = x->shape();
+                long need = cgt_amd_conv_same_padded_size(s[0] * s[1], s[2], s[3], cl->kernel_h, cl->kernel_w);
+                cgt_check(write->size() == need, "ConvPad: output has %ld floats, the geometry needs %ld", write->size(), need);
+                if (cgtGlobalStatus != cgtStatusOK) return;
+                int rc = cgt_amd_conv_same_pad_f32((const float*)x->data(), s[0] * s[1], s[2], s[3],
+                    cl->kernel_h, cl->kernel_w, (float*)write->data(), cgt_get_stream());
+                cgt_check(rc == CGT_AMD_OK, "ConvPad: %s", cgt_amd_last_error());
+            }"""
+        return core.NativeCompileInfo(code, includes=["cgt_amd.h"], closure_triples=info2closure(self.info),
+                                      gpu_deref_mask=(True,))
+
+
+_CHECK_PADDED = r"""
+                long need = cgt_amd_conv_same_padded_size(%s, H, W, cl->kernel_h, cl->kernel_w);
+                cgt_check(%s->size() == need, "%s: padded operand has %%ld floats, the geometry needs %%ld", %s->size(), need);
+"""
+
+
+class ConvForward(core.Op):
+    """inputs [x, xpad, f] -> y [B,L,H,W].  x gives the shape and receives the gradient;
+    the product reads xpad = ConvPad(x)."""
+    available_impls = ("native_gpu",)
+
+    def __init__(self, info):
+        self.info = info
+
+    def get_diff(self, _):
+        return [True, False, True]
+
+    def shp_apply(self, inputs):
+        B, _, H, W = core.shape(inputs[0])
+        return [B, core.size(inputs[2], 0), H, W]
+
+    def typ_apply(self, input_types):
+        return core.TensorType("f4", 4)
+
+    def pullback(self, inputs, output, goutput):
+        return self.pullback_wanted(inputs, output, goutput, [True, False, True])
+
+    def pullback_wanted(self, inputs, output, goutput, wanted):
+        x, xpad, f = inputs
+        gypad = core.Result(ConvPad(self.info), [goutput])
+        gx = core.Result(ConvBackwardData(self.info), [gypad, f, x]) if wanted[0] else None
+        gf = core.Result(ConvBackwardFilter(self.info), [gypad, xpad, f, x]) if wanted[2] else None
+        return [gx, None, gf]
+
+    def get_native_compile_info(self, input_types, devtype):
+        assert devtype == "gpu"
+        code = r"""
+            CGT_EXPORT_C void $function($closure* cl, cgtArray** reads, cgtArray* write) {
+                cgtArray *x = reads[0], *xpad = reads[1], *f = reads[2];
+                long B = x->shape()[0], C = x->shape()[1], H = x->shape()[2], W = x->shape()[3], L = f->shape()[0];
+                cgt_check(f->ndim() == 4 && f->shape()[1] == C && f->shape()[2] == cl->kernel_h && f->shape()[3] == cl->kernel_w
+                          && write->size() == B * L * H * W, "ConvForward: filters or output do not fit the input");
+""" + _CHECK_PADDED % ("B * C", "xpad", "ConvForward", "xpad") + r"""
+                if (cgtGlobalStatus != cgtStatusOK) return;
+                int rc = cgt_amd_conv_same_fwd_f32((const float*)xpad->data(), (const float*)f->data(), NULL, 0,
+                    B, C, H, W, L, cl->kernel_h, cl->kernel_w, (float*)write->data(), cgt_get_stream());
+                cgt_check(rc == CGT_AMD_OK, "ConvForward: %s", cgt_amd_last_error());
+            }"""
+        return core.NativeCompileInfo(code, includes=["cgt_amd.h"], closure_triples=info2closure(self.info),
+                                      gpu_deref_mask=(False, True, True))
+
+
+class ConvBackwardData(core.Op):
+    """inputs [gypad, f, x] -> gx (x gives the shape only)."""
+    available_impls = ("native_gpu",)
+
+    def __init__(self, info):
+        self.info = info
+
+    def shp_apply(self, inputs):
+        return core.shape(inputs[2])
+
+    def typ_apply(self, input_types):
+        return core.TensorType("f4", 4)
+
+    def get_native_compile_info(self, input_types, devtype):
+        assert devtype == "gpu"
+        code = r"""
+            CGT_EXPORT_C void $function($closure* cl, cgtArray** reads, cgtArray* write) {
+                cgtArray *gypad = reads[0], *f = reads[1], *x = reads[2];
+                long B = x->shape()[0], C = x->shape()[1], H = x->shape()[2], W = x->shape()[3], L = f->shape()[0];
+                cgt_check(f->ndim() == 4 && f->shape()[1] == C && f->shape()[2] == cl->kernel_h && f->shape()[3] == cl->kernel_w
+                          && write->size() == x->size(), "ConvBackwardData: filters or output do not fit the input");
+""" + _CHECK_PADDED % ("B * L", "gypad", "ConvBackwardData", "gypad") + r"""
+                if (cgtGlobalStatus != cgtStatusOK) return;
+                int rc = cgt_amd_conv_same_bwd_data_f32((const float*)gypad->data(), (const float*)f->data(),
+                    B, C, H, W, L, cl->kernel_h, cl->kernel_w, (float*)write->data(), cgt_get_stream());
+                cgt_check(rc == CGT_AMD_OK, "ConvBackwardData: %s", cgt_amd_last_error());
+            }"""
+        return core.NativeCompileInfo(code, includes=["cgt_amd.h"], closure_triples=info2closure(self.info),
+                                      gpu_deref_mask=(True, True, False))
+
+
+class ConvBackwardFilter(core.Op):
+    """inputs [gypad, xpad, f, x] -> gf (f and x give shapes only)."""
+    available_impls = ("native_gpu",)
+
+    def __init__(self, info):
+        self.info = info
+
+    def shp_apply(self, inputs):
+        return core.shape(inputs[2])
+
+    def typ_apply(self, input_types):
+        return core.TensorType("f4", 4)
+
+    def get_native_compile_info(self, input_types, devtype):
+        assert devtype == "gpu"
+        code = r"""
+            CGT_EXPORT_C void $function($closure* cl, cgtArray** reads, cgtArray* write) {
+                cgtArray *gypad = reads[0], *xpad = reads[1], *f = reads[2], *x = reads[3];
+                long B = x->shape()[0], C = x->shape()[1], H = x->shape()[2], W = x->shape()[3], L = f->shape()[0];
+                cgt_check(f->ndim() == 4 && f->shape()[1] == C && f->shape()[2] == cl->kernel_h && f->shape()[3] == cl->kernel_w
+                          && write->size() == f->size(), "ConvBackwardFilter: output does not fit the filters");
+""" + _CHECK_PADDED % ("B * L", "gypad", "ConvBackwardFilter", "gypad") + _CHECK_PADDED.replace("long need", "need") % ("B * C", "xpad", "ConvBackwardFilter", "xpad") + r"""
+                if (cgtGlobalStatus != cgtStatusOK) return;
+                int rc = cgt_amd_conv_same_bwd_filter_f32((const float*)gypad->data(), (const float*)xpad->data(),
+                    B, C, H, W, L, cl->kernel_h, cl->kernel_w, (float*)write->data(), cgt_get_stream());
+                cgt_check(rc == CGT_AMD_OK, "ConvBackwardFilter: %s", cgt_amd_last_error());
+            }"""
+        return core.NativeCompileInfo(code, includes=["cgt_amd.h"], closure_triples=info2closure(self.info),
+                                      gpu_deref_mask=(True, True, False, False))
+
+
+def supported(x, f, kernelshape, pad, stride):
+    """Whether these ops cover the layer (see cgt_amd_conv_same_supported)."""
+    from .. import kernels
+    return kernels.conv_same_supported(core.size(x, 1), core.size(f, 0), kernelshape, pad, stride)
+
+
+def conv_same(x, f, kernelshape):
+    x, f = core.as_node(x), core.as_node(f)
+    info = ConvSameInfo(int(kernelshape[0]), int(kernelshape[1]))
+    xpad = core.Result(ConvPad(info), [x])
+    return core.Result(ConvForward(info), [x, xpad, f])

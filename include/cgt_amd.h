@@ -324,6 +324,26 @@ int cgt_amd_conv_same_fwd_f32(const float *xpad, const float *f, const float *bi
                               long B, long C, long H, long W, long L, int kh, int kw,
                               float *y, void *stream);
 
+/* The pieces the three products are made of, one kernel each (plus the GEMM's
+ * own reduce kernel), for a host that keeps the intermediate buffers itself:
+ *   filter   f [L,C,kh,kw] -> fk: [L][tap][C] (flipped = 0: forward) or
+ *            [C][flipped tap][L] (flipped = 1: the data gradient's filter bank)
+ *   rows     rows[b][q][n] = sum_{tap,c} imgpad[b][c][q + tapoff] * fk[n][tap][c],
+ *            q = h*(W+2pw) + w, cgt_amd_conv_same_rows_size floats (each image's
+ *            rows are rounded up to whole tiles of 128)
+ *   rows_to_nchw   rows -> out [B,N,H,W] (+ bias, rectify)
+ *   wgrad    gfk [L][tap][C] from the two padded arrays; transpose4 {0,3,1,2}
+ *            of it viewed [L,kh,kw,C] is gf [L,C,kh,kw] */
+int cgt_amd_conv_same_filter_f32(const float *f, long L, long C, int kh, int kw, int flipped,
+                                 float *fk, void *stream);
+long cgt_amd_conv_same_rows_size(long B, long H, long W, long N, int kh, int kw);
+int cgt_amd_conv_same_rows_f32(const float *imgpad, const float *fk, long B, long Cin, long H, long W,
+                               long N, int kh, int kw, float *rows, void *stream);
+int cgt_amd_conv_same_rows_to_nchw_f32(const float *rows, const float *bias, int relu, long B, long N,
+                                       long H, long W, int kh, int kw, float *out, void *stream);
+int cgt_amd_conv_same_wgrad_f32(const float *gypad, const float *xpad, long B, long C, long H, long W,
+                                long L, int kh, int kw, float *gfk, void *stream);
+
 /* gx [B,C,H,W] from the padded cotangent gypad (L planes per image). */
 int cgt_amd_conv_same_bwd_data_f32(const float *gypad, const float *f, long B, long C, long H, long W,
                                    long L, int kh, int kw, float *gx, void *stream);

@@ -107,3 +107,74 @@ def test_conv_same_supported_rule(K):
     assert not K.conv_same_supported(128, 128, (3, 3), (0, 0), (1, 1))    # valid padding
     assert not K.conv_same_supported(128, 128, (2, 2), (0, 0), (1, 1))    # even kernel
     assert not K.conv_same_supported(32, 64, (5, 5), (2, 2), (1, 1))      # 64 filters: no weight-gradient tile
+
+
+def test_nn_conv2d_takes_the_fused_ops_and_grad_goes_through_them(K):
+    # nn.conv2d picks the fused ops for a layer they cover; grad walks ConvForward's own
+    # pullback (ConvPad of the cotangent, ConvBackwardData, ConvBackwardFilter); a compiled
+    # function replays the same closures and serves another batch size
+    import cgt_amd as cgt
+    from cgt_amd import nn
+    from cgt_amd.nn_ops import conv_same
+    rs = np.random.RandomState(3)
+    x = rs.randn(3, 32, 12, 10).astype(np.float32)
+    f = (rs.randn(128, 32, 3, 3) / 17).astype(np.float32)
+
+    def graph(xn, fn):
+        y = nn.conv2d(xn, fn, (3, 3), pad=(1, 1))
+        pooled = nn.max_pool_2d(nn.rectify(y), (2, 2), (0, 0), (2, 2))
+        loss = cgt.sum(pooled * pooled)
+        gx, gf = cgt.grad(loss, [xn, fn])
+        return y, loss, gx, gf
+
+    xn, fn = cgt.constant(x), cgt.constant(f)
+    y, loss, gx, gf = graph(xn, fn)
+    assert isinstance(y.op, conv_same.ConvForward) and isinstance(gx.op, conv_same.ConvBackwardData)
+    assert isinstance(gf.op, conv_same.ConvBackwardFilter)
+    d = np.float64
+    y64 = O.conv2d(x.astype(d), f.astype(d), (1, 1), (1, 1))
+    r64 = y64 * (y64 >= 0)
+    p64, mask = O.max_pool(r64, (2, 2), (0, 0), (2, 2))
+    gr = O.max_pool_pullback(r64.shape, mask, 2 * p64) * (y64 >= 0)
+    gx64, gf64 = O.conv2d_pullback(x.astype(d), f.astype(d), gr, (1, 1), (1, 1))
+    assert relfro(y.get(), y64) <= TOL and abs(float(loss.get()) - (p64 ** 2).sum()) <= TOL * (p64 ** 2).sum()
+    assert relfro(gx.get(), gx64) <= TOL and relfro(gf.get(), gf64) <= TOL
+    # the im2col composition of the same layer: same results to rounding
+    old = nn.conv_algo("im2col")
+    try:
+        y_c, loss_c, gx_c, gf_c = graph(cgt.constant(x), cgt.constant(f))
+        assert not isinstance(y_c.op, conv_same.ConvForward)
+    finally:
+        nn.conv_algo(old)
+    assert relfro(y.get(), y_c.get()) <= 1e-5 and relfro(gx.get(), gx_c.get()) <= 1e-4 and relfro(gf.get(), gf_c.get()) <= 1e-4
+    fun = cgt.function([xn], [y, loss, gx, gf])
+    for got, node in zip(fun(x), (y, loss, gx, gf)):
+        assert np.array_equal(got.view(np.uint32), node.get().view(np.uint32))
+    x5 = rs.randn(5, 32, 12, 10).astype(np.float32)
+    fresh = graph(cgt.constant(x5), fn)
+    for got, node in zip(fun(x5), fresh):
+        assert np.array_equal(got.view(np.uint32), node.get().view(np.uint32))
+
+
+def test_vgg_layer_full_size_through_the_fused_ops(K):
+    # the headline layer at full size: slices against the float64 oracle, the rest through
+    # the adjoint identity <conv(x), gy> = <x, conv^T(gy)> and linearity in the filters
+    from cgt_amd.gpuarray import to_gpu
+    rs = np.random.RandomState(0)
+    B, C, H, W, L = 64, 128, 56, 56, 128
+    x = rs.randn(B, C, H, W).astype(np.float32)
+    f = (rs.randn(L, C, 3, 3) * np.sqrt(1.0 / (C * 9))).astype(np.float32)
+    gy = rs.randn(B, L, H, W).astype(np.float32)
+    xg, fg = to_gpu(x), to_gpu(f)
+    xpad, gypad = K.conv_same_pad(xg, (3, 3)), K.conv_same_pad(to_gpu(gy), (3, 3))
+    y = K.conv_same_fwd(xpad, fg, x.shape).get()
+    gx = K.conv_same_bwd_data(gypad, fg, x.shape).get()
+    gf = K.conv_same_bwd_filter(gypad, xpad, x.shape, f.shape).get()
+    d = np.float64
+    for b in (0, 37, 63):
+        y64 = O.conv2d(x[b:b + 1].astype(d), f.astype(d), (1, 1), (1, 1))
+        gx64, _ = O.conv2d_pullback(x[b:b + 1].astype(d), f.astype(d), gy[b:b + 1].astype(d), (1, 1), (1, 1))
+        assert relfro(y[b:b + 1], y64) <= TOL and relfro(gx[b:b + 1], gx64) <= TOL
+    lhs = float(np.vdot(y.astype(d), gy.astype(d)))
+    assert abs(lhs - float(np.vdot(x.astype(d), gx.astype(d)))) <= 1e-5 * abs(lhs)
+    assert abs(lhs - float(np.vdot(f.astype(d), gf.astype(d)))) <= 1e-5 * abs(lhs)

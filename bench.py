@@ -61,9 +61,12 @@ WORKLOADS = {
 GEMM_WORKLOAD = "raw_gemm_4096_and_batched_64x512"
 DEFAULT_WORKLOAD = "vgg_mid_conv3x3_128x56x56_b64"
 
-# The workloads the default run reports beside the headline one, under "workloads"
-EXTRA_WORKLOADS = ["alexnet_conv1_11x11s4_3x227x227_b128", GEMM_WORKLOAD, "cifar_conv1_5x5_3x32x32_b128",
-                   "mnist_conv3x3_1x28x28_b64"]
+# The workloads the default run reports beside the headline one, under "workloads"; the
+# headline layer once more as the im2col -> Mul22 -> col2im composition, which is how
+# layers the fused ops do not cover run and where the VGG-sized im2col / col2im figures are
+IM2COL_SUFFIX = "/im2col"
+EXTRA_WORKLOADS = [DEFAULT_WORKLOAD + IM2COL_SUFFIX, "alexnet_conv1_11x11s4_3x227x227_b128", GEMM_WORKLOAD,
+                   "cifar_conv1_5x5_3x32x32_b128", "mnist_conv3x3_1x28x28_b64"]
 
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries of this script, per workload
 PROFILE_PREFIX = {
@@ -93,13 +96,21 @@ def _pmc_rows(path):
     return scale, rows
 
 
-def traffic_from_profiles(workload, profiles_dir=None):
+def profile_prefix(workload, algo):
+    base = workload[:-len(IM2COL_SUFFIX)] if workload.endswith(IM2COL_SUFFIX) else workload
+    prefix = PROFILE_PREFIX.get(base)
+    if prefix is None:
+        return None
+    return prefix + ("_im2col" if algo == "im2col" and base == DEFAULT_WORKLOAD else "")
+
+
+def traffic_from_profiles(workload, algo=None, stage_names=("gemm_fwd_NT", "gemm_dgrad_NN", "gemm_wgrad_TN"), profiles_dir=None):
     """HBM bytes per launch of each GEMM stage of a step, read from the committed counter
     summaries: stage -> calibrated FETCH_SIZE + WRITE_SIZE bytes of the sgemm launch and of
     the reduce kernel that follows it (split-K / tail partials).  The summaries list kernels
     in launch order, so the sgemm rows are, in order, the forward product, the data gradient
     and the weight gradient.  {} when the workload has no summaries."""
-    prefix = PROFILE_PREFIX.get(workload)
+    prefix = profile_prefix(workload, algo)
     profiles_dir = profiles_dir or os.path.join(ROOT, "profiles")
     if prefix is None:
         return {}
@@ -111,7 +122,7 @@ def traffic_from_profiles(workload, profiles_dir=None):
         scale, rows = _pmc_rows(path)
         if scale is None:
             return {}
-        order = iter(["gemm_fwd_NT", "gemm_dgrad_NN", "gemm_wgrad_TN"])
+        order = iter(stage_names)
         stage = None
         for name, mb in rows:
             if "sgemm_kernel" in name:
@@ -148,7 +159,7 @@ class Stage(object):
 class LayerOnGpu(object):
     """One configured layer with every buffer pre-allocated on the device."""
 
-    def __init__(self, cfg, overlap=False, glue=False):
+    def __init__(self, cfg, overlap=False, glue=False, algo="auto"):
         from cgt_amd import capi, kernels as K
         from cgt_amd.gpuarray import empty, to_gpu
         # two streams (default priority): the weight-gradient GEMM depends only on
@@ -170,12 +181,19 @@ class LayerOnGpu(object):
         self.dims = dict(B=B, C=C, H=H, W=W, L=L, r=r, c=c, m=m, n=n, Z=Z, Bmn=Bmn)
         self.x, self.f = to_gpu(x), to_gpu(f)
         self.f_LZ = self.f.reshape(L, Z)
+        nelem = lambda a: int(np.prod(a.shape))  # noqa: E731
+        # what nn.conv2d builds for this layer: the fused ops without a column buffer where they
+        # apply (stride 1, same padding, tile-sized channel counts), else im2col -> Mul22
+        self.algo = "direct" if algo == "auto" and K.conv_same_supported(C, L, (r, c), pad, stride) else "im2col"
+        if self.algo == "direct":
+            self.overlap = False
+            self._direct_stages(K, cfg, nelem)
+            return
         self.col = empty((B, m, n, Z))
         self.col2 = self.col.reshape(Bmn, Z)
         self.y_mnL = empty((Bmn, L))
         self.y = empty((B, L, m, n))
         act = self.y
-        nelem = lambda a: int(np.prod(a.shape))  # noqa: E731
         st = []
         s = stream
         gemm_bytes = 4 * (Bmn * Z + L * Z + Bmn * L)      # the three conv products touch the same three matrices
@@ -257,6 +275,69 @@ class LayerOnGpu(object):
                             lambda: K.sum_keepdims(self.gpre, (0, 2, 3), out=self.gbias, stream=s), 4 * ny, "hbm"))
             ex.append(Stage("loss_sum", "sum_rkr_kernel",
                             lambda: K.sum_keepdims(self.act, (0, 1, 2, 3), out=self.loss, stream=s), 4 * ny, "hbm"))
+
+    def _direct_stages(self, K, cfg, nelem):
+        """The same layer without a column buffer: pad -> GEMM over the padded image -> NCHW,
+        pool both ways, pad of the cotangent -> data-gradient GEMM -> NCHW, weight-gradient GEMM.
+        Every stage is one kernel (plus the GEMM's own reduce kernel)."""
+        from cgt_amd import capi
+        from cgt_amd.gpuarray import empty, to_gpu
+        lib = capi.lib()
+        d = self.dims
+        B, C, H, W, L, r, c, Bmn, Z = d["B"], d["C"], d["H"], d["W"], d["L"], d["r"], d["c"], d["Bmn"], d["Z"]
+        s = self.stream
+        self.xpad = empty((K.conv_same_padded_size(B * C, H, W, (r, c)),))
+        self.gypad = empty((K.conv_same_padded_size(B * L, H, W, (r, c)),))
+        self.rows = empty((max(lib.cgt_amd_conv_same_rows_size(B, H, W, L, r, c), lib.cgt_amd_conv_same_rows_size(B, H, W, C, r, c)),))
+        self.fk, self.fflip, self.gfk = empty((L, r * c, C)), empty((C, r * c, L)), empty((L, r, c, C))
+        self.y, self.gx, self.gf = empty((B, L, H, W)), empty(self.x.shape), empty(self.f.shape)
+
+        def call(fn, *a):
+            capi.check(fn(*a))
+        gemm_flops = 2 * Bmn * L * Z
+        gemm_bytes = 4 * (nelem(self.x) + L * Z + Bmn * L)       # image + filters + result: no column buffer
+        st = []
+        st.append(Stage("pad_x", "pad_planes_kernel", lambda: K.conv_same_pad(self.x, (r, c), out=self.xpad, stream=s),
+                        4 * (nelem(self.x) + nelem(self.xpad)), "hbm"))
+        st.append(Stage("filter_fwd", "batched_transpose_kernel",
+                        lambda: call(lib.cgt_amd_conv_same_filter_f32, self.f.ptr, L, C, r, c, 0, self.fk.ptr, s), 8 * L * Z, "hbm"))
+        st.append(Stage("gemm_fwd", "sgemm_kernel", lambda: call(lib.cgt_amd_conv_same_rows_f32, self.xpad.ptr, self.fk.ptr, B, C, H, W, L, r, c, self.rows.ptr, s),
+                        gemm_flops, "mfma", gemm_bytes))
+        st.append(Stage("rows_to_nchw_y", "rows_to_nchw_kernel",
+                        lambda: call(lib.cgt_amd_conv_same_rows_to_nchw_f32, self.rows.ptr, None, 0, B, L, H, W, r, c, self.y.ptr, s),
+                        8 * nelem(self.y), "hbm"))
+        act = self.y
+        if cfg["pool"]:
+            pk, pp, ps = cfg["pool"]
+            PH, PW = K.pool_outsize(H, pk[0], pp[0], ps[0]), K.pool_outsize(W, pk[1], pp[1], ps[1])
+            self.pool, self.mask = empty((B, L, PH, PW)), empty((B, L, PH, PW), np.int32)
+            self.gpool = to_gpu(np.ones((B, L, PH, PW), np.float32))
+            self.gact = empty(self.y.shape)
+            st.append(Stage("max_pool_fwd", "max_pool_fwd_kernel", lambda: K.max_pool(act, pk, pp, ps, out=(self.pool, self.mask), stream=s),
+                            4 * (nelem(self.y) + 2 * nelem(self.pool)), "hbm"))
+            st.append(Stage("max_pool_bwd", "max_pool_bwd_block_kernel",
+                            lambda: K.max_pool_pullback(self.y.shape, self.mask, self.gpool, pk, pp, ps, out=self.gact, stream=s),
+                            4 * (2 * nelem(self.pool) + nelem(self.y)), "hbm"))
+            gy = self.gact
+        else:
+            gy = to_gpu(np.ones(self.y.shape, np.float32))
+        self.gy = gy
+        st.append(Stage("pad_gy", "pad_planes_kernel", lambda: K.conv_same_pad(self.gy, (r, c), out=self.gypad, stream=s),
+                        4 * (nelem(self.y) + nelem(self.gypad)), "hbm"))
+        st.append(Stage("filter_flip", "flip_filters_kernel",
+                        lambda: call(lib.cgt_amd_conv_same_filter_f32, self.f.ptr, L, C, r, c, 1, self.fflip.ptr, s), 8 * L * Z, "hbm"))
+        st.append(Stage("gemm_dgrad", "sgemm_kernel", lambda: call(lib.cgt_amd_conv_same_rows_f32, self.gypad.ptr, self.fflip.ptr, B, L, H, W, C, r, c, self.rows.ptr, s),
+                        gemm_flops, "mfma", gemm_bytes))
+        st.append(Stage("rows_to_nchw_gx", "rows_to_nchw_kernel",
+                        lambda: call(lib.cgt_amd_conv_same_rows_to_nchw_f32, self.rows.ptr, None, 0, B, C, H, W, r, c, self.gx.ptr, s),
+                        8 * nelem(self.x), "hbm"))
+        st.append(Stage("gemm_wgrad", "sgemm_kernel", lambda: call(lib.cgt_amd_conv_same_wgrad_f32, self.gypad.ptr, self.xpad.ptr, B, C, H, W, L, r, c, self.gfk.ptr, s),
+                        gemm_flops, "mfma", gemm_bytes))
+        st.append(Stage("filter_grad_layout", "batched_transpose_kernel",
+                        lambda: K.transpose4(self.gfk, (0, 3, 1, 2), out=self.gf, stream=s), 8 * L * Z, "hbm"))
+        self.stages = st
+        self.conv_flops = 6 * Bmn * L * Z
+        self.extra_stages = []
 
     def step(self):
         from cgt_amd import capi
@@ -475,8 +556,9 @@ def measure(workload, args, primary):
         layer = GemmOnGpu()
         parity = {"ok": True, "skipped": True} if args.no_check else check_gemm_against_oracle()
     else:
-        cfg = WORKLOADS[workload]
-        layer = LayerOnGpu(cfg, overlap=primary and args.overlap and not args.no_overlap, glue=primary and args.glue)
+        cfg = WORKLOADS[workload[:-len(IM2COL_SUFFIX)] if workload.endswith(IM2COL_SUFFIX) else workload]
+        layer = LayerOnGpu(cfg, overlap=primary and args.overlap and not args.no_overlap, glue=primary and args.glue,
+                           algo="im2col" if workload.endswith(IM2COL_SUFFIX) else args.conv_algo)
         parity = {"ok": True, "skipped": True} if args.no_check else check_against_oracle(cfg)
 
     for _ in range(args.warmup):
@@ -541,13 +623,18 @@ def measure(workload, args, primary):
                             "bytes": st.work, "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4)})
     gemm_tf = gemm_flops / (gemm_ms * 1e-3) / 1e12
     value = layer.conv_flops / (ms_per_step * 1e-3) / 1e12
-    traffic = traffic_from_profiles(workload).get(dominant.name)
+    mfma_stages = [st.name for st in layer.stages if st.bound == "mfma"]
+    algo = getattr(layer, "algo", None)
+    traffic = traffic_from_profiles(workload, algo, mfma_stages).get(dominant.name)
     config = {"workload": workload, "x": list(cfg["x"]), "filters": list(cfg["f"]),
               "pad": list(cfg["pad"]), "stride": list(cfg["stride"]),
               "value_is": "conv GEMM flops (6*B*m*n*L*Z) / whole step time incl. im2col, col2im, "
                           "transposes, pool and LRN stages",
               "schedule": ("one stream" if not getattr(layer, "overlap", False) else
                            "weight-gradient GEMM on a second stream beside col2im")}
+    if algo:
+        config["conv_algo"] = ("fused ops, no column buffer (pad -> GEMM over the padded image -> NCHW)" if algo == "direct"
+                               else "im2col -> Mul22 -> transpose; transpose -> Mul22 -> col2im, Mul22")
     if is_gemm:
         config["value_is"] = "flops of Mul22 4096^3 x {NN,NT,TN,TT} + BatchedMul22 64x512^3 / step time"
     elif cfg.get("lrn"):
@@ -567,7 +654,7 @@ def measure(workload, args, primary):
                      "avg_launch_ms_back_to_back": None if dominant.ms is None else round(dominant.ms, 4),
                      "traffic": traffic,
                      "traffic_source": None if traffic is None else
-                     "profiles/%s_pmc_{FETCH,WRITE}_SIZE.txt, calibrated" % PROFILE_PREFIX[workload]},
+                     "profiles/%s_pmc_{FETCH,WRITE}_SIZE.txt, calibrated" % profile_prefix(workload, algo)},
         "gemm_all_launches": {"TFLOPs": round(gemm_tf, 2), "frac": round(gemm_tf / FP32_MFMA_PEAK_TFLOPS, 4)},
         "stages": stages,
         "glue_stages": glue_stages,
@@ -597,6 +684,9 @@ def main():
     ap.add_argument("--no-op-api", action="store_true", help="skip timing the same step through the Op API")
     ap.add_argument("--no-check", action="store_true",
                     help="skip the parity gate (profiling runs: keeps its small launches out of the kernel statistics)")
+    ap.add_argument("--conv-algo", default="auto", choices=["auto", "im2col"],
+                    help="auto: the fused convolution ops where they apply (what nn.conv2d builds); im2col: always the "
+                         "im2col -> Mul22 composition")
     ap.add_argument("--only", action="store_true",
                     help="measure --workload alone (profiling runs); by default the headline workload is followed by "
                          "the other configurations, reported under `workloads`")

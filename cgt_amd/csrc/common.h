@@ -27,7 +27,7 @@ void release_stream_workspaces(void* stream);
 
 // GEMM over an operand read straight from a zero-padded image (gemm.hip): the products of
 // a stride-1 convolution with pad = (kernel - 1) / 2, without a column buffer.
-//   mode 1: rows[B * tpi * 128][N] = sum over (tap, c) of img[b][c][q + tapoff] * Wk[n][tap*C + c]
+//   mode 1: rows[B * tpi * 128][N] = sum over (c, tap) of img[b][c][q + tapoff] * Wk[n][c/16][tap][c%16]
 //           (q = row within the image's tpi * 128 rows of the padded grid)
 //   mode 2: out[M][taps * C] = sum over (b, q) of A[b][m][q] * img[b][c][q + tapoff]
 struct ConvGemm {

@@ -9,7 +9,7 @@
 // "tap (ho, wo) of pixel q" is the plain offset q + ho * Wp + wo: every operand tile is a
 // contiguous run per channel, loaded straight into LDS like any GEMM tile.
 //
-//   forward        rows[b][q][l]   = sum_{tap,c} xpad[b][c][q + tapoff] * f[l][c][tap]
+//   forward        rows[b][q][l]   = sum_{c,tap} xpad[b][c][q + tapoff] * f[l][c][tap]
 //   data gradient  rows[b][q][c]   = sum_{tap,l} gypad[b][l][q + tapoff] * f[l][c][flipped tap]
 //   weight grad    gf[l][tap][c]   = sum_{b,q}   gypad[b][l][q + center] * xpad[b][c][q + tapoff]
 // (the padding columns of gypad are zero, so the junk positions of q contribute nothing).
@@ -125,18 +125,21 @@ __global__ __launch_bounds__(256) void rows_to_nchw_kernel(const float* __restri
     }
 }
 
-// filters [L][C][kh][kw] -> [C][(kh-1-ho, kw-1-wo) taps][L]: the filter bank of the data
-// gradient seen as a forward convolution of the cotangent
+// filters [L][C][kh][kw] -> [C][L/16][(kh-1-ho, kw-1-wo) taps][16]: the filter bank of the
+// data gradient seen as a forward convolution of the cotangent (L channels in, C filters),
+// in the K order of the product (block of 16 channels, tap, channel in the block)
 __global__ __launch_bounds__(256) void flip_filters_kernel(const float* __restrict__ f, float* __restrict__ out,
                                                            int L, int C, int kh, int kw) {
     const int taps = kh * kw;
     const long total = (long)L * C * taps;
     for (long o = (long)blockIdx.x * 256 + threadIdx.x; o < total; o += (long)gridDim.x * 256) {
-        const int l = (int)(o % L);
-        const long r = o / L;
-        const int tap = (int)(r % taps), c = (int)(r / taps);
+        const int li = (int)(o % 16);
+        long r = o / 16;
+        const int tap = (int)(r % taps);
+        r /= taps;
+        const int lb = (int)(r % (L / 16)), c = (int)(r / (L / 16));
         const int ho = tap / kw, wo = tap - ho * kw;
-        out[o] = f[(((long)l * C + c) * kh + (kh - 1 - ho)) * kw + (kw - 1 - wo)];
+        out[o] = f[(((long)(lb * 16 + li) * C + c) * kh + (kh - 1 - ho)) * kw + (kw - 1 - wo)];
     }
 }
 
@@ -200,8 +203,9 @@ CGT_API int cgt_amd_conv_same_pad_f32(const float* x, long planes, long H, long 
 CGT_API int cgt_amd_conv_same_filter_f32(const float* f, long L, long C, int kh, int kw, int flipped, float* fk,
                                          void* stream) {
     CGT_ARG_CHECK(L > 0 && C > 0 && kh > 0 && kw > 0 && f && fk, "conv_same_filter: bad arguments");
-    if (!flipped) {     // [L][C][kh][kw] -> [L][tap][C]: the K axis of the product is (tap, channel)
-        const long fs[4] = {L, C, kh, kw};
+    CGT_ARG_CHECK(C % 16 == 0 && L % 16 == 0, "conv_same_filter: channel and filter counts must be multiples of 16");
+    if (!flipped) {     // [L][C/16][16][taps] -> [L][C/16][taps][16]: the K order of the product
+        const long fs[4] = {L * (C / 16), 16, kh, kw};
         const int ax[4] = {0, 2, 3, 1};
         return cgt_amd_transpose4_f32(f, fs, ax, fk, stream);
     }

@@ -99,14 +99,16 @@ struct GemmArgs {
     int main_wgs, tail_splits, tail_kchunk;
     int wide;          // a leading dimension too large for 32-bit tile offsets: tested loads everywhere
     // Implicit convolution (stride 1, pad = (kernel-1)/2): an operand is read straight
-    // from the zero-padded image [B][C][plane] instead of a column buffer.  The K axis
-    // is ordered (tap, channel), so a slice of 16 is one tap and 16 consecutive channels.
+    // from the zero-padded image [B][C][plane] instead of a column buffer.
     //   mode 1 (forward / data gradient): A[row][k] = img[b][c][q + tapoff], rows are the
-    //     pixels q = h*Wp + w of the padded grid, cv_tpi tiles of rows per image;
+    //     pixels q = h*Wp + w of the padded grid, cv_tpi tiles of rows per image; the K axis
+    //     is ordered (block of 16 channels, tap, channel in the block): a slice of 16 is one
+    //     tap of one channel block, and the taps of a block follow each other, so the
+    //     block's pixels (16 KB per tile) are fetched once and re-read from cache;
     //   mode 2 (weight gradient): the K axis runs over those pixels, cv_spi slices per
     //     image; A[l][q] and B[tap*C + c][q] are both q-contiguous.
     int conv;
-    int cv_wp, cv_kw, cv_cpb, cv_tpi, cv_spi, cv_c;   // padded width, kernel width, C/16, tiles / slices per image, C
+    int cv_wp, cv_kw, cv_kh, cv_tpi, cv_spi, cv_c;    // padded width, kernel, tiles / slices per image, C
     long cv_plane, cv_imgA, cv_imgB;                  // plane stride and per-image strides (floats)
 };
 
@@ -371,16 +373,15 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
     // of scalar adds and compares per slice (everything here is wave-uniform).
     const char* cvA = nullptr;
     const char* cvB = nullptr;
-    int cv_i = 0, cv_j = 0;        // mode 1: channel block, kernel column; mode 2: slice within the image
+    int cv_i = 0, cv_j = 0;        // mode 1: kernel row, kernel column; mode 2: slice within the image
     if constexpr (CONV == 1) {
-        const int s0 = kbeg / KT;
-        const int tap = s0 / a.cv_cpb;
-        cv_i = s0 - tap * a.cv_cpb;
-        const int ho = tap / a.cv_kw;
-        cv_j = tap - ho * a.cv_kw;
+        const int s0 = kbeg / KT, taps = a.cv_kh * a.cv_kw;
+        const int cb = s0 / taps, tap = s0 - cb * taps;
+        cv_i = tap / a.cv_kw;
+        cv_j = tap - cv_i * a.cv_kw;
         const int img = tm / a.cv_tpi, t = tm - img * a.cv_tpi;
-        cvA = reinterpret_cast<const char*>(A + (long)img * a.cv_imgA + (long)t * BM + (long)ho * a.cv_wp + cv_j +
-                                            (long)cv_i * KT * a.cv_plane);
+        cvA = reinterpret_cast<const char*>(A + (long)img * a.cv_imgA + (long)t * BM + (long)cv_i * a.cv_wp + cv_j +
+                                            (long)cb * KT * a.cv_plane);
     } else if constexpr (CONV == 2) {
         const int s0 = kbeg / KT;
         const int img = s0 / a.cv_spi;
@@ -397,13 +398,13 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
             oa = cvA;
             ob = originB;
             originB += stepB;
-            cvA += (long)KT * a.cv_plane * 4;
-            if (++cv_i == a.cv_cpb) {             // next tap: back to channel 0, one pixel to the right
-                cv_i = 0;
-                cvA += 4 - (long)a.cv_cpb * KT * a.cv_plane * 4;
-                if (++cv_j == a.cv_kw) {          // next kernel row
-                    cv_j = 0;
-                    cvA += (long)(a.cv_wp - a.cv_kw) * 4;
+            cvA += 4;                             // next tap: one pixel to the right
+            if (++cv_j == a.cv_kw) {              // next kernel row
+                cv_j = 0;
+                cvA += (long)(a.cv_wp - a.cv_kw) * 4;
+                if (++cv_i == a.cv_kh) {          // next block of 16 channels, back to the first tap
+                    cv_i = 0;
+                    cvA += ((long)KT * a.cv_plane - (long)a.cv_kh * a.cv_wp) * 4;
                 }
             }
         } else if constexpr (CONV == 2) {
@@ -920,7 +921,7 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     GemmArgs a;
     a.conv = cv ? cv->mode : 0;
     if (cv) {
-        a.cv_wp = cv->wp; a.cv_kw = cv->kw; a.cv_cpb = (int)(cv->C / KT); a.cv_c = (int)cv->C;
+        a.cv_wp = cv->wp; a.cv_kw = cv->kw; a.cv_kh = cv->kh; a.cv_c = (int)cv->C;
         a.cv_tpi = (int)cv->tpi; a.cv_spi = (int)cv->spi;
         a.cv_plane = cv->plane;
         // mode 1: A is the image; mode 2: A is the (shifted) padded cotangent with M planes per image, B the image

@@ -326,9 +326,11 @@ int cgt_amd_conv_same_fwd_f32(const float *xpad, const float *f, const float *bi
 
 /* The pieces the three products are made of, one kernel each (plus the GEMM's
  * own reduce kernel), for a host that keeps the intermediate buffers itself:
- *   filter   f [L,C,kh,kw] -> fk: [L][tap][C] (flipped = 0: forward) or
- *            [C][flipped tap][L] (flipped = 1: the data gradient's filter bank)
- *   rows     rows[b][q][n] = sum_{tap,c} imgpad[b][c][q + tapoff] * fk[n][tap][c],
+ *   filter   f [L,C,kh,kw] -> fk in the K order of the product (block of 16
+ *            channels, tap, channel in the block): [L][C/16][tap][16] (flipped = 0:
+ *            forward) or [C][L/16][flipped tap][16] (flipped = 1: the data
+ *            gradient's filter bank)
+ *   rows     rows[b][q][n] = sum_{c,tap} imgpad[b][c][q + tapoff] * fk[n][c/16][tap][c%16],
  *            q = h*(W+2pw) + w, cgt_amd_conv_same_rows_size floats (each image's
  *            rows are rounded up to whole tiles of 128)
  *   rows_to_nchw   rows -> out [B,N,H,W] (+ bias, rectify)

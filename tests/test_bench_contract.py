@@ -25,8 +25,10 @@ def test_more_than_one_gpu_is_refused():
 def _traffic_by_hand(workload, stage):
     """2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE megabytes of the stage's sgemm launch and the reduce
     kernel behind it, read from the summaries with nothing but string splitting."""
-    prefix = {"vgg_mid_conv3x3_128x56x56_b64": "vgg_mid_conv3x3_b64"}[workload]
-    nth = ["gemm_fwd_NT", "gemm_dgrad_NN", "gemm_wgrad_TN"].index(stage)
+    prefix = {"vgg_mid_conv3x3_128x56x56_b64": "vgg_mid_conv3x3_b64",
+              "vgg_mid_conv3x3_128x56x56_b64/im2col": "vgg_mid_conv3x3_b64_im2col"}[workload]
+    nth = [["gemm_fwd", "gemm_dgrad", "gemm_wgrad"], ["gemm_fwd_NT", "gemm_dgrad_NN", "gemm_wgrad_TN"]][
+        workload.endswith("/im2col")].index(stage)
     total = 0.0
     for counter, factor in (("FETCH_SIZE", 2.0), ("WRITE_SIZE", 1.0)):
         lines = open(os.path.join(ROOT, "profiles", "%s_pmc_%s.txt" % (prefix, counter))).read().splitlines()
@@ -47,12 +49,19 @@ def _traffic_by_hand(workload, stage):
 
 def test_traffic_is_read_from_the_profile_summaries():
     import bench
-    t = bench.traffic_from_profiles("vgg_mid_conv3x3_128x56x56_b64")
+    w = "vgg_mid_conv3x3_128x56x56_b64"
+    t = bench.traffic_from_profiles(w + "/im2col", "im2col")
     assert set(t) == {"gemm_fwd_NT", "gemm_dgrad_NN", "gemm_wgrad_TN"}
     for stage, v in t.items():
-        assert v == _traffic_by_hand("vgg_mid_conv3x3_128x56x56_b64", stage)
-        assert 1.0e9 < v < 1.3e9          # 1028 MB algorithmic per product of the VGG layer
-    assert bench.traffic_from_profiles("mnist_conv3x3_1x28x28_b64") == {}
+        assert v == _traffic_by_hand(w + "/im2col", stage)
+        assert 1.0e9 < v < 1.3e9          # 1028 MB algorithmic per product with a column buffer
+    # the fused ops read the image, not a column buffer: 206 MB algorithmic per product
+    t = bench.traffic_from_profiles(w, "direct", ["gemm_fwd", "gemm_dgrad", "gemm_wgrad"])
+    assert set(t) == {"gemm_fwd", "gemm_dgrad", "gemm_wgrad"}
+    for stage, v in t.items():
+        assert v == _traffic_by_hand(w, stage)
+        assert 2.0e8 < v < 5.0e8
+    assert bench.traffic_from_profiles("mnist_conv3x3_1x28x28_b64", "im2col") == {}
 
 
 @pytest.mark.gpu
@@ -81,10 +90,14 @@ def test_default_workload_prints_the_contract_line():
     # the traffic figure is what the committed counter summaries say, not a constant
     import bench
     assert roof["traffic"] == _traffic_by_hand(out["config"]["workload"], roof["stage"])
-    assert roof["traffic"] == bench.traffic_from_profiles(out["config"]["workload"])[roof["stage"]]
+    assert roof["traffic"] == bench.traffic_from_profiles(out["config"]["workload"], "direct",
+                                                          ["gemm_fwd", "gemm_dgrad", "gemm_wgrad"])[roof["stage"]]
+    assert "no column buffer" in out["config"]["conv_algo"]
     # the other configurations ride along: AlexNet conv1 (LRN both ways, k = 2), the raw products,
     # and the first layers whose GEMMs are priced against both roofs
     w = out["workloads"]
+    assert "im2col" in w["vgg_mid_conv3x3_128x56x56_b64/im2col"]["config"]["conv_algo"]
+    assert [r["stage"] for r in w["vgg_mid_conv3x3_128x56x56_b64/im2col"]["stages"]][:2] == ["im2col", "gemm_fwd_NT"]
     alex = w["alexnet_conv1_11x11s4_3x227x227_b128"]
     assert alex["config"]["lrn"]["k"] == 2.0
     names = [r["stage"] for r in alex["stages"]]

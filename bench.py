@@ -277,9 +277,9 @@ class LayerOnGpu(object):
                             lambda: K.sum_keepdims(self.act, (0, 1, 2, 3), out=self.loss, stream=s), 4 * ny, "hbm"))
 
     def _direct_stages(self, K, cfg, nelem):
-        """The same layer without a column buffer: pad -> GEMM over the padded image -> NCHW,
-        pool both ways, pad of the cotangent -> data-gradient GEMM -> NCHW, weight-gradient GEMM.
-        Every stage is one kernel (plus the GEMM's own reduce kernel)."""
+        """The same layer without a column buffer: pad -> GEMM over the padded image (writes
+        NCHW itself), pool both ways, pad of the cotangent -> data-gradient GEMM, weight-gradient
+        GEMM.  Every stage is one kernel (plus the weight gradient's split-K reduce kernel)."""
         from cgt_amd import capi
         from cgt_amd.gpuarray import empty, to_gpu
         lib = capi.lib()
@@ -288,7 +288,6 @@ class LayerOnGpu(object):
         s = self.stream
         self.xpad = empty((K.conv_same_padded_size(B * C, H, W, (r, c)),))
         self.gypad = empty((K.conv_same_padded_size(B * L, H, W, (r, c)),))
-        self.rows = empty((max(lib.cgt_amd_conv_same_rows_size(B, H, W, L, r, c), lib.cgt_amd_conv_same_rows_size(B, H, W, C, r, c)),))
         self.fk, self.fflip, self.gfk = empty((L, r * c, C)), empty((C, r * c, L)), empty((L, r, c, C))
         self.y, self.gx, self.gf = empty((B, L, H, W)), empty(self.x.shape), empty(self.f.shape)
 
@@ -301,11 +300,9 @@ class LayerOnGpu(object):
                         4 * (nelem(self.x) + nelem(self.xpad)), "hbm"))
         st.append(Stage("filter_fwd", "batched_transpose_kernel",
                         lambda: call(lib.cgt_amd_conv_same_filter_f32, self.f.ptr, L, C, r, c, 0, self.fk.ptr, s), 8 * L * Z, "hbm"))
-        st.append(Stage("gemm_fwd", "sgemm_kernel", lambda: call(lib.cgt_amd_conv_same_rows_f32, self.xpad.ptr, self.fk.ptr, B, C, H, W, L, r, c, self.rows.ptr, s),
+        st.append(Stage("gemm_fwd", "sgemm_kernel",
+                        lambda: call(lib.cgt_amd_conv_same_product_f32, self.xpad.ptr, self.fk.ptr, None, 0, B, C, H, W, L, r, c, self.y.ptr, s),
                         gemm_flops, "mfma", gemm_bytes))
-        st.append(Stage("rows_to_nchw_y", "rows_to_nchw_kernel",
-                        lambda: call(lib.cgt_amd_conv_same_rows_to_nchw_f32, self.rows.ptr, None, 0, B, L, H, W, r, c, self.y.ptr, s),
-                        8 * nelem(self.y), "hbm"))
         act = self.y
         if cfg["pool"]:
             pk, pp, ps = cfg["pool"]
@@ -326,11 +323,9 @@ class LayerOnGpu(object):
                         4 * (nelem(self.y) + nelem(self.gypad)), "hbm"))
         st.append(Stage("filter_flip", "flip_filters_kernel",
                         lambda: call(lib.cgt_amd_conv_same_filter_f32, self.f.ptr, L, C, r, c, 1, self.fflip.ptr, s), 8 * L * Z, "hbm"))
-        st.append(Stage("gemm_dgrad", "sgemm_kernel", lambda: call(lib.cgt_amd_conv_same_rows_f32, self.gypad.ptr, self.fflip.ptr, B, L, H, W, C, r, c, self.rows.ptr, s),
+        st.append(Stage("gemm_dgrad", "sgemm_kernel",
+                        lambda: call(lib.cgt_amd_conv_same_product_f32, self.gypad.ptr, self.fflip.ptr, None, 0, B, L, H, W, C, r, c, self.gx.ptr, s),
                         gemm_flops, "mfma", gemm_bytes))
-        st.append(Stage("rows_to_nchw_gx", "rows_to_nchw_kernel",
-                        lambda: call(lib.cgt_amd_conv_same_rows_to_nchw_f32, self.rows.ptr, None, 0, B, C, H, W, r, c, self.gx.ptr, s),
-                        8 * nelem(self.x), "hbm"))
         st.append(Stage("gemm_wgrad", "sgemm_kernel", lambda: call(lib.cgt_amd_conv_same_wgrad_f32, self.gypad.ptr, self.xpad.ptr, B, C, H, W, L, r, c, self.gfk.ptr, s),
                         gemm_flops, "mfma", gemm_bytes))
         st.append(Stage("filter_grad_layout", "batched_transpose_kernel",

@@ -21,23 +21,26 @@ inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 // stream -- it is retired and released with the stream (cgt_amd_stream_destroy).
 // Growth while the stream is being captured is refused (an allocation would break the
 // capture): returns nullptr with the message set.
-enum WorkspaceUser { kWsGemm = 0, kWsSum = 1, kWsConvRows = 2, kWsConvFilter = 3, kWsUsers = 4 };
+enum WorkspaceUser { kWsGemm = 0, kWsSum = 1, kWsConvFilter = 2, kWsUsers = 3 };
 float* stream_workspace(void* stream, WorkspaceUser user, size_t bytes, const char* what);
 void release_stream_workspaces(void* stream);
 
 // GEMM over an operand read straight from a zero-padded image (gemm.hip): the products of
 // a stride-1 convolution with pad = (kernel - 1) / 2, without a column buffer.
-//   mode 1: rows[B * tpi * 128][N] = sum over (c, tap) of img[b][c][q + tapoff] * Wk[n][c/16][tap][c%16]
-//           (q = row within the image's tpi * 128 rows of the padded grid)
 //   mode 2: out[M][taps * C] = sum over (b, q) of A[b][m][q] * img[b][c][q + tapoff]
+//   mode 3: out[b][m][h][w] = sum over (c, tap) of Wk[m][c/16][tap][c%16] * img[b][c][q + tapoff] (+ bias[m], rectify),
+//           q = h*Wp + w: the pixels of the padded grid are the columns, tpi tiles of 128 per image
 struct ConvGemm {
     int mode;
     long B, C, plane;      // images, channels of `img`, floats per padded plane
     int wp, kh, kw;        // padded width, kernel
-    long tpi, spi;         // mode 1: row tiles (of 128) per image; mode 2: K slices (of 16) per image
+    long tpi, spi;         // mode 3: pixel tiles (of 128) per image; mode 2: K slices (of 16) per image
+    long H, W;             // mode 3: image extents
+    const float* bias;     // mode 3: per-output-channel bias or null
+    int relu;              // mode 3: x * (x >= 0) on the way out
 };
 int sgemm_conv(const ConvGemm& cv, long M, long N, const float* A, const float* B, float* C, long ldc, void* stream);
-// 1 if sgemm_conv has a tile shape for these extents (mode 1: N filters; mode 2: M filters, C channels)
+// 1 if sgemm_conv has a tile shape for these extents (output channels of the product, channels of the image)
 bool sgemm_conv_supported(int mode, long filters, long channels);
 
 constexpr int kWave = 64;    // CDNA wavefront width

@@ -4,13 +4,13 @@
 //
 // Padded layout: [B * C planes][plane floats] + a zeroed tail, plane = (H + 2p)(W + 2q)
 // rounded up past 16 zero floats; pixel (h, w) of a plane sits at (h + p) * Wp + (w + q).
-// A row of the forward GEMM is a pixel of the padded grid, q = h * Wp + w (the Wp - W
-// positions at the end of each grid row are junk rows that nobody reads back), so that
+// A column of the forward GEMM is a pixel of the padded grid, q = h * Wp + w (the Wp - W
+// positions at the end of each grid row are junk columns that are never stored), so that
 // "tap (ho, wo) of pixel q" is the plain offset q + ho * Wp + wo: every operand tile is a
 // contiguous run per channel, loaded straight into LDS like any GEMM tile.
 //
-//   forward        rows[b][q][l]   = sum_{c,tap} xpad[b][c][q + tapoff] * f[l][c][tap]
-//   data gradient  rows[b][q][c]   = sum_{tap,l} gypad[b][l][q + tapoff] * f[l][c][flipped tap]
+//   forward        y[b][l][q]      = sum_{c,tap} f[l][c][tap] * xpad[b][c][q + tapoff]
+//   data gradient  gx[b][c][q]     = sum_{l,tap} f[l][c][flipped tap] * gypad[b][l][q + tapoff]
 //   weight grad    gf[l][tap][c]   = sum_{b,q}   gypad[b][l][q + center] * xpad[b][c][q + tapoff]
 // (the padding columns of gypad are zero, so the junk positions of q contribute nothing).
 #include "common.h"
@@ -69,62 +69,6 @@ __global__ __launch_bounds__(256) void pad_planes_kernel(const float* __restrict
     }
 }
 
-// rows [B][rows_per_image][L] (row q = h * Wp + w) -> out [B][L][H][W] (+ optional
-// per-channel bias and ReLU, applied as x * (x >= 0)).  A workgroup takes 64 consecutive
-// output positions of one image and all L channels: the rows it needs are one contiguous
-// block of the input (64 positions + the junk rows between them), copied to LDS with
-// 16-byte loads; each channel then leaves as a run of 64 floats.
-constexpr int kR2NPos = 64;
-__global__ __launch_bounds__(256) void rows_to_nchw_kernel(const float* __restrict__ rows, float* __restrict__ out,
-                                                           const float* __restrict__ bias, int relu,
-                                                           int HW, int W, int Wp, int L, long rows_per_image,
-                                                           int tiles, int npos) {
-    extern __shared__ float tile[];          // [max_rows][L | 1]
-    const int LD = L | 1;
-    const int bid = blockIdx.x;
-    const int b = bid / tiles, t = bid - b * tiles;
-    const int p0 = t * npos;
-    const int np = min(npos, HW - p0);
-    const int h0 = p0 / W, w0 = p0 - h0 * W;
-    const int q0 = h0 * Wp + w0;
-    const int pl = p0 + np - 1, hl = pl / W;
-    const int q1 = hl * Wp + (pl - hl * W);          // last row needed
-    const int nrows = q1 - q0 + 1;                   // <= max_rows
-    const float* blk = rows + ((long)b * rows_per_image + q0) * L;
-    const int n = nrows * L;                          // L % 4 == 0
-    const float rL = 1.0f / (float)L;
-    for (int i0 = threadIdx.x * 4; i0 < n; i0 += 1024 * 4) {
-        v4f v[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const v4f*>(blk + min(i0 + u * 1024, n - 4));
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int i = i0 + u * 1024;
-            if (i < n) {
-                int r = (int)((float)i * rL);
-                int c = i - r * L;
-                if (c < 0) { --r; c += L; }
-                if (c >= L) { ++r; c -= L; }
-                float* d = tile + r * LD + c;
-                d[0] = v[u].x; d[1] = v[u].y; d[2] = v[u].z; d[3] = v[u].w;
-            }
-        }
-    }
-    __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    if (lane < np) {
-        const int p = p0 + lane, h = p / W, w = p - h * W;
-        const int r = h * Wp + w - q0;
-        float* dst = out + (long)b * L * HW + p;
-        for (int c = wave; c < L; c += 4) {
-            float v = tile[r * LD + c];
-            if (bias) v += bias[c];
-            if (relu) v = v * (v >= 0.0f ? 1.0f : 0.0f);
-            dst[(long)c * HW] = v;
-        }
-    }
-}
-
 // filters [L][C][kh][kw] -> [C][L/16][(kh-1-ho, kw-1-wo) taps][16]: the filter bank of the
 // data gradient seen as a forward convolution of the cotangent (L channels in, C filters),
 // in the K order of the product (block of 16 channels, tap, channel in the block)
@@ -143,22 +87,6 @@ __global__ __launch_bounds__(256) void flip_filters_kernel(const float* __restri
     }
 }
 
-static int rows_to_nchw(const SameGeom& g, const float* rows, long Lout, const float* bias, int relu, float* out,
-                        hipStream_t st) {
-    const long HW = g.H * g.W;
-    // positions per workgroup: 64, fewer for narrow images whose junk rows would not fit LDS
-    int npos = kR2NPos;
-    auto rows_needed = [&](int n) { return std::min((long)n + (n / g.W + 2) * (g.Wp - g.W), g.H * g.Wp); };
-    while (npos > 1 && rows_needed(npos) * (Lout | 1) * (long)sizeof(float) > 48 * 1024) npos /= 2;
-    const size_t lds = (size_t)rows_needed(npos) * (Lout | 1) * sizeof(float);
-    const long tiles = cdiv(HW, (long)npos);
-    CGT_ARG_CHECK(lds <= 64 * 1024 && g.B * tiles < (1L << 31), "conv_same: output tile does not fit LDS");
-    rows_to_nchw_kernel<<<dim3((unsigned)(g.B * tiles)), dim3(256), lds, st>>>(
-        rows, out, bias, relu, (int)HW, (int)g.W, (int)g.Wp, (int)Lout, g.tpi * 128, (int)tiles, npos);
-    CGT_LAUNCH_CHECK("rows_to_nchw_kernel");
-    return CGT_AMD_OK;
-}
-
 static int check_same(const char* what, SameGeom& g, long B, long C, long H, long W, long L, int kh, int kw) {
     CGT_ARG_CHECK(B >= 0 && C > 0 && H > 0 && W > 0 && L > 0, "%s: bad shape", what);
     CGT_ARG_CHECK(make_geom(g, B, C, H, W, L, kh, kw), "%s: the kernel must be odd x odd (pad = (kernel - 1) / 2)", what);
@@ -172,9 +100,8 @@ using namespace cgt_amd;
 
 CGT_API int cgt_amd_conv_same_supported(long C, long L, int kh, int kw, int ph, int pw, int sh, int sw) {
     if (sh != 1 || sw != 1 || kh % 2 == 0 || kw % 2 == 0 || ph != (kh - 1) / 2 || pw != (kw - 1) / 2) return 0;
-    if (L > 128 || L % 4 != 0 || C > 128 || C % 4 != 0) return 0;   // rows -> NCHW keeps all channels of 64 pixels in LDS
     // forward: C channels in, L filters; data gradient: L channels in, C "filters"; weight gradient: both
-    return sgemm_conv_supported(1, L, C) && sgemm_conv_supported(1, C, L) && sgemm_conv_supported(2, L, C) ? 1 : 0;
+    return sgemm_conv_supported(3, L, C) && sgemm_conv_supported(3, C, L) && sgemm_conv_supported(2, L, C) ? 1 : 0;
 }
 
 CGT_API long cgt_amd_conv_same_padded_size(long planes, long H, long W, int kh, int kw) {
@@ -216,32 +143,17 @@ CGT_API int cgt_amd_conv_same_filter_f32(const float* f, long L, long C, int kh,
     return CGT_AMD_OK;
 }
 
-CGT_API long cgt_amd_conv_same_rows_size(long B, long H, long W, long N, int kh, int kw) {
+// out [B,N,H,W] = conv of the padded image with fk (+ bias, rectify), written in place by the GEMM
+CGT_API int cgt_amd_conv_same_product_f32(const float* imgpad, const float* fk, const float* bias, int relu, long B,
+                                          long Cin, long H, long W, long N, int kh, int kw, float* out, void* stream) {
     SameGeom g;
-    if (B < 0 || N <= 0 || H <= 0 || W <= 0 || !make_geom(g, B, 1, H, W, N, kh, kw)) return -1;
-    return B * g.tpi * 128 * N;
-}
-
-CGT_API int cgt_amd_conv_same_rows_f32(const float* imgpad, const float* fk, long B, long Cin, long H, long W,
-                                       long N, int kh, int kw, float* rows, void* stream) {
-    SameGeom g;
-    int rc = check_same("conv_same_rows", g, B, Cin, H, W, N, kh, kw);
+    int rc = check_same("conv_same_product", g, B, Cin, H, W, N, kh, kw);
     if (rc) return rc;
     if (B == 0) return CGT_AMD_OK;
-    CGT_ARG_CHECK(imgpad && fk && rows, "conv_same_rows: null pointer");
-    CGT_ARG_CHECK(sgemm_conv_supported(1, N, Cin), "conv_same_rows: unsupported extents (%ld channels, %ld filters)", Cin, N);
-    ConvGemm cv = {1, B, Cin, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi};
-    return sgemm_conv(cv, B * g.tpi * 128, N, imgpad, fk, rows, N, stream);
-}
-
-CGT_API int cgt_amd_conv_same_rows_to_nchw_f32(const float* rows, const float* bias, int relu, long B, long N,
-                                               long H, long W, int kh, int kw, float* out, void* stream) {
-    SameGeom g;
-    int rc = check_same("conv_same_rows_to_nchw", g, B, 1, H, W, N, kh, kw);
-    if (rc) return rc;
-    if (B == 0) return CGT_AMD_OK;
-    CGT_ARG_CHECK(rows && out && N % 4 == 0 && N <= 128, "conv_same_rows_to_nchw: bad arguments");
-    return rows_to_nchw(g, rows, N, bias, relu, out, as_stream(stream));
+    CGT_ARG_CHECK(imgpad && fk && out, "conv_same_product: null pointer");
+    CGT_ARG_CHECK(sgemm_conv_supported(3, N, Cin), "conv_same_product: unsupported extents (%ld channels, %ld filters)", Cin, N);
+    ConvGemm cv = {3, B, Cin, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi, H, W, bias, relu};
+    return sgemm_conv(cv, N, B * g.tpi * 128, fk, imgpad, out, H * W, stream);
 }
 
 CGT_API int cgt_amd_conv_same_wgrad_f32(const float* gypad, const float* xpad, long B, long C, long H, long W,
@@ -255,7 +167,7 @@ CGT_API int cgt_amd_conv_same_wgrad_f32(const float* gypad, const float* xpad, l
     CGT_ARG_CHECK(gypad && xpad, "conv_same_wgrad: null pointer");
     CGT_ARG_CHECK(sgemm_conv_supported(2, L, C), "conv_same_wgrad: unsupported extents (%ld channels, %ld filters)", C, L);
     // pixel q of the padded grid <-> cotangent at q + (ph * Wp + pw): its padding is zero, so junk pixels add nothing
-    ConvGemm cv = {2, B, C, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi};
+    ConvGemm cv = {2, B, C, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi, H, W, nullptr, 0};
     return sgemm_conv(cv, L, taps * C, gypad + g.ph * g.Wp + g.pw, xpad, gfk, taps * C, stream);
 }
 
@@ -271,11 +183,9 @@ CGT_API int cgt_amd_conv_same_fwd_f32(const float* xpad, const float* f, const f
     CGT_ARG_CHECK(cgt_amd_conv_same_supported(C, L, kh, kw, g.ph, g.pw, 1, 1), "conv_same_fwd: unsupported extents C=%ld L=%ld", C, L);
     const long taps = (long)kh * kw;
     float* wk = stream_workspace(stream, kWsConvFilter, (size_t)L * C * taps * sizeof(float), "conv_same_fwd");
-    float* rows = stream_workspace(stream, kWsConvRows, (size_t)B * g.tpi * 128 * std::max(L, C) * sizeof(float), "conv_same_fwd");
-    if (!wk || !rows) return CGT_AMD_ERR_NOMEM;
+    if (!wk) return CGT_AMD_ERR_NOMEM;
     if ((rc = cgt_amd_conv_same_filter_f32(f, L, C, kh, kw, 0, wk, stream))) return rc;
-    if ((rc = cgt_amd_conv_same_rows_f32(xpad, wk, B, C, H, W, L, kh, kw, rows, stream))) return rc;
-    return rows_to_nchw(g, rows, L, bias, relu, y, as_stream(stream));
+    return cgt_amd_conv_same_product_f32(xpad, wk, bias, relu, B, C, H, W, L, kh, kw, y, stream);
 }
 
 CGT_API int cgt_amd_conv_same_bwd_data_f32(const float* gypad, const float* f, long B, long C, long H, long W, long L,
@@ -288,12 +198,10 @@ CGT_API int cgt_amd_conv_same_bwd_data_f32(const float* gypad, const float* f, l
     CGT_ARG_CHECK(cgt_amd_conv_same_supported(C, L, kh, kw, g.ph, g.pw, 1, 1), "conv_same_bwd_data: unsupported extents C=%ld L=%ld", C, L);
     const long taps = (long)kh * kw;
     float* wk = stream_workspace(stream, kWsConvFilter, (size_t)L * C * taps * sizeof(float), "conv_same_bwd_data");
-    float* rows = stream_workspace(stream, kWsConvRows, (size_t)B * g.tpi * 128 * std::max(L, C) * sizeof(float), "conv_same_bwd_data");
-    if (!wk || !rows) return CGT_AMD_ERR_NOMEM;
-    // a forward convolution of the cotangent: L channels in, C "filters" [C][flipped tap][L]
+    if (!wk) return CGT_AMD_ERR_NOMEM;
+    // a forward convolution of the cotangent: L channels in, C "filters" [C][L/16][flipped tap][16]
     if ((rc = cgt_amd_conv_same_filter_f32(f, L, C, kh, kw, 1, wk, stream))) return rc;
-    if ((rc = cgt_amd_conv_same_rows_f32(gypad, wk, B, L, H, W, C, kh, kw, rows, stream))) return rc;
-    return rows_to_nchw(g, rows, C, nullptr, 0, gx, as_stream(stream));
+    return cgt_amd_conv_same_product_f32(gypad, wk, nullptr, 0, B, L, H, W, C, kh, kw, gx, stream);
 }
 
 CGT_API int cgt_amd_conv_same_bwd_filter_f32(const float* gypad, const float* xpad, long B, long C, long H, long W,

@@ -100,15 +100,19 @@ struct GemmArgs {
     int wide;          // a leading dimension too large for 32-bit tile offsets: tested loads everywhere
     // Implicit convolution (stride 1, pad = (kernel-1)/2): an operand is read straight
     // from the zero-padded image [B][C][plane] instead of a column buffer.
-    //   mode 1 (forward / data gradient): A[row][k] = img[b][c][q + tapoff], rows are the
-    //     pixels q = h*Wp + w of the padded grid, cv_tpi tiles of rows per image; the K axis
-    //     is ordered (block of 16 channels, tap, channel in the block): a slice of 16 is one
-    //     tap of one channel block, and the taps of a block follow each other, so the
-    //     block's pixels (16 KB per tile) are fetched once and re-read from cache;
+    //   mode 3 (forward / data gradient): C[n][q] = sum_k Wk[n][k] * img[b][c][q + tapoff]:
+    //     the columns are the pixels q = h*Wp + w of the padded grid, cv_tpi tiles of 128
+    //     columns per image, and the result is written straight into NCHW (junk pixels
+    //     skipped) with an optional per-row bias and x * (x >= 0).  The K axis is ordered
+    //     (block of 16 channels, tap, channel in the block): a slice of 16 is one tap of one
+    //     channel block, and the taps of a block follow each other, so the block's pixels
+    //     (16 KB per tile) are fetched once and re-read from cache;
     //   mode 2 (weight gradient): the K axis runs over those pixels, cv_spi slices per
     //     image; A[l][q] and B[tap*C + c][q] are both q-contiguous.
     int conv;
     int cv_wp, cv_kw, cv_kh, cv_tpi, cv_spi, cv_c;    // padded width, kernel, tiles / slices per image, C
+    int cv_h, cv_w, cv_relu;                          // mode 3: image extents, rectify flag
+    const float* cv_bias;                             // mode 3: per-row (output channel) bias or null
     long cv_plane, cv_imgA, cv_imgB;                  // plane stride and per-image strides (floats)
 };
 
@@ -254,8 +258,9 @@ __device__ __forceinline__ int xcd_remap(int id, int n) {
 template <bool AKC, bool BKC, bool PIPE, int WGM, int WGN, int TM, int TN, bool DEEP = false, int CONV = 0>
 __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmArgs a) {
     static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
-    static_assert(CONV == 0 || (!PIPE && !DEEP && BKC && AKC == (CONV == 2)),
-                  "implicit convolution: plain loop; mode 1 reads A row-contiguous, mode 2 k-contiguous");
+    static_assert(CONV == 0 || ((CONV == 2 || CONV == 3) && !PIPE && !DEEP && AKC && BKC == (CONV == 2)),
+                  "implicit convolution: plain loop; the image operand is B, row-contiguous in mode 3; "
+                  "both operands k-contiguous in mode 2");
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
     typedef OperandTile<AKC, BM> TileA;
     typedef OperandTile<BKC, BN> TileB;
@@ -373,14 +378,14 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
     // of scalar adds and compares per slice (everything here is wave-uniform).
     const char* cvA = nullptr;
     const char* cvB = nullptr;
-    int cv_i = 0, cv_j = 0;        // mode 1: kernel row, kernel column; mode 2: slice within the image
-    if constexpr (CONV == 1) {
+    int cv_i = 0, cv_j = 0;        // mode 3: kernel row, kernel column; mode 2: slice within the image
+    if constexpr (CONV == 3) {
         const int s0 = kbeg / KT, taps = a.cv_kh * a.cv_kw;
         const int cb = s0 / taps, tap = s0 - cb * taps;
         cv_i = tap / a.cv_kw;
         cv_j = tap - cv_i * a.cv_kw;
-        const int img = tm / a.cv_tpi, t = tm - img * a.cv_tpi;
-        cvA = reinterpret_cast<const char*>(A + (long)img * a.cv_imgA + (long)t * BM + (long)cv_i * a.cv_wp + cv_j +
+        const int img = tn / a.cv_tpi, t = tn - img * a.cv_tpi;
+        cvB = reinterpret_cast<const char*>(B + (long)img * a.cv_imgB + (long)t * BN + (long)cv_i * a.cv_wp + cv_j +
                                             (long)cb * KT * a.cv_plane);
     } else if constexpr (CONV == 2) {
         const int s0 = kbeg / KT;
@@ -394,17 +399,17 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
     }
     // origins of the next slice to be issued, then step to the one after it
     auto conv_next = [&](const char*& oa, const char*& ob) {
-        if constexpr (CONV == 1) {
-            oa = cvA;
-            ob = originB;
-            originB += stepB;
-            cvA += 4;                             // next tap: one pixel to the right
-            if (++cv_j == a.cv_kw) {              // next kernel row
+        if constexpr (CONV == 3) {
+            oa = originA;
+            ob = cvB;
+            originA += stepA;
+            cvB += 4;
+            if (++cv_j == a.cv_kw) {
                 cv_j = 0;
-                cvA += (long)(a.cv_wp - a.cv_kw) * 4;
-                if (++cv_i == a.cv_kh) {          // next block of 16 channels, back to the first tap
+                cvB += (long)(a.cv_wp - a.cv_kw) * 4;
+                if (++cv_i == a.cv_kh) {
                     cv_i = 0;
-                    cvA += ((long)KT * a.cv_plane - (long)a.cv_kh * a.cv_wp) * 4;
+                    cvB += ((long)KT * a.cv_plane - (long)a.cv_kh * a.cv_wp) * 4;
                 }
             }
         } else if constexpr (CONV == 2) {
@@ -596,8 +601,8 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
             }
         }
     };
-    if (wholeA) ta.init_offsets(CONV != 0 ? a.cv_plane : a.lda);
-    if (wholeB) tb.init_offsets(CONV == 2 ? a.cv_plane : a.ldb);
+    if (wholeA) ta.init_offsets(CONV == 2 ? a.cv_plane : a.lda);
+    if (wholeB) tb.init_offsets(CONV == 2 || CONV == 3 ? a.cv_plane : a.ldb);
     if constexpr (CONV != 0) {
         main_loop(std::integral_constant<int, kFast>{});      // the host sends whole tiles and whole slices only
     } else {
@@ -606,6 +611,40 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
     }
 
     // accumulator element e of a 32x32 block: row 8*(e/4) + 4*half + e%4, column l32.
+    if (CONV == 3 && tail_piece < 0) {
+        // Rows are output channels, columns pixels of the padded grid: the tile goes straight
+        // into out[image][channel][h][w].  A lane's column is the same for every row, so its
+        // offset inside a channel plane (and whether its pixel is a junk position) is worked
+        // out once per 32-column block; row origins are wave-uniform as in the plain epilogue.
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+        const int wm_u = wave_u / WGN, wn_u = wave_u % WGN;
+        const int img = tn / a.cv_tpi, t = tn - img * a.cv_tpi;
+        const long HW = (long)a.cv_h * a.cv_w;
+        const int r0 = m0 + wm_u * TM * 32;
+        char* base = reinterpret_cast<char*>(a.C + ((long)img * a.M + r0) * HW);
+        const long step1 = HW * 4, step5 = HW * 20;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int q = t * BN + (wn_u * TN + j) * 32 + l32;
+            const int h = q / a.cv_wp, w = q - h * a.cv_wp;
+            if (h < a.cv_h && w < a.cv_w) {
+                unsigned lane_off = (unsigned)((4 * half * HW + (long)h * a.cv_w + w) * 4);
+                char* row = base;
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        asm volatile("" : "+v"(lane_off));
+                        float v = acc[i][j][e];
+                        if (a.cv_bias) v += a.cv_bias[r0 + i * 32 + 8 * (e / 4) + (e % 4) + 4 * half];
+                        if (a.cv_relu) v = v * (v >= 0.0f ? 1.0f : 0.0f);
+                        *reinterpret_cast<float*>(row + lane_off) = v;
+                        row += (e % 4 == 3) ? step5 : step1;
+                    }
+            }
+        }
+        return;
+    }
     // Destination: C, this split's partial matrix, or (tail pieces) a tile-local
     // [BM][BN] block that is written whole -- the reduction clips.
     float* out;
@@ -697,6 +736,50 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restric
 #pragma unroll
     for (int j = 0; j < 4; ++j)
         if (n0 + c + j < a.N) dst[j] = o[j];
+}
+
+// The same for a mode-3 convolution product: tile rows are output channels, tile columns
+// pixels of the padded grid; the sums go to out[image][channel][h][w], junk pixels dropped,
+// with the optional bias and rectify of the in-place epilogue.
+__global__ __launch_bounds__(256) void tail_reduce_conv_kernel(const float* __restrict__ ws, GemmArgs a, int bm, int bn) {
+    const int lid = a.main_wgs + blockIdx.y;
+    constexpr int GM = 8;
+    const int per_group = GM * a.tiles_n;
+    const int group = lid / per_group, in_group = lid - group * per_group;
+    const int first_m = group * GM;
+    const int gsz = min(a.tiles_m - first_m, GM);
+    const int tm = first_m + in_group % gsz, tn = in_group / gsz;
+    const int i = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= bm * bn) return;
+    const float* src = ws + (long)blockIdx.y * a.tail_splits * (bm * bn) + i;
+    float4 v[kMaxTailSplits];
+#pragma unroll
+    for (int k = 0; k < kMaxTailSplits; ++k)
+        if (k < a.tail_splits) v[k] = *reinterpret_cast<const float4*>(src + (long)k * (bm * bn));
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int k = 0; k < kMaxTailSplits; ++k)
+        if (k < a.tail_splits) {
+            s.x += v[k].x; s.y += v[k].y; s.z += v[k].z; s.w += v[k].w;
+        }
+    const int r = i / bn, c = i - r * bn;
+    const int row = tm * bm + r;                         // output channel
+    const int img = tn / a.cv_tpi, t = tn - img * a.cv_tpi;
+    const long HW = (long)a.cv_h * a.cv_w;
+    float* dst = a.C + ((long)img * a.M + row) * HW;
+    const float bias = a.cv_bias ? a.cv_bias[row] : 0.0f;
+    const float o[4] = {s.x, s.y, s.z, s.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int q = t * bn + c + j;
+        const int h = q / a.cv_wp, w = q - h * a.cv_wp;
+        if (h < a.cv_h && w < a.cv_w) {
+            float x = o[j];
+            if (a.cv_bias) x += bias;
+            if (a.cv_relu) x = x * (x >= 0.0f ? 1.0f : 0.0f);
+            dst[(long)h * a.cv_w + w] = x;
+        }
+    }
 }
 
 // C[r][c] = sum over splits of ws[s][r][c].  A workgroup takes 64 columns of
@@ -825,14 +908,13 @@ static void launch_shape(int shape, dim3 grid, hipStream_t st, const GemmArgs& a
     }
 }
 
-// implicit-convolution variants: 128-row tiles, N tile of 128 / 64 / 32
+// implicit-convolution variants
 static void launch_conv(int mode, int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
     dim3 block(kGemmThreads);
-    if (mode == 1) {
+    if (mode == 3) {
         switch (shape) {
-            case 0: sgemm_kernel<false, true, false, 2, 2, 2, 2, false, 1><<<grid, block, 0, st>>>(a); break;
-            case 2: sgemm_kernel<false, true, false, 4, 1, 1, 2, false, 1><<<grid, block, 0, st>>>(a); break;
-            default: sgemm_kernel<false, true, false, 4, 1, 1, 1, false, 1><<<grid, block, 0, st>>>(a); break;
+            case 0: sgemm_kernel<true, false, false, 2, 2, 2, 2, false, 3><<<grid, block, 0, st>>>(a); break;
+            default: sgemm_kernel<true, false, false, 1, 4, 2, 1, false, 3><<<grid, block, 0, st>>>(a); break;   // 64 x 128
         }
     } else {
         switch (shape) {
@@ -844,11 +926,16 @@ static void launch_conv(int mode, int shape, dim3 grid, hipStream_t st, const Ge
 }
 
 // tile shape (index into kShapes) of an implicit-convolution product, -1 if none fits:
-// tiles must be whole -- 128 rows, and an N tile that divides the filter count (mode 1) or
-// the channel count, so that a tile of the (tap, channel) axis lies in one tap (mode 2)
+// tiles must be whole -- mode 3: 128 (or one tile of 64) output channels x 128 pixels;
+// mode 2: 128 filters x an N tile that divides the channel count, so that a tile of the
+// (tap, channel) axis lies in one tap
 static int conv_shape(int mode, long filters, long channels) {
-    const long n = mode == 1 ? filters : channels;
-    if (mode == 2 && filters % 128 != 0) return -1;
+    if (mode == 3) {        // rows = filters: 128-row tiles, or one 64-row tile; 128 pixels per tile
+        if (channels % KT != 0) return -1;
+        return filters % 128 == 0 ? 0 : (filters == 64 ? 5 : -1);
+    }
+    const long n = channels;
+    if (filters % 128 != 0) return -1;
     if (channels % KT != 0) return -1;
     if (n % 128 == 0) return 0;
     if (n == 64) return 2;
@@ -914,7 +1001,8 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
         return p;
     };
     if (cv) {
-        shape = conv_shape(cv->mode, cv->mode == 1 ? N : M, cv->C);
+        shape = conv_shape(cv->mode, M, cv->C);
+        CGT_ARG_CHECK(cv->mode != 3 || (long)cv->tpi * cv->B * 128 == N, "sgemm_conv: mode 3 takes whole tiles of pixels");
         CGT_ARG_CHECK(shape >= 0, "sgemm_conv: no tile shape for these extents");
         CGT_ARG_CHECK(cv->plane < (1L << 24), "sgemm_conv: padded plane too large");
     }
@@ -924,9 +1012,10 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
         a.cv_wp = cv->wp; a.cv_kw = cv->kw; a.cv_kh = cv->kh; a.cv_c = (int)cv->C;
         a.cv_tpi = (int)cv->tpi; a.cv_spi = (int)cv->spi;
         a.cv_plane = cv->plane;
-        // mode 1: A is the image; mode 2: A is the (shifted) padded cotangent with M planes per image, B the image
-        a.cv_imgA = (cv->mode == 1 ? cv->C : M) * cv->plane;
+        // mode 2: A is the (shifted) padded cotangent with M planes per image; B is the image in both modes
+        a.cv_imgA = M * cv->plane;
         a.cv_imgB = cv->C * cv->plane;
+        a.cv_h = (int)cv->H; a.cv_w = (int)cv->W; a.cv_relu = cv->relu; a.cv_bias = cv->bias;
     }
     a.A = A; a.B = B; a.C = C;
     a.lda = lda; a.ldb = ldb; a.ldc = ldc;
@@ -940,7 +1029,7 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     a.kchunk = (int)(cdiv(std::max(K, 1L), KT) * KT);
     a.ws = nullptr;
     a.wide = (!cv && (lda >= (1L << 23) || ldb >= (1L << 23))) ? 1 : 0;
-    if (P == 1 && tiles < 512 && K >= 64 * KT) {
+    if (P == 1 && tiles < 512 && K >= 64 * KT && !(cv && cv->mode == 3)) {
         long want = std::max(1L, 1024 / tiles);
         want = std::min(want, K / (8 * KT));                    // at least 8 slices per split
         const long cap = (256L << 20) / (M * N * (long)sizeof(float));  // workspace <= 256 MiB
@@ -1006,6 +1095,10 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
         if (vec) splitk_reduce_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a.ws, C, MN, (int)N, ldc, a.splits);
         else splitk_reduce_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a.ws, C, MN, (int)N, ldc, a.splits);
         CGT_LAUNCH_CHECK("splitk_reduce_kernel");
+    } else if (tail_tiles > 0 && cv && cv->mode == 3) {
+        tail_reduce_conv_kernel<<<dim3((unsigned)cdiv(kShapes[shape].bm * kShapes[shape].bn, 1024), (unsigned)tail_tiles), dim3(256), 0, st>>>(
+            a.ws, a, kShapes[shape].bm, kShapes[shape].bn);
+        CGT_LAUNCH_CHECK("tail_reduce_conv_kernel");
     } else if (tail_tiles > 0) {
         tail_reduce_kernel<<<dim3((unsigned)cdiv(kShapes[shape].bm * kShapes[shape].bn, 1024), (unsigned)tail_tiles), dim3(256), 0, st>>>(
             a.ws, C, a, kShapes[shape].bm, kShapes[shape].bn);
@@ -1017,8 +1110,8 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
 int sgemm_conv(const ConvGemm& cv, long M, long N, const float* A, const float* B, float* C, long ldc,
                void* stream) {
     const long taps = (long)cv.kh * cv.kw;
-    if (cv.mode == 1)   // A = image (row-contiguous operand), B = filters [N][taps * C]
-        return gemm_dispatch(1, 1, 1, M, N, taps * cv.C, A, M, 0, B, taps * cv.C, 0, C, ldc, 0, stream, false, &cv);
+    if (cv.mode == 3)   // A = filters [M][taps * C], B = image (row-contiguous operand); C is NCHW, written by the kernel
+        return gemm_dispatch(0, 0, 1, M, N, taps * cv.C, A, taps * cv.C, 0, B, N, 0, C, N, 0, stream, false, &cv);
     // A = cotangent planes [B][M][plane], B = image; K runs over (image, pixel slice)
     return gemm_dispatch(0, 1, 1, M, N, cv.B * cv.spi * KT, A, cv.plane, 0, B, cv.plane, 0, C, ldc, 0, stream, false, &cv);
 }

@@ -304,8 +304,8 @@ int cgt_amd_sgemm_batched(int tA, int tB, long P, long M, long N, long K,
  * elsewhere, plus a zeroed tail; cgt_amd_conv_same_pad_f32 writes all of it. */
 
 /* 1 if the three entry points below cover this layer: stride 1, odd kernel,
- * pad = (kernel - 1) / 2, C and L in {32, 64, 128}, L = 128 for the weight
- * gradient's tiles.  Otherwise use im2col + cgt_amd_sgemm + col2im. */
+ * pad = (kernel - 1) / 2, L a multiple of 128, C a multiple of 128 or 64
+ * (whole GEMM tiles).  Otherwise use im2col + cgt_amd_sgemm + col2im. */
 int cgt_amd_conv_same_supported(long C, long L, int kh, int kw, int ph, int pw, int sh, int sw);
 
 /* Floats in the padded copy of `planes` planes of H x W (tail included); -1 on bad arguments. */
@@ -330,19 +330,15 @@ int cgt_amd_conv_same_fwd_f32(const float *xpad, const float *f, const float *bi
  *            channels, tap, channel in the block): [L][C/16][tap][16] (flipped = 0:
  *            forward) or [C][L/16][flipped tap][16] (flipped = 1: the data
  *            gradient's filter bank)
- *   rows     rows[b][q][n] = sum_{c,tap} imgpad[b][c][q + tapoff] * fk[n][c/16][tap][c%16],
- *            q = h*(W+2pw) + w, cgt_amd_conv_same_rows_size floats (each image's
- *            rows are rounded up to whole tiles of 128)
- *   rows_to_nchw   rows -> out [B,N,H,W] (+ bias, rectify)
+ *   product  out [B,N,H,W] = sum_{c,tap} fk[n][c/16][tap][c%16] * imgpad[b][c][q + tapoff]
+ *            (+ bias[n], rectify), written in NCHW by the GEMM itself
  *   wgrad    gfk [L][tap][C] from the two padded arrays; transpose4 {0,3,1,2}
  *            of it viewed [L,kh,kw,C] is gf [L,C,kh,kw] */
 int cgt_amd_conv_same_filter_f32(const float *f, long L, long C, int kh, int kw, int flipped,
                                  float *fk, void *stream);
-long cgt_amd_conv_same_rows_size(long B, long H, long W, long N, int kh, int kw);
-int cgt_amd_conv_same_rows_f32(const float *imgpad, const float *fk, long B, long Cin, long H, long W,
-                               long N, int kh, int kw, float *rows, void *stream);
-int cgt_amd_conv_same_rows_to_nchw_f32(const float *rows, const float *bias, int relu, long B, long N,
-                                       long H, long W, int kh, int kw, float *out, void *stream);
+int cgt_amd_conv_same_product_f32(const float *imgpad, const float *fk, const float *bias, int relu,
+                                  long B, long Cin, long H, long W, long N, int kh, int kw,
+                                  float *out, void *stream);
 int cgt_amd_conv_same_wgrad_f32(const float *gypad, const float *xpad, long B, long C, long H, long W,
                                 long L, int kh, int kw, float *gfk, void *stream);
 

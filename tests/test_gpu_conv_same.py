@@ -42,11 +42,13 @@ def _padded_reference(x, kernel, total):
 
 CASES = [
     # B, C, H, W, L, kernel
-    (2, 32, 9, 11, 128, (3, 3)),
+    (2, 64, 9, 11, 128, (3, 3)),
+    (2, 128, 6, 9, 256, (3, 3)),
+    (1, 256, 5, 5, 128, (3, 3)),
     (3, 128, 14, 14, 128, (3, 3)),
     (2, 64, 7, 20, 128, (5, 5)),
     (1, 128, 56, 56, 128, (3, 3)),
-    (5, 32, 3, 70, 128, (3, 5)),
+    (5, 64, 3, 70, 128, (3, 5)),
     (2, 128, 1, 1, 128, (3, 3)),
 ]
 
@@ -82,10 +84,12 @@ def test_conv_same_forward_and_gradients_vs_oracle(K, B, C, H, W, L, kernel):
     assert y2 is y and np.array_equal(K.conv_same_bwd_filter(gypad, xpad, x.shape, f.shape, out=gf).get(), gf.get())
 
 
-def test_conv_same_fused_bias_and_rectify_match_the_separate_ops(K):
+@pytest.mark.parametrize("B,C,H,W,L", [(3, 64, 10, 13, 128), (11, 64, 56, 56, 128)])
+def test_conv_same_fused_bias_and_rectify_match_the_separate_ops(K, B, C, H, W, L):
+    # the second size has 286 pixel tiles on 256 CUs: its last 30 go through the tail split,
+    # whose reduce kernel applies the bias and the rectify too
     from cgt_amd.gpuarray import to_gpu
     rs = np.random.RandomState(11)
-    B, C, H, W, L = 3, 64, 10, 13, 128
     x = rs.randn(B, C, H, W).astype(np.float32)
     f = (rs.randn(L, C, 3, 3) / 24).astype(np.float32)
     b = rs.randn(L).astype(np.float32)
@@ -97,11 +101,16 @@ def test_conv_same_fused_bias_and_rectify_match_the_separate_ops(K):
     assert np.array_equal(fused.view(np.uint32), want.view(np.uint32))
     only_bias = K.conv_same_fwd(xpad, to_gpu(f), x.shape, bias=to_gpu(b)).get()
     assert np.array_equal(only_bias.view(np.uint32), pre.view(np.uint32))
+    if B > 4:
+        y64 = O.conv2d(x[-1:].astype(np.float64), f.astype(np.float64), (1, 1), (1, 1))
+        assert relfro(plain[-1:], y64) <= TOL
 
 
 def test_conv_same_supported_rule(K):
     assert K.conv_same_supported(128, 128, (3, 3), (1, 1), (1, 1))
-    assert K.conv_same_supported(32, 128, (5, 5), (2, 2), (1, 1))
+    assert K.conv_same_supported(64, 128, (5, 5), (2, 2), (1, 1))
+    assert K.conv_same_supported(256, 512, (3, 3), (1, 1), (1, 1))
+    assert not K.conv_same_supported(32, 128, (5, 5), (2, 2), (1, 1))     # 32 channels: no data-gradient tile
     assert not K.conv_same_supported(3, 96, (11, 11), (0, 0), (4, 4))     # AlexNet conv1: strided
     assert not K.conv_same_supported(3, 32, (5, 5), (2, 2), (1, 1))       # 3 channels: not a multiple of 16
     assert not K.conv_same_supported(128, 128, (3, 3), (0, 0), (1, 1))    # valid padding
@@ -117,8 +126,8 @@ def test_nn_conv2d_takes_the_fused_ops_and_grad_goes_through_them(K):
     from cgt_amd import nn
     from cgt_amd.nn_ops import conv_same
     rs = np.random.RandomState(3)
-    x = rs.randn(3, 32, 12, 10).astype(np.float32)
-    f = (rs.randn(128, 32, 3, 3) / 17).astype(np.float32)
+    x = rs.randn(3, 64, 12, 10).astype(np.float32)
+    f = (rs.randn(128, 64, 3, 3) / 24).astype(np.float32)
 
     def graph(xn, fn):
         y = nn.conv2d(xn, fn, (3, 3), pad=(1, 1))
@@ -150,7 +159,7 @@ def test_nn_conv2d_takes_the_fused_ops_and_grad_goes_through_them(K):
     fun = cgt.function([xn], [y, loss, gx, gf])
     for got, node in zip(fun(x), (y, loss, gx, gf)):
         assert np.array_equal(got.view(np.uint32), node.get().view(np.uint32))
-    x5 = rs.randn(5, 32, 12, 10).astype(np.float32)
+    x5 = rs.randn(5, 64, 12, 10).astype(np.float32)
     fresh = graph(cgt.constant(x5), fn)
     for got, node in zip(fun(x5), fresh):
         assert np.array_equal(got.view(np.uint32), node.get().view(np.uint32))

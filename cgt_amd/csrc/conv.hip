@@ -2,8 +2,11 @@
 // buffer: forward, data gradient and weight gradient as GEMMs whose image operand is read
 // straight from a zero-padded copy of the image (sgemm_conv in gemm.hip).
 //
-// Padded layout: [B * C planes][plane floats] + a zeroed tail, plane = (H + 2p)(W + 2q)
-// rounded up past 16 zero floats; pixel (h, w) of a plane sits at (h + p) * Wp + (w + q).
+// Padded layout: [B * C planes][plane floats] + a zeroed tail.  A plane is q zeros, then
+// H + 2p rows of Wp = W + q floats (W pixels followed by q zeros; the first and last p rows
+// all zero), rounded up past 16 zero floats: pixel (h, w) sits at q + (h + p) * Wp + w.
+// The zeros that end a row are also the left padding of the next one, so a row costs
+// W + q floats, not W + 2q.
 // A column of the forward GEMM is a pixel of the padded grid, q = h * Wp + w (the Wp - W
 // positions at the end of each grid row are junk columns that are never stored), so that
 // "tap (ho, wo) of pixel q" is the plain offset q + ho * Wp + wo: every operand tile is a
@@ -31,8 +34,8 @@ static bool make_geom(SameGeom& g, long B, long C, long H, long W, long L, int k
     if (kh < 1 || kw < 1 || kh % 2 == 0 || kw % 2 == 0) return false;
     g.B = B; g.C = C; g.H = H; g.W = W; g.L = L;
     g.kh = kh; g.kw = kw; g.ph = (kh - 1) / 2; g.pw = (kw - 1) / 2;
-    g.Hp = H + 2 * g.ph; g.Wp = W + 2 * g.pw;
-    g.plane = (g.Hp * g.Wp + 16 + 15) / 16 * 16;
+    g.Hp = H + 2 * g.ph; g.Wp = W + g.pw;
+    g.plane = (g.pw + g.Hp * g.Wp + 16 + 15) / 16 * 16;
     g.tail = (256 + (long)kh * g.Wp + 3) / 4 * 4;
     g.tpi = cdiv(H * g.Wp, 128);
     g.spi = cdiv(H * g.Wp, 16);
@@ -54,14 +57,16 @@ __global__ __launch_bounds__(256) void pad_planes_kernel(const float* __restrict
             const int e0 = (int)(u - pl * units_per_plane) * 4;
             const float* sp = src + pl * (long)H * W;
             // row of e0 by reciprocal multiplication (plane < 2^21 is checked on the host), fixed up exactly
-            int hp = (int)(((float)e0 + 0.5f) * rWp);
-            int wp = e0 - hp * Wp;
+            // element e of a plane is column (e - pw) % Wp of padded row (e - pw) / Wp
+            const int e1 = e0 - pw + Wp;                 // shifted by one row so that it is never negative
+            int hp = (int)(((float)e1 + 0.5f) * rWp);
+            int wp = e1 - hp * Wp;
             if (wp < 0) { --hp; wp += Wp; }
             if (wp >= Wp) { ++hp; wp -= Wp; }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int h = hp - ph, w = wp - pw;
-                if (h >= 0 && h < H && w >= 0 && w < W) o[j] = sp[h * W + w];
+                const int h = hp - 1 - ph;
+                if (h >= 0 && h < H && wp < W) o[j] = sp[h * W + wp];
                 if (++wp == Wp) { wp = 0; ++hp; }
             }
         }

@@ -23,8 +23,9 @@ def info2closure(info):
 def padded_size(planes, H, W, info):
     """Floats in the padded copy of `planes` planes (cgt_amd_conv_same_padded_size), as a
     shape expression."""
-    Hp, Wp = H + 2 * ((info.kernel_h - 1) // 2), W + 2 * ((info.kernel_w - 1) // 2)
-    plane = (Hp * Wp + 16 + 15) // 16 * 16
+    pw = (info.kernel_w - 1) // 2
+    Hp, Wp = H + 2 * ((info.kernel_h - 1) // 2), W + pw
+    plane = (pw + Hp * Wp + 16 + 15) // 16 * 16
     tail = (256 + info.kernel_h * Wp + 3) // 4 * 4
     return planes * plane + tail
 

@@ -300,8 +300,9 @@ int cgt_amd_sgemm_batched(int tA, int tB, long P, long M, long N, long K,
  * bit for bit.
  *
  * Padded layout: `planes` planes of cgt_amd_conv_same_padded_size(1,...) -
- * tail floats each, pixel (h, w) at (h + ph) * (W + 2 pw) + (w + pw), zeros
- * elsewhere, plus a zeroed tail; cgt_amd_conv_same_pad_f32 writes all of it. */
+ * tail floats each, pixel (h, w) at pw + (h + ph) * (W + pw) + w (the pw zeros
+ * that end a row are the left padding of the next one), zeros elsewhere, plus
+ * a zeroed tail; cgt_amd_conv_same_pad_f32 writes all of it. */
 
 /* 1 if the three entry points below cover this layer: stride 1, odd kernel,
  * pad = (kernel - 1) / 2, L a multiple of 128, C a multiple of 128 or 64

@@ -30,13 +30,14 @@ def relfro(a, b):
 def _padded_reference(x, kernel, total):
     B, C, H, W = x.shape
     ph, pw = (kernel[0] - 1) // 2, (kernel[1] - 1) // 2
-    Hp, Wp = H + 2 * ph, W + 2 * pw
-    plane = (Hp * Wp + 16 + 15) // 16 * 16
+    # a plane: pw zeros, then H + 2 ph rows of W + pw floats (W pixels, pw zeros)
+    Hp, Wp = H + 2 * ph, W + pw
+    plane = (pw + Hp * Wp + 16 + 15) // 16 * 16
     ref = np.zeros(total, np.float32)
     body = ref[:B * C * plane].reshape(B * C, plane)
     img = np.zeros((B * C, Hp, Wp), np.float32)
-    img[:, ph:ph + H, pw:pw + W] = x.reshape(B * C, H, W)
-    body[:, :Hp * Wp] = img.reshape(B * C, -1)
+    img[:, ph:ph + H, :W] = x.reshape(B * C, H, W)
+    body[:, pw:pw + Hp * Wp] = img.reshape(B * C, -1)
     return ref
 
 

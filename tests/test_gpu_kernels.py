@@ -164,6 +164,9 @@ POOL_CASES = [
     ((2, 3, 11, 13), (3, 3), (1, 1), (2, 2)),      # compiled-in geometry, odd extents, padding
     ((3, 4, 7, 9), (2, 2), (0, 0), (2, 2)),        # odd width: no paired stores in the pullback
     ((600, 9, 6, 6), (2, 2), (0, 0), (2, 2)),      # many small planes per workgroup
+    ((2, 3, 12, 16), (3, 3), (1, 1), (2, 2)),      # W % 4 == 0: the pullback writes 16-byte rows (overlapping windows, padding)
+    ((3, 5, 4, 4), (2, 2), (0, 0), (2, 2)),        # one 16-byte unit per row
+    ((2, 2, 9, 8), (3, 3), (0, 0), (2, 2)),
 ]
 
 

@@ -187,6 +187,7 @@ class LayerOnGpu(object):
         self.algo = "direct" if algo == "auto" and K.conv_same_supported(C, L, (r, c), pad, stride) else "im2col"
         if self.algo == "direct":
             self.overlap = False
+            self.glue = glue
             self._direct_stages(K, cfg, nelem)
             return
         self.col = empty((B, m, n, Z))
@@ -301,7 +302,7 @@ class LayerOnGpu(object):
         st.append(Stage("filter_fwd", "batched_transpose_kernel",
                         lambda: call(lib.cgt_amd_conv_same_filter_f32, self.f.ptr, L, C, r, c, 0, self.fk.ptr, s), 8 * L * Z, "hbm"))
         st.append(Stage("gemm_fwd", "sgemm_kernel",
-                        lambda: call(lib.cgt_amd_conv_same_product_f32, self.xpad.ptr, self.fk.ptr, None, 0, B, C, H, W, L, r, c, self.y.ptr, s),
+                        lambda: call(lib.cgt_amd_conv_same_product_f32, self.xpad.ptr, self.fk.ptr, None, 0, B, C, H, W, L, r, c, self.y.ptr, None, s),
                         gemm_flops, "mfma", gemm_bytes))
         act = self.y
         if cfg["pool"]:
@@ -324,7 +325,7 @@ class LayerOnGpu(object):
         st.append(Stage("filter_flip", "flip_filters_kernel",
                         lambda: call(lib.cgt_amd_conv_same_filter_f32, self.f.ptr, L, C, r, c, 1, self.fflip.ptr, s), 8 * L * Z, "hbm"))
         st.append(Stage("gemm_dgrad", "sgemm_kernel",
-                        lambda: call(lib.cgt_amd_conv_same_product_f32, self.gypad.ptr, self.fflip.ptr, None, 0, B, L, H, W, C, r, c, self.gx.ptr, s),
+                        lambda: call(lib.cgt_amd_conv_same_product_f32, self.gypad.ptr, self.fflip.ptr, None, 0, B, L, H, W, C, r, c, self.gx.ptr, None, s),
                         gemm_flops, "mfma", gemm_bytes))
         st.append(Stage("gemm_wgrad", "sgemm_kernel", lambda: call(lib.cgt_amd_conv_same_wgrad_f32, self.gypad.ptr, self.xpad.ptr, B, C, H, W, L, r, c, self.gfk.ptr, s),
                         gemm_flops, "mfma", gemm_bytes))
@@ -333,6 +334,29 @@ class LayerOnGpu(object):
         self.stages = st
         self.conv_flops = 6 * Bmn * L * Z
         self.extra_stages = []
+        if self.glue:
+            # bias add + rectify: inside the forward product's epilogue (one launch, the mask of the
+            # rectify's gradient written beside the result) against the separate passes of the unfused graph
+            ex = self.extra_stages
+            ny = nelem(self.y)
+            self.bias = to_gpu(np.zeros((1, L, 1, 1), np.float32))
+            self.zero = to_gpu(np.float32(0).reshape(()))
+            self.bias_full, self.pre, self.act = empty(self.y.shape), empty(self.y.shape), empty(self.y.shape)
+            self.mask_ge = empty(self.y.shape, np.int8)
+            ex.append(Stage("gemm_fwd_bias_relu_fused", "sgemm_kernel",
+                            lambda: call(lib.cgt_amd_conv_same_product_f32, self.xpad.ptr, self.fk.ptr, self.bias.ptr, 1, B, C, H, W, L,
+                                         r, c, self.act.ptr, self.mask_ge.ptr, s), gemm_bytes + ny, "hbm"))
+            ex.append(Stage("gemm_fwd_plain", "sgemm_kernel",
+                            lambda: call(lib.cgt_amd_conv_same_product_f32, self.xpad.ptr, self.fk.ptr, None, 0, B, C, H, W, L,
+                                         r, c, self.y.ptr, None, s), gemm_bytes, "hbm"))
+            ex.append(Stage("repeat_bias", "repeat_rkr_kernel",
+                            lambda: K.repeat(self.bias, (0, 2, 3), (B, H, W), out=self.bias_full, stream=s), 4 * ny, "hbm"))
+            ex.append(Stage("add_bias", "elwise_binary_kernel",
+                            lambda: K.elwise_binary("+", self.y, self.bias_full, out=self.pre, stream=s), 12 * ny, "hbm"))
+            ex.append(Stage("relu_mask_ge", "elwise_binary_kernel",
+                            lambda: K.elwise_binary(">=", self.pre, self.zero, out=self.mask_ge, stream=s), 5 * ny, "hbm"))
+            ex.append(Stage("relu_mul", "elwise_binary_kernel",
+                            lambda: K.elwise_binary("*", self.pre, self.mask_ge, out=self.act, stream=s), 9 * ny, "hbm"))
 
     def step(self):
         from cgt_amd import capi

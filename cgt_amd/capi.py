@@ -63,9 +63,9 @@ PROTOTYPES = {
     "cgt_amd_conv_same_padded_size": (c_long, [c_long, c_long, c_long, c_int, c_int]),
     "cgt_amd_conv_same_pad_f32": (c_int, [c_void_p, c_long, c_long, c_long, c_int, c_int, c_void_p, c_void_p]),
     "cgt_amd_conv_same_filter_f32": (c_int, [c_void_p, c_long, c_long, c_int, c_int, c_int, c_void_p, c_void_p]),
-    "cgt_amd_conv_same_product_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int] + [c_long] * 5 + [c_int, c_int, c_void_p, c_void_p]),
+    "cgt_amd_conv_same_product_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int] + [c_long] * 5 + [c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "cgt_amd_conv_same_wgrad_f32": (c_int, [c_void_p, c_void_p] + [c_long] * 5 + [c_int, c_int, c_void_p, c_void_p]),
-    "cgt_amd_conv_same_fwd_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int] + [c_long] * 5 + [c_int, c_int, c_void_p, c_void_p]),
+    "cgt_amd_conv_same_fwd_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int] + [c_long] * 5 + [c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "cgt_amd_conv_same_bwd_data_f32": (c_int, [c_void_p, c_void_p] + [c_long] * 5 + [c_int, c_int, c_void_p, c_void_p]),
     "cgt_amd_conv_same_bwd_filter_f32": (c_int, [c_void_p, c_void_p] + [c_long] * 5 + [c_int, c_int, c_void_p, c_void_p]),
     "cgt_amd_elwise_unary_f32": (c_int, [c_int, c_long, c_void_p, c_void_p, c_void_p]),

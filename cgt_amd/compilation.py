@@ -223,6 +223,7 @@ def prebuild_standard_ops():
         (core.Transpose((0, 3, 1, 2)), [T4]),
         (nn_ops.conv_same.ConvPad(cinfo), [T4]),
         (nn_ops.conv_same.ConvForward(cinfo), [T4, T1, T4]),
+        (nn_ops.conv_same.ConvForward(cinfo, True, True), [T4, T1, T4, T4]),
         (nn_ops.conv_same.ConvBackwardData(cinfo), [T1, T4, T4]),
         (nn_ops.conv_same.ConvBackwardFilter(cinfo), [T1, T1, T4, T4]),
         (core.Transport("gpu"), [T4]),

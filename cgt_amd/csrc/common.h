@@ -38,6 +38,7 @@ struct ConvGemm {
     long H, W;             // mode 3: image extents
     const float* bias;     // mode 3: per-output-channel bias or null
     int relu;              // mode 3: x * (x >= 0) on the way out
+    signed char* mask;     // mode 3: (x >= 0) as int8, same shape as the output, or null
 };
 int sgemm_conv(const ConvGemm& cv, long M, long N, const float* A, const float* B, float* C, long ldc, void* stream);
 // 1 if sgemm_conv has a tile shape for these extents (output channels of the product, channels of the image)

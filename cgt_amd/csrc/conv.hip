@@ -150,14 +150,15 @@ CGT_API int cgt_amd_conv_same_filter_f32(const float* f, long L, long C, int kh,
 
 // out [B,N,H,W] = conv of the padded image with fk (+ bias, rectify), written in place by the GEMM
 CGT_API int cgt_amd_conv_same_product_f32(const float* imgpad, const float* fk, const float* bias, int relu, long B,
-                                          long Cin, long H, long W, long N, int kh, int kw, float* out, void* stream) {
+                                          long Cin, long H, long W, long N, int kh, int kw, float* out,
+                                          signed char* mask, void* stream) {
     SameGeom g;
     int rc = check_same("conv_same_product", g, B, Cin, H, W, N, kh, kw);
     if (rc) return rc;
     if (B == 0) return CGT_AMD_OK;
     CGT_ARG_CHECK(imgpad && fk && out, "conv_same_product: null pointer");
     CGT_ARG_CHECK(sgemm_conv_supported(3, N, Cin), "conv_same_product: unsupported extents (%ld channels, %ld filters)", Cin, N);
-    ConvGemm cv = {3, B, Cin, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi, H, W, bias, relu};
+    ConvGemm cv = {3, B, Cin, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi, H, W, bias, relu, mask};
     return sgemm_conv(cv, N, B * g.tpi * 128, fk, imgpad, out, H * W, stream);
 }
 
@@ -172,14 +173,15 @@ CGT_API int cgt_amd_conv_same_wgrad_f32(const float* gypad, const float* xpad, l
     CGT_ARG_CHECK(gypad && xpad, "conv_same_wgrad: null pointer");
     CGT_ARG_CHECK(sgemm_conv_supported(2, L, C), "conv_same_wgrad: unsupported extents (%ld channels, %ld filters)", C, L);
     // pixel q of the padded grid <-> cotangent at q + (ph * Wp + pw): its padding is zero, so junk pixels add nothing
-    ConvGemm cv = {2, B, C, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi, H, W, nullptr, 0};
+    ConvGemm cv = {2, B, C, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi, H, W, nullptr, 0, nullptr};
     return sgemm_conv(cv, L, taps * C, gypad + g.ph * g.Wp + g.pw, xpad, gfk, taps * C, stream);
 }
 
 // ---- the three products of a layer, composed from the pieces with library-owned workspaces
 
 CGT_API int cgt_amd_conv_same_fwd_f32(const float* xpad, const float* f, const float* bias, int relu, long B, long C,
-                                      long H, long W, long L, int kh, int kw, float* y, void* stream) {
+                                      long H, long W, long L, int kh, int kw, float* y, signed char* mask,
+                                      void* stream) {
     SameGeom g;
     int rc = check_same("conv_same_fwd", g, B, C, H, W, L, kh, kw);
     if (rc) return rc;
@@ -190,7 +192,7 @@ CGT_API int cgt_amd_conv_same_fwd_f32(const float* xpad, const float* f, const f
     float* wk = stream_workspace(stream, kWsConvFilter, (size_t)L * C * taps * sizeof(float), "conv_same_fwd");
     if (!wk) return CGT_AMD_ERR_NOMEM;
     if ((rc = cgt_amd_conv_same_filter_f32(f, L, C, kh, kw, 0, wk, stream))) return rc;
-    return cgt_amd_conv_same_product_f32(xpad, wk, bias, relu, B, C, H, W, L, kh, kw, y, stream);
+    return cgt_amd_conv_same_product_f32(xpad, wk, bias, relu, B, C, H, W, L, kh, kw, y, mask, stream);
 }
 
 CGT_API int cgt_amd_conv_same_bwd_data_f32(const float* gypad, const float* f, long B, long C, long H, long W, long L,
@@ -206,7 +208,7 @@ CGT_API int cgt_amd_conv_same_bwd_data_f32(const float* gypad, const float* f, l
     if (!wk) return CGT_AMD_ERR_NOMEM;
     // a forward convolution of the cotangent: L channels in, C "filters" [C][L/16][flipped tap][16]
     if ((rc = cgt_amd_conv_same_filter_f32(f, L, C, kh, kw, 1, wk, stream))) return rc;
-    return cgt_amd_conv_same_product_f32(gypad, wk, nullptr, 0, B, L, H, W, C, kh, kw, gx, stream);
+    return cgt_amd_conv_same_product_f32(gypad, wk, nullptr, 0, B, L, H, W, C, kh, kw, gx, nullptr, stream);
 }
 
 CGT_API int cgt_amd_conv_same_bwd_filter_f32(const float* gypad, const float* xpad, long B, long C, long H, long W,

@@ -113,6 +113,7 @@ struct GemmArgs {
     int cv_wp, cv_kw, cv_kh, cv_tpi, cv_spi, cv_c;    // padded width, kernel, tiles / slices per image, C
     int cv_h, cv_w, cv_relu;                          // mode 3: image extents, rectify flag
     const float* cv_bias;                             // mode 3: per-row (output channel) bias or null
+    signed char* cv_mask;                             // mode 3: where (x >= 0) goes as int8, or null
     long cv_plane, cv_imgA, cv_imgB;                  // plane stride and per-image strides (floats)
 };
 
@@ -637,6 +638,8 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                         asm volatile("" : "+v"(lane_off));
                         float v = acc[i][j][e];
                         if (a.cv_bias) v += a.cv_bias[r0 + i * 32 + 8 * (e / 4) + (e % 4) + 4 * half];
+                        if (a.cv_mask)      // same element index as in the float array: byte offset / 4
+                            a.cv_mask[((row - reinterpret_cast<char*>(a.C)) + lane_off) >> 2] = v >= 0.0f ? 1 : 0;
                         if (a.cv_relu) v = v * (v >= 0.0f ? 1.0f : 0.0f);
                         *reinterpret_cast<float*>(row + lane_off) = v;
                         row += (e % 4 == 3) ? step5 : step1;
@@ -776,6 +779,7 @@ __global__ __launch_bounds__(256) void tail_reduce_conv_kernel(const float* __re
         if (h < a.cv_h && w < a.cv_w) {
             float x = o[j];
             if (a.cv_bias) x += bias;
+            if (a.cv_mask) a.cv_mask[(dst - a.C) + (long)h * a.cv_w + w] = x >= 0.0f ? 1 : 0;
             if (a.cv_relu) x = x * (x >= 0.0f ? 1.0f : 0.0f);
             dst[(long)h * a.cv_w + w] = x;
         }
@@ -1015,7 +1019,7 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
         // mode 2: A is the (shifted) padded cotangent with M planes per image; B is the image in both modes
         a.cv_imgA = M * cv->plane;
         a.cv_imgB = cv->C * cv->plane;
-        a.cv_h = (int)cv->H; a.cv_w = (int)cv->W; a.cv_relu = cv->relu; a.cv_bias = cv->bias;
+        a.cv_h = (int)cv->H; a.cv_w = (int)cv->W; a.cv_relu = cv->relu; a.cv_bias = cv->bias; a.cv_mask = cv->mask;
     }
     a.A = A; a.B = B; a.C = C;
     a.lda = lda; a.ldb = ldb; a.ldc = ldc;

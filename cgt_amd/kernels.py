@@ -298,8 +298,9 @@ def conv_same_pad(x, kernel, out=None, stream=None):
     return res
 
 
-def conv_same_fwd(xpad, f, xshape, bias=None, relu=False, out=None, stream=None):
-    """conv2d (stride 1, same padding) from the padded input; optional fused bias add and rectify."""
+def conv_same_fwd(xpad, f, xshape, bias=None, relu=False, out=None, mask=None, stream=None):
+    """conv2d (stride 1, same padding) from the padded input; optional fused bias add and
+    rectify; `mask` (int8 array of the output's shape) receives (pre-activation >= 0)."""
     _f32(xpad, f)
     B, C, H, W = xshape
     L, C2, kh, kw = f.shape
@@ -307,7 +308,7 @@ def conv_same_fwd(xpad, f, xshape, bias=None, relu=False, out=None, stream=None)
         raise ValueError("filter channels %d != input channels %d" % (C2, C))
     y = _out(out, (B, L, H, W))
     capi.check(capi.lib().cgt_amd_conv_same_fwd_f32(xpad.ptr, f.ptr, None if bias is None else bias.ptr, int(bool(relu)),
-                                                    B, C, H, W, L, kh, kw, y.ptr, stream))
+                                                    B, C, H, W, L, kh, kw, y.ptr, None if mask is None else mask.ptr, stream))
     return y
 
 

@@ -44,9 +44,26 @@ def conv2d(x_BKRC, f_LKrc, kernelshape, pad=(0, 0), stride=(1, 1)):
     return col_Bmn_L.reshape([B, m, n, L]).transpose([0, 3, 1, 2])
 
 
+_CONV_FUSION = True
+
+
+def conv_fusion(on=None):
+    """Whether SpatialConvolution's bias add and a rectify that follows a fused convolution
+    go into the convolution's epilogue (default) or stay separate ops.  Returns the
+    previous setting."""
+    global _CONV_FUSION
+    old = _CONV_FUSION
+    if on is not None:
+        _CONV_FUSION = bool(on)
+    return old
+
+
 def rectify(x):
-    """ReLU as the reference builds it: x * (x >= 0) (cgt/nn.py:44-45)."""
+    """ReLU as the reference builds it: x * (x >= 0) (cgt/nn.py:44-45).  On the result of a
+    fused convolution it becomes part of that op (same values, same gradient)."""
     x = core.as_node(x)
+    if _CONV_FUSION and isinstance(x.op, conv_same.ConvForward) and not x.op.relu:
+        return conv_same.rectified(x)
     return x * (x >= 0)
 
 
@@ -70,6 +87,10 @@ class SpatialConvolution(object):
         self.bias = core.constant(b)
 
     def __call__(self, x):
+        x = core.as_node(x)
+        if (_CONV_FUSION and _CONV_ALGO == "auto"
+                and conv_same.supported(x, self.weight, self.kernelshape, self.pad, self.stride)):
+            return conv_same.conv_same(x, self.weight, self.kernelshape, bias=self.bias)
         tmp = conv2d(x, self.weight, self.kernelshape, self.pad, self.stride)
         return core.broadcast("+", tmp, self.bias, "xxxx,1x11")
 

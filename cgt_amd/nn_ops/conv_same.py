@@ -72,49 +72,81 @@ _CHECK_PADDED = r"""
 
 
 class ConvForward(core.Op):
-    """inputs [x, xpad, f] -> y [B,L,H,W].  x gives the shape and receives the gradient;
-    the product reads xpad = ConvPad(x)."""
+    """inputs [x, xpad, f] (+ [bias] when has_bias) -> y [B,L,H,W]; with relu, the tuple
+    (y, mask): y = pre * (pre >= 0) and mask = (pre >= 0) as int8, pre = conv + bias.
+
+    x gives the shape and receives the gradient; the product reads xpad = ConvPad(x).  The
+    bias add and the rectify are the SpatialConvolution bias (cgt/nn.py:231-233) and
+    nn.rectify (cgt/nn.py:44-45) applied in the product's epilogue with the same fp32
+    operations, and the pullback is built from the same ops the unfused graph would use
+    (mask * gy, Sum over (0, 2, 3) for the bias), so values and gradients have the bits of
+    the unfused graph."""
     available_impls = ("native_gpu",)
 
-    def __init__(self, info):
-        self.info = info
+    def __init__(self, info, has_bias=False, relu=False):
+        self.info, self.has_bias, self.relu = info, bool(has_bias), bool(relu)
 
     def get_diff(self, _):
-        return [True, False, True]
+        return [True, False, True] + ([True] if self.has_bias else [])
 
     def shp_apply(self, inputs):
         B, _, H, W = core.shape(inputs[0])
-        return [B, core.size(inputs[2], 0), H, W]
+        shp = [B, core.size(inputs[2], 0), H, W]
+        return (shp, list(shp)) if self.relu else shp
 
     def typ_apply(self, input_types):
-        return core.TensorType("f4", 4)
+        t = core.TensorType("f4", 4)
+        return core.TupleType(t, core.TensorType("i1", 4)) if self.relu else t
 
     def pullback(self, inputs, output, goutput):
-        return self.pullback_wanted(inputs, output, goutput, [True, False, True])
+        return self.pullback_wanted(inputs, output, goutput, self.get_diff(len(inputs)))
 
     def pullback_wanted(self, inputs, output, goutput, wanted):
-        x, xpad, f = inputs
-        gypad = core.Result(ConvPad(self.info), [goutput])
-        gx = core.Result(ConvBackwardData(self.info), [gypad, f, x]) if wanted[0] else None
-        gf = core.Result(ConvBackwardFilter(self.info), [gypad, xpad, f, x]) if wanted[2] else None
-        return [gx, None, gf]
+        x, xpad, f = inputs[:3]
+        if self.relu:
+            _y, mask = core.unpack(output)
+            gy = core.elwise_binary("*", mask, goutput[0])     # what x * (x >= 0) hands back: (x >= 0) * gz
+        else:
+            gy = goutput
+        gbias = None
+        if self.has_bias and wanted[3]:
+            gbias = core.sum(gy, axis=(0, 2, 3), keepdims=True)  # the pullback of the bias' Repeat
+        gx = gf = None
+        if wanted[0] or wanted[2]:
+            gypad = core.Result(ConvPad(self.info), [gy])
+            gx = core.Result(ConvBackwardData(self.info), [gypad, f, x]) if wanted[0] else None
+            gf = core.Result(ConvBackwardFilter(self.info), [gypad, xpad, f, x]) if wanted[2] else None
+        return [gx, None, gf] + ([gbias] if self.has_bias else [])
+
+    def get_closure(self):
+        return info2closure(self.info) + [("has_bias", ctypes.c_int, int(self.has_bias)), ("relu", ctypes.c_int, int(self.relu))]
 
     def get_native_compile_info(self, input_types, devtype):
         assert devtype == "gpu"
-        code = r"""
+        head = (r"""
+            CGT_EXPORT_C void $function($closure* cl, cgtArray** reads, cgtTuple* out) {
+                cgtArray* write = static_cast<cgtArray*>(out->getitem(0));
+                cgtArray* mask = static_cast<cgtArray*>(out->getitem(1));
+                cgt_check(mask->size() == write->size() && mask->dtype() == cgt_i1, "ConvForward: the mask must be an int8 array of the output's shape");
+""" if self.relu else r"""
             CGT_EXPORT_C void $function($closure* cl, cgtArray** reads, cgtArray* write) {
-                cgtArray *x = reads[0], *xpad = reads[1], *f = reads[2];
+                cgtArray* mask = NULL;
+""")
+        code = head + r"""
+                cgtArray *x = reads[0], *xpad = reads[1], *f = reads[2], *bias = cl->has_bias ? reads[3] : NULL;
                 long B = x->shape()[0], C = x->shape()[1], H = x->shape()[2], W = x->shape()[3], L = f->shape()[0];
                 cgt_check(f->ndim() == 4 && f->shape()[1] == C && f->shape()[2] == cl->kernel_h && f->shape()[3] == cl->kernel_w
-                          && write->size() == B * L * H * W, "ConvForward: filters or output do not fit the input");
+                          && write->size() == B * L * H * W && (!bias || bias->size() == L),
+                          "ConvForward: filters, bias or output do not fit the input");
 """ + _CHECK_PADDED % ("B * C", "xpad", "ConvForward", "xpad") + r"""
                 if (cgtGlobalStatus != cgtStatusOK) return;
-                int rc = cgt_amd_conv_same_fwd_f32((const float*)xpad->data(), (const float*)f->data(), NULL, 0,
-                    B, C, H, W, L, cl->kernel_h, cl->kernel_w, (float*)write->data(), cgt_get_stream());
+                int rc = cgt_amd_conv_same_fwd_f32((const float*)xpad->data(), (const float*)f->data(),
+                    bias ? (const float*)bias->data() : NULL, cl->relu, B, C, H, W, L, cl->kernel_h, cl->kernel_w,
+                    (float*)write->data(), mask ? (signed char*)mask->data() : NULL, cgt_get_stream());
                 cgt_check(rc == CGT_AMD_OK, "ConvForward: %s", cgt_amd_last_error());
             }"""
-        return core.NativeCompileInfo(code, includes=["cgt_amd.h"], closure_triples=info2closure(self.info),
-                                      gpu_deref_mask=(False, True, True))
+        return core.NativeCompileInfo(code, includes=["cgt_amd.h"], closure_triples=self.get_closure(),
+                                      gpu_deref_mask=(False, True, True) + ((True,) if self.has_bias else ()))
 
 
 class ConvBackwardData(core.Op):
@@ -185,8 +217,21 @@ def supported(x, f, kernelshape, pad, stride):
     return kernels.conv_same_supported(core.size(x, 1), core.size(f, 0), kernelshape, pad, stride)
 
 
-def conv_same(x, f, kernelshape):
+def conv_same(x, f, kernelshape, bias=None, relu=False):
+    """conv2d (+ per-channel bias [1,L,1,1]) (+ rectify) through the fused ops."""
     x, f = core.as_node(x), core.as_node(f)
     info = ConvSameInfo(int(kernelshape[0]), int(kernelshape[1]))
     xpad = core.Result(ConvPad(info), [x])
-    return core.Result(ConvForward(info), [x, xpad, f])
+    parents = [x, xpad, f] + ([core.as_node(bias)] if bias is not None else [])
+    out = core.Result(ConvForward(info, bias is not None, relu), parents)
+    return out[0] if relu else out
+
+
+def rectified(node):
+    """The rectify of a ConvForward result as ONE fused op: the same inputs run again with
+    the rectify in the epilogue.  Nodes are evaluated as they are built, so this costs a
+    second product while the graph is traced; a compiled function replays only the fused
+    one (the plain result is no longer reachable from the outputs)."""
+    op = node.op
+    assert isinstance(op, ConvForward) and not op.relu
+    return core.Result(ConvForward(op.info, op.has_bias, True), node.parents)[0]

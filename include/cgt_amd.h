@@ -320,10 +320,12 @@ int cgt_amd_conv_same_pad_f32(const float *x, long planes, long H, long W, int k
  * may be NULL) is added per channel and, if relu != 0, the result is replaced by
  * v * (v >= 0) -- the bias add and rectify of SpatialConvolution + nn.rectify
  * (cgt/nn.py:44-45, 231-233) applied while the result is written, with the same
- * fp32 operations as the separate ops.  Uses workspaces owned by the library. */
+ * fp32 operations as the separate ops.  `mask` (int8 [B,L,H,W], may be NULL)
+ * receives (v >= 0) of the value before the rectify: the factor of the
+ * rectify's gradient.  Uses workspaces owned by the library. */
 int cgt_amd_conv_same_fwd_f32(const float *xpad, const float *f, const float *bias, int relu,
                               long B, long C, long H, long W, long L, int kh, int kw,
-                              float *y, void *stream);
+                              float *y, signed char *mask, void *stream);
 
 /* The pieces the three products are made of, one kernel each (plus the GEMM's
  * own reduce kernel), for a host that keeps the intermediate buffers itself:
@@ -339,7 +341,7 @@ int cgt_amd_conv_same_filter_f32(const float *f, long L, long C, int kh, int kw,
                                  float *fk, void *stream);
 int cgt_amd_conv_same_product_f32(const float *imgpad, const float *fk, const float *bias, int relu,
                                   long B, long Cin, long H, long W, long N, int kh, int kw,
-                                  float *out, void *stream);
+                                  float *out, signed char *mask, void *stream);
 int cgt_amd_conv_same_wgrad_f32(const float *gypad, const float *xpad, long B, long C, long H, long W,
                                 long L, int kh, int kw, float *gfk, void *stream);
 

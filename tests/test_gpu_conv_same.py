@@ -166,6 +166,56 @@ def test_nn_conv2d_takes_the_fused_ops_and_grad_goes_through_them(K):
         assert np.array_equal(got.view(np.uint32), node.get().view(np.uint32))
 
 
+def test_spatial_convolution_bias_and_rectify_fused_have_the_bits_of_the_separate_ops(K):
+    # SpatialConvolution's bias add and the nn.rectify behind it go into the product's epilogue;
+    # values, loss and all three gradients are bit-identical to the graph with the separate
+    # Repeat / add / >= / * ops, and the compiled function is shorter
+    import cgt_amd as cgt
+    from cgt_amd import nn
+    from cgt_amd.nn_ops import conv_same
+    rs = np.random.RandomState(8)
+    x = rs.randn(3, 64, 11, 9).astype(np.float32)
+    w = (rs.randn(128, 64, 3, 3) / 24).astype(np.float32)
+    b = (0.3 * rs.randn(1, 128, 1, 1)).astype(np.float32)
+    layer = nn.SpatialConvolution(64, 128, (3, 3), (1, 1), weight_init=w, bias_init=b)
+
+    def graph(xn):
+        act = nn.rectify(layer(xn))
+        pooled = nn.max_pool_2d(act, (2, 2), (0, 0), (2, 2))
+        loss = cgt.sum(pooled * pooled)
+        gx, gw, gb = cgt.grad(loss, [xn, layer.weight, layer.bias])
+        return [act, loss, gx, gw, gb]
+
+    xn = cgt.constant(x)
+    fused = graph(xn)
+    producer = fused[0].parents[0].op                       # act = TupleIndex(0) of the fused op's (y, mask)
+    assert isinstance(producer, conv_same.ConvForward) and producer.relu and producer.has_bias
+    old = nn.conv_fusion(False)
+    try:
+        xu = cgt.constant(x)
+        unfused = graph(xu)
+        assert isinstance(unfused[0].op, cgt.ElwiseBinary)
+    finally:
+        nn.conv_fusion(old)
+    for a, u in zip(fused, unfused):
+        assert np.array_equal(a.get().view(np.uint32), u.get().view(np.uint32))
+    # and against the float64 chain
+    d = np.float64
+    pre = O.conv2d(x.astype(d), w.astype(d), (1, 1), (1, 1)) + b
+    act64 = pre * (pre >= 0)
+    p64, mask = O.max_pool(act64, (2, 2), (0, 0), (2, 2))
+    gpre = O.max_pool_pullback(act64.shape, mask, 2 * p64) * (pre >= 0)
+    gx64, gw64 = O.conv2d_pullback(x.astype(d), w.astype(d), gpre, (1, 1), (1, 1))
+    assert relfro(fused[0].get(), act64) <= TOL and relfro(fused[2].get(), gx64) <= TOL
+    assert relfro(fused[3].get(), gw64) <= TOL and relfro(fused[4].get(), gpre.sum((0, 2, 3), keepdims=True)) <= TOL
+    f_fused, f_unfused = cgt.function([xn], fused), cgt.function([xu], unfused)
+    launches = lambda f: sum(1 for s in f.plan_steps() if s[0] == "byref")      # noqa: E731
+    assert launches(f_fused) <= launches(f_unfused) - 4          # Repeat, +, >=, * are gone
+    x2 = rs.randn(5, 64, 11, 9).astype(np.float32)
+    for a, u in zip(f_fused(x2), f_unfused(x2)):
+        assert np.array_equal(a.view(np.uint32), u.view(np.uint32))
+
+
 def test_vgg_layer_full_size_through_the_fused_ops(K):
     # the headline layer at full size: slices against the float64 oracle, the rest through
     # the adjoint identity <conv(x), gy> = <x, conv^T(gy)> and linearity in the filters

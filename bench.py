@@ -455,6 +455,44 @@ class GemmOnGpu(object):
     time_stages = LayerOnGpu.time_stages
 
 
+def hbm_reference(reps=10):
+    """What plain streaming kernels of this library reach on this box, measured in the same
+    run on arrays (1 GiB each) far larger than the 256 MB last-level cache: a device-to-device
+    copy, a pure write (fill), a pure read (sum) and an elementwise add (two reads, one
+    write).  The HBM-bound stages are priced against the published 8 TB/s; these rows say
+    how much of that a kernel with no index arithmetic at all gets here."""
+    from cgt_amd import capi, kernels as K
+    from cgt_amd.gpuarray import empty
+    n = 1 << 28
+    a, b, c = empty((n,)), empty((n,)), empty((n,))
+    s = capi.Stream()
+    st = s.handle
+    K.fill(1.0, (n,), out=a, stream=st)
+    K.fill(2.0, (n,), out=b, stream=st)
+    lib = capi.lib()
+    small = empty((1,))
+    rows = {}
+
+    def timed(name, fn, nbytes):
+        for _ in range(2):
+            fn()
+        e0, e1 = capi.Event(), capi.Event()
+        e0.record(st)
+        for _ in range(reps):
+            fn()
+        e1.record(st)
+        ms = e0.elapsed_ms(e1) / reps
+        rows[name] = {"ms": round(ms, 4), "bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1),
+                      "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+    timed("copy_1GiB", lambda: capi.check(lib.cgt_amd_memcpy_async(capi.GPU, capi.GPU, c.ptr, a.ptr, 4 * n, st)), 8 * n)
+    timed("write_fill_1GiB", lambda: K.fill(3.0, (n,), out=c, stream=st), 4 * n)
+    timed("read_sum_1GiB", lambda: K.sum_keepdims(a, (0,), out=small, stream=st), 4 * n)
+    timed("add_2r1w_1GiB", lambda: K.elwise_binary("+", a, b, out=c, stream=st), 12 * n)
+    s.synchronize()
+    return rows
+
+
 def check_gemm_against_oracle():
     from cgt_amd import kernels as K
     from cgt_amd.gpuarray import to_gpu
@@ -736,12 +774,20 @@ def main():
     # the other configurations, same measurement (their stage tables carry the in-step clock;
     # the raw GEMMs, which have no step around them, the back-to-back one)
     if not args.only and args.workload == DEFAULT_WORKLOAD:
+        out["hbm_reference"] = hbm_reference()
         out["workloads"] = {}
         for name in EXTRA_WORKLOADS:
             r, _ = measure(name, args, primary=False)
             parity_ok = parity_ok and r["parity"]["ok"]
             r["unit"] = "TFLOP/s"
             out["workloads"][name] = r
+    if "hbm_reference" in out:
+        # every HBM-bound stage also against what a plain device-to-device copy reaches in this run
+        copy = out["hbm_reference"]["copy_1GiB"]["GBps"]
+        for table in [out["stages"]] + [w["stages"] for w in out["workloads"].values()]:
+            for row in table:
+                if row["bound"] == "hbm" and "GBps_in_step" in row:
+                    row["vs_measured_copy"] = round(row["GBps_in_step"] / copy, 3)
     if not args.no_cpu and not is_gemm:
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample)
     elif not args.no_cpu:

@@ -107,6 +107,10 @@ def test_default_workload_prints_the_contract_line():
     for name in ("cifar_conv1_5x5_3x32x32_b128", "mnist_conv3x3_1x28x28_b64"):
         gemms = [r for r in w[name]["stages"] if r["bound"] == "mfma"]
         assert len(gemms) == 3 and all(r["roof"] == "hbm" and r["frac_hbm"] > 0 and r["frac_in_step"] > 0 for r in gemms)
+    ref = out["hbm_reference"]
+    assert set(ref) == {"copy_1GiB", "write_fill_1GiB", "read_sum_1GiB", "add_2r1w_1GiB"}
+    assert all(0.2 < r["frac"] < 1.0 for r in ref.values())
+    assert all("vs_measured_copy" in r for r in out["stages"] if r["bound"] == "hbm")
     cpu = out["cpu_baseline"]
     assert cpu["kind"] in ("port", "reference") and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
     assert out["parity"]["ok"] is True

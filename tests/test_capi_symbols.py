@@ -65,6 +65,34 @@ def test_staged_pool_kernels_stay_inside_their_index_range():
     assert lib.cgt_amd_pool_staged_planes(0, 1, 1, 1001, 1001) in (0, 1, 2)
 
 
+def test_conv_same_host_side_rules():
+    # which layers the im2col-free products cover, and the padded layout's size: host code only
+    from cgt_amd import capi, core
+    from cgt_amd.nn_ops import conv_same
+    lib = capi.lib()
+    ok = lambda C, L, k, p, s: lib.cgt_amd_conv_same_supported(C, L, k, k, p, p, s, s)      # noqa: E731
+    assert ok(128, 128, 3, 1, 1) and ok(64, 128, 5, 2, 1) and ok(256, 512, 3, 1, 1) and ok(128, 256, 7, 3, 1)
+    assert not ok(3, 96, 11, 0, 4) and not ok(128, 128, 3, 0, 1) and not ok(128, 128, 3, 1, 2)
+    assert not ok(32, 64, 5, 2, 1) and not ok(120, 128, 3, 1, 1) and not ok(128, 96, 3, 1, 1)
+    assert not lib.cgt_amd_conv_same_supported(128, 128, 2, 2, 0, 0, 1, 1)
+    # pw zeros, then H + 2 ph rows of W + pw floats, rounded up past 16 zeros to a multiple of 16; + tail
+    plane = (1 + 58 * 57 + 16 + 15) // 16 * 16
+    tail = (256 + 3 * 57 + 3) // 4 * 4
+    assert lib.cgt_amd_conv_same_padded_size(1, 56, 56, 3, 3) == plane + tail
+    assert lib.cgt_amd_conv_same_padded_size(64 * 128, 56, 56, 3, 3) == 64 * 128 * plane + tail
+    assert lib.cgt_amd_conv_same_padded_size(5, 9, 20, 5, 3) == 5 * ((1 + 13 * 21 + 31) // 16 * 16) + (256 + 5 * 21 + 3) // 4 * 4
+    assert lib.cgt_amd_conv_same_padded_size(1, 56, 56, 2, 2) == -1
+    # the Op's shape rule is the same number, symbolically
+    info = conv_same.ConvSameInfo(3, 3)
+    B = core.ShapeInt(64, ("size", object(), 0))
+    n = conv_same.padded_size(B * 128, 56, 56, info)
+    assert n == 64 * 128 * plane + tail and not n.is_constant()
+    rc = lib.cgt_amd_conv_same_fwd_f32(None, None, None, 0, 1, 128, 8, 8, 128, 3, 3, None, None, None)
+    assert rc == 1 and "null" in capi.last_error()
+    rc = lib.cgt_amd_conv_same_bwd_filter_f32(None, None, 1, 128, 8, 8, 128, 4, 4, None, None)
+    assert rc == 1 and "odd" in capi.last_error()
+
+
 def test_argument_errors_are_reported_not_fatal():
     # argument validation happens on the host before any launch
     from cgt_amd import capi

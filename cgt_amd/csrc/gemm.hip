@@ -142,14 +142,32 @@ struct OperandTile {
     }
 
     // needs (ROWS - 1) * ld * 4 + 64 < 2^32 (the host checks)
-    __device__ __forceinline__ void init_offsets(long ld) {
+    // rows_valid < ROWS (k-contiguous operands of the convolution products only): rows past
+    // it load the last valid row again -- valid memory, and what they produce is never stored
+    __device__ __forceinline__ void init_offsets(long ld, int rows_valid = ROWS) {
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int idx = threadIdx.x + i * kGemmThreads;
             // the piece this thread fetches is the one whose LDS slot it fills: slot idx & 3
             // of row idx >> 2 holds chunk chunk_pos(row, idx & 3) (the permutation is an involution)
-            const long e = KC ? (long)(idx >> 2) * ld + chunk_pos(idx >> 2, idx & 3) * 4
+            const long e = KC ? (long)min(idx >> 2, rows_valid - 1) * ld + chunk_pos(idx >> 2, idx & 3) * 4
                               : (long)(idx / (ROWS / 4)) * ld + (idx % (ROWS / 4)) * 4;
+            goff[i] = (unsigned)(e * 4);
+        }
+    }
+
+    // Weight gradient of a convolution: row n of the (tap, channel) axis is channel n % C of
+    // the padded image shifted by tap n / C, so the row's offset is not n * ld but folds the
+    // tap's shift in; a tile may span several taps.  Rows past n_valid repeat the last one.
+    __device__ __forceinline__ void init_offsets_taps(long plane, int n0, int n_valid, int C, int kw, int wp) {
+        static_assert(KC, "pixel-contiguous operand");
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int idx = threadIdx.x + i * kGemmThreads;
+            const int n = min(n0 + (idx >> 2), n_valid - 1);
+            const int tap = n / C, c = n - tap * C;
+            const int ho = tap / kw, wo = tap - ho * kw;
+            const long e = (long)c * plane + (long)ho * wp + wo + chunk_pos(idx >> 2, idx & 3) * 4;
             goff[i] = (unsigned)(e * 4);
         }
     }
@@ -392,11 +410,9 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
         const int s0 = kbeg / KT;
         const int img = s0 / a.cv_spi;
         cv_i = s0 - img * a.cv_spi;
-        const int tap = n0 / a.cv_c, c0 = n0 - tap * a.cv_c;
-        const int ho = tap / a.cv_kw, wo = tap - ho * a.cv_kw;
+        // the rows of B (channel and tap of each column of the result) are folded into its lane offsets
         cvA = reinterpret_cast<const char*>(A + (long)img * a.cv_imgA + (long)m0 * a.cv_plane + (long)cv_i * KT);
-        cvB = reinterpret_cast<const char*>(B + (long)img * a.cv_imgB + (long)c0 * a.cv_plane + (long)ho * a.cv_wp + wo +
-                                            (long)cv_i * KT);
+        cvB = reinterpret_cast<const char*>(B + (long)img * a.cv_imgB + (long)cv_i * KT);
     }
     // origins of the next slice to be issued, then step to the one after it
     auto conv_next = [&](const char*& oa, const char*& ob) {
@@ -602,8 +618,16 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
             }
         }
     };
-    if (wholeA) ta.init_offsets(CONV == 2 ? a.cv_plane : a.lda);
-    if (wholeB) tb.init_offsets(CONV == 2 || CONV == 3 ? a.cv_plane : a.ldb);
+    if constexpr (CONV == 2) {
+        ta.init_offsets(a.cv_plane, min(BM, a.M - m0));
+        tb.init_offsets_taps(a.cv_plane, n0, a.N, a.cv_c, a.cv_kw, a.cv_wp);
+    } else if constexpr (CONV == 3) {
+        ta.init_offsets(a.lda, min(BM, a.M - m0));
+        tb.init_offsets(a.cv_plane);
+    } else {
+        if (wholeA) ta.init_offsets(a.lda);
+        if (wholeB) tb.init_offsets(a.ldb);
+    }
     if constexpr (CONV != 0) {
         main_loop(std::integral_constant<int, kFast>{});      // the host sends whole tiles and whole slices only
     } else {
@@ -624,28 +648,37 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
         const int r0 = m0 + wm_u * TM * 32;
         char* base = reinterpret_cast<char*>(a.C + ((long)img * a.M + r0) * HW);
         const long step1 = HW * 4, step5 = HW * 20;
+        const int rows_left = a.M - r0 - 4 * half;           // of this lane: output channels left in the result
+        auto store_tile = [&](auto wholec) {
+            constexpr bool WHOLE = decltype(wholec)::value;
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int q = t * BN + (wn_u * TN + j) * 32 + l32;
-            const int h = q / a.cv_wp, w = q - h * a.cv_wp;
-            if (h < a.cv_h && w < a.cv_w) {
-                unsigned lane_off = (unsigned)((4 * half * HW + (long)h * a.cv_w + w) * 4);
-                char* row = base;
+            for (int j = 0; j < TN; ++j) {
+                const int q = t * BN + (wn_u * TN + j) * 32 + l32;
+                const int h = q / a.cv_wp, w = q - h * a.cv_wp;
+                if (h < a.cv_h && w < a.cv_w) {
+                    unsigned lane_off = (unsigned)((4 * half * HW + (long)h * a.cv_w + w) * 4);
+                    char* row = base;
 #pragma unroll
-                for (int i = 0; i < TM; ++i)
+                    for (int i = 0; i < TM; ++i)
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        asm volatile("" : "+v"(lane_off));
-                        float v = acc[i][j][e];
-                        if (a.cv_bias) v += a.cv_bias[r0 + i * 32 + 8 * (e / 4) + (e % 4) + 4 * half];
-                        if (a.cv_mask)      // same element index as in the float array: byte offset / 4
-                            a.cv_mask[((row - reinterpret_cast<char*>(a.C)) + lane_off) >> 2] = v >= 0.0f ? 1 : 0;
-                        if (a.cv_relu) v = v * (v >= 0.0f ? 1.0f : 0.0f);
-                        *reinterpret_cast<float*>(row + lane_off) = v;
-                        row += (e % 4 == 3) ? step5 : step1;
-                    }
+                        for (int e = 0; e < 16; ++e) {
+                            asm volatile("" : "+v"(lane_off));
+                            const int r = i * 32 + 8 * (e / 4) + (e % 4);
+                            if (WHOLE || r < rows_left) {
+                                float v = acc[i][j][e];
+                                if (a.cv_bias) v += a.cv_bias[r0 + r + 4 * half];
+                                if (a.cv_mask)      // same element index as in the float array: byte offset / 4
+                                    a.cv_mask[((row - reinterpret_cast<char*>(a.C)) + lane_off) >> 2] = v >= 0.0f ? 1 : 0;
+                                if (a.cv_relu) v = v * (v >= 0.0f ? 1.0f : 0.0f);
+                                *reinterpret_cast<float*>(row + lane_off) = v;
+                            }
+                            row += (e % 4 == 3) ? step5 : step1;
+                        }
+                }
             }
-        }
+        };
+        if (m0 + BM <= a.M) store_tile(std::true_type{});
+        else store_tile(std::false_type{});
         return;
     }
     // Destination: C, this split's partial matrix, or (tail pieces) a tile-local
@@ -767,6 +800,7 @@ __global__ __launch_bounds__(256) void tail_reduce_conv_kernel(const float* __re
         }
     const int r = i / bn, c = i - r * bn;
     const int row = tm * bm + r;                         // output channel
+    if (row >= a.M) return;
     const int img = tn / a.cv_tpi, t = tn - img * a.cv_tpi;
     const long HW = (long)a.cv_h * a.cv_w;
     float* dst = a.C + ((long)img * a.M + row) * HW;
@@ -918,36 +952,45 @@ static void launch_conv(int mode, int shape, dim3 grid, hipStream_t st, const Ge
     if (mode == 3) {
         switch (shape) {
             case 0: sgemm_kernel<true, false, false, 2, 2, 2, 2, false, 3><<<grid, block, 0, st>>>(a); break;
+            case 4: sgemm_kernel<true, false, false, 1, 4, 3, 1, false, 3><<<grid, block, 0, st>>>(a); break;    // 96 x 128
             default: sgemm_kernel<true, false, false, 1, 4, 2, 1, false, 3><<<grid, block, 0, st>>>(a); break;   // 64 x 128
         }
     } else {
         switch (shape) {
             case 0: sgemm_kernel<true, true, false, 2, 2, 2, 2, false, 2><<<grid, block, 0, st>>>(a); break;
+            case 1: sgemm_kernel<true, true, false, 4, 1, 1, 3, false, 2><<<grid, block, 0, st>>>(a); break;
             case 2: sgemm_kernel<true, true, false, 4, 1, 1, 2, false, 2><<<grid, block, 0, st>>>(a); break;
-            default: sgemm_kernel<true, true, false, 4, 1, 1, 1, false, 2><<<grid, block, 0, st>>>(a); break;
+            case 3: sgemm_kernel<true, true, false, 4, 1, 1, 1, false, 2><<<grid, block, 0, st>>>(a); break;
+            case 4: sgemm_kernel<true, true, false, 1, 4, 3, 1, false, 2><<<grid, block, 0, st>>>(a); break;
+            default: sgemm_kernel<true, true, false, 1, 4, 2, 1, false, 2><<<grid, block, 0, st>>>(a); break;
         }
     }
 }
 
-// tile shape (index into kShapes) of an implicit-convolution product, -1 if none fits:
-// tiles must be whole -- mode 3: 128 (or one tile of 64) output channels x 128 pixels;
-// mode 2: 128 filters x an N tile that divides the channel count, so that a tile of the
-// (tap, channel) axis lies in one tap
-static int conv_shape(int mode, long filters, long channels) {
-    if (mode == 3) {        // rows = filters: 128-row tiles, or one 64-row tile; 128 pixels per tile
-        if (channels % KT != 0) return -1;
-        return filters % 128 == 0 ? 0 : (filters == 64 ? 5 : -1);
+// tile shape (index into kShapes) of an implicit-convolution product, -1 if none fits: the
+// shape with the least padded work; rows past the end of the result (filters that do not
+// fill the last tile) are computed from repeated operand rows and never stored.
+//   mode 3: `rows` output channels x 128 pixels per tile; the K slices need whole blocks of 16 channels;
+//   mode 2: `rows` filters x `cols` = taps * channels.
+static int conv_shape(int mode, long rows, long cols, long channels) {
+    if (channels % KT != 0 || rows < 1) return -1;
+    int best = -1;
+    double best_work = 0;
+    for (int i = 0; i < (int)(sizeof(kShapes) / sizeof(kShapes[0])); ++i) {
+        if (mode == 3 && kShapes[i].bn != 128) continue;
+        const double work = (double)(cdiv(rows, kShapes[i].bm) * kShapes[i].bm) *
+                            (mode == 3 ? 1.0 : (double)(cdiv(cols, kShapes[i].bn) * kShapes[i].bn));
+        if (best < 0 || work < best_work * 0.97) {
+            best = i;
+            best_work = work;
+        }
     }
-    const long n = channels;
-    if (filters % 128 != 0) return -1;
-    if (channels % KT != 0) return -1;
-    if (n % 128 == 0) return 0;
-    if (n == 64) return 2;
-    if (n == 32) return 3;
-    return -1;
+    return best;
 }
 
-bool sgemm_conv_supported(int mode, long filters, long channels) { return conv_shape(mode, filters, channels) >= 0; }
+bool sgemm_conv_supported(int mode, long filters, long channels) {
+    return filters >= 1 && channels >= KT && channels % KT == 0 && mode >= 2 && mode <= 3;
+}
 
 static void launch_trans(int tA, int tB, bool pipe, bool deep, int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
     dim3 block(kGemmThreads);
@@ -1005,10 +1048,12 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
         return p;
     };
     if (cv) {
-        shape = conv_shape(cv->mode, M, cv->C);
+        shape = conv_shape(cv->mode, M, N, cv->C);
         CGT_ARG_CHECK(cv->mode != 3 || (long)cv->tpi * cv->B * 128 == N, "sgemm_conv: mode 3 takes whole tiles of pixels");
-        CGT_ARG_CHECK(shape >= 0, "sgemm_conv: no tile shape for these extents");
-        CGT_ARG_CHECK(cv->plane < (1L << 24), "sgemm_conv: padded plane too large");
+        CGT_ARG_CHECK(shape >= 0, "sgemm_conv: the image must have a multiple of 16 channels");
+        // lane offsets are 32-bit: a tile's rows (mode 2: the channels of a whole image) span less than 4 GB
+        CGT_ARG_CHECK(cv->plane < (1L << 23) && (cv->mode != 2 || cv->C * cv->plane < (1L << 30)),
+                      "sgemm_conv: padded planes too large");
     }
     GemmArgs a;
     a.conv = cv ? cv->mode : 0;

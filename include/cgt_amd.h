@@ -305,8 +305,10 @@ int cgt_amd_sgemm_batched(int tA, int tB, long P, long M, long N, long K,
  * a zeroed tail; cgt_amd_conv_same_pad_f32 writes all of it. */
 
 /* 1 if the three entry points below cover this layer: stride 1, odd kernel,
- * pad = (kernel - 1) / 2, L a multiple of 128, C a multiple of 128 or 64
- * (whole GEMM tiles).  Otherwise use im2col + cgt_amd_sgemm + col2im. */
+ * pad = (kernel - 1) / 2, C and L multiples of 16 (the products walk the
+ * channels in blocks of 16; tiles are whole when L and C are multiples of 128,
+ * 96 or 64 and padded otherwise).  Otherwise use im2col + cgt_amd_sgemm +
+ * col2im. */
 int cgt_amd_conv_same_supported(long C, long L, int kh, int kw, int ph, int pw, int sh, int sw);
 
 /* Floats in the padded copy of `planes` planes of H x W (tail included); -1 on bad arguments. */

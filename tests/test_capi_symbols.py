@@ -73,7 +73,9 @@ def test_conv_same_host_side_rules():
     ok = lambda C, L, k, p, s: lib.cgt_amd_conv_same_supported(C, L, k, k, p, p, s, s)      # noqa: E731
     assert ok(128, 128, 3, 1, 1) and ok(64, 128, 5, 2, 1) and ok(256, 512, 3, 1, 1) and ok(128, 256, 7, 3, 1)
     assert not ok(3, 96, 11, 0, 4) and not ok(128, 128, 3, 0, 1) and not ok(128, 128, 3, 1, 2)
-    assert not ok(32, 64, 5, 2, 1) and not ok(120, 128, 3, 1, 1) and not ok(128, 96, 3, 1, 1)
+    # channels and filters in multiples of 16 (tiles that are not whole are padded)
+    assert ok(32, 64, 5, 2, 1) and ok(128, 96, 3, 1, 1) and ok(16, 16, 3, 1, 1) and ok(48, 80, 1, 0, 1)
+    assert not ok(120, 128, 3, 1, 1) and not ok(128, 72, 3, 1, 1) and not ok(3, 32, 5, 2, 1)
     assert not lib.cgt_amd_conv_same_supported(128, 128, 2, 2, 0, 0, 1, 1)
     # pw zeros, then H + 2 ph rows of W + pw floats, rounded up past 16 zeros to a multiple of 16; + tail
     plane = (1 + 58 * 57 + 16 + 15) // 16 * 16

@@ -51,6 +51,13 @@ CASES = [
     (1, 128, 56, 56, 128, (3, 3)),
     (5, 64, 3, 70, 128, (3, 5)),
     (2, 128, 1, 1, 128, (3, 3)),
+    # filters / channels that do not fill the last tile of rows, tiles that span several taps
+    (4, 32, 15, 15, 64, (5, 5)),            # the second convolution of the CIFAR stack
+    (2, 16, 8, 9, 16, (3, 3)),
+    (2, 48, 7, 12, 80, (3, 3)),
+    (1, 160, 6, 6, 96, (3, 3)),
+    (2, 96, 5, 13, 208, (1, 3)),
+    (3, 64, 13, 13, 64, (3, 3)),
 ]
 
 
@@ -111,12 +118,15 @@ def test_conv_same_supported_rule(K):
     assert K.conv_same_supported(128, 128, (3, 3), (1, 1), (1, 1))
     assert K.conv_same_supported(64, 128, (5, 5), (2, 2), (1, 1))
     assert K.conv_same_supported(256, 512, (3, 3), (1, 1), (1, 1))
-    assert not K.conv_same_supported(32, 128, (5, 5), (2, 2), (1, 1))     # 32 channels: no data-gradient tile
+    assert K.conv_same_supported(32, 64, (5, 5), (2, 2), (1, 1))          # tiles padded in both products
+    assert K.conv_same_supported(16, 16, (3, 3), (1, 1), (1, 1))
+    assert K.conv_same_supported(48, 80, (1, 3), (0, 1), (1, 1))
+    assert not K.conv_same_supported(24, 128, (5, 5), (2, 2), (1, 1))     # channels: not a multiple of 16
+    assert not K.conv_same_supported(128, 72, (5, 5), (2, 2), (1, 1))     # filters (channels of the data gradient)
     assert not K.conv_same_supported(3, 96, (11, 11), (0, 0), (4, 4))     # AlexNet conv1: strided
     assert not K.conv_same_supported(3, 32, (5, 5), (2, 2), (1, 1))       # 3 channels: not a multiple of 16
     assert not K.conv_same_supported(128, 128, (3, 3), (0, 0), (1, 1))    # valid padding
     assert not K.conv_same_supported(128, 128, (2, 2), (0, 0), (1, 1))    # even kernel
-    assert not K.conv_same_supported(32, 64, (5, 5), (2, 2), (1, 1))      # 64 filters: no weight-gradient tile
 
 
 def test_nn_conv2d_takes_the_fused_ops_and_grad_goes_through_them(K):

@@ -183,8 +183,14 @@ class LayerOnGpu(object):
         self.f_LZ = self.f.reshape(L, Z)
         nelem = lambda a: int(np.prod(a.shape))  # noqa: E731
         # what nn.conv2d builds for this layer: the fused ops without a column buffer where they
-        # apply (stride 1, same padding, tile-sized channel counts), else im2col -> Mul22
-        self.algo = "direct" if algo == "auto" and K.conv_same_supported(C, L, (r, c), pad, stride) else "im2col"
+        # apply (stride 1, same padding, channel counts in multiples of 16), else im2col and the fused
+        # products over the column buffer ("col"); "im2col" is the literal composition with Mul22 and
+        # the two transposes
+        if algo == "auto":
+            self.algo = "direct" if K.conv_same_supported(C, L, (r, c), pad, stride) else "col"
+        else:
+            self.algo = algo
+        fused_col = self.algo == "col"
         if self.algo == "direct":
             self.overlap = False
             self.glue = glue
@@ -192,7 +198,7 @@ class LayerOnGpu(object):
             return
         self.col = empty((B, m, n, Z))
         self.col2 = self.col.reshape(Bmn, Z)
-        self.y_mnL = empty((Bmn, L))
+        self.y_mnL = None if fused_col else empty((Bmn, L))
         self.y = empty((B, L, m, n))
         act = self.y
         st = []
@@ -200,11 +206,15 @@ class LayerOnGpu(object):
         gemm_bytes = 4 * (Bmn * Z + L * Z + Bmn * L)      # the three conv products touch the same three matrices
         st.append(Stage("im2col", "im2col_linear_kernel or im2col_pipe_kernel", lambda: K.im2col(self.x, (r, c), pad, stride, out=self.col, stream=s),
                         4 * (nelem(self.x) + nelem(self.col)), "hbm"))
-        st.append(Stage("gemm_fwd_NT", "sgemm_kernel", lambda: K.mul22(self.col2, self.f_LZ, False, True, out=self.y_mnL, stream=s),
-                        2 * Bmn * L * Z, "mfma", gemm_bytes))
-        st.append(Stage("transpose_0312", "thin_transpose_kernel or batched_transpose_kernel",
-                        lambda: K.transpose4(self.y_mnL.reshape(B, m, n, L), (0, 3, 1, 2), out=self.y, stream=s),
-                        2 * 4 * nelem(self.y), "hbm"))
+        if fused_col:       # the product writes [B,L,m,n] itself
+            st.append(Stage("gemm_fwd", "sgemm_kernel", lambda: K.conv_col_fwd(self.col, self.f, out=self.y, stream=s),
+                            2 * Bmn * L * Z, "mfma", gemm_bytes))
+        else:
+            st.append(Stage("gemm_fwd_NT", "sgemm_kernel", lambda: K.mul22(self.col2, self.f_LZ, False, True, out=self.y_mnL, stream=s),
+                            2 * Bmn * L * Z, "mfma", gemm_bytes))
+            st.append(Stage("transpose_0312", "thin_transpose_kernel or batched_transpose_kernel",
+                            lambda: K.transpose4(self.y_mnL.reshape(B, m, n, L), (0, 3, 1, 2), out=self.y, stream=s),
+                            2 * 4 * nelem(self.y), "hbm"))
         if cfg["lrn"]:
             size, alpha, beta, k = cfg["lrn"]
             self.top, self.scale = empty(self.y.shape), empty(self.y.shape)
@@ -234,20 +244,30 @@ class LayerOnGpu(object):
                             5 * 4 * nelem(self.y), "hbm"))
             gy = self.gy_lrn
         self.gy = gy
-        self.gc = empty((B, m, n, L))
-        self.gc2 = self.gc.reshape(Bmn, L)
         self.gcol = empty((Bmn, Z))
         self.gx = empty(self.x.shape)
         self.gf = empty((L, Z))
-        st.append(Stage("transpose_0231", "thin_transpose_kernel or batched_transpose_kernel", lambda: K.transpose4(self.gy, (0, 2, 3, 1), out=self.gc, stream=s),
-                        2 * 4 * nelem(self.y), "hbm"))
-        st.append(Stage("gemm_dgrad_NN", "sgemm_kernel", lambda: K.mul22(self.gc2, self.f_LZ, False, False, out=self.gcol, stream=s),
-                        2 * Bmn * L * Z, "mfma", gemm_bytes))
-        st.append(Stage("col2im", "col2im_stream_kernel",
-                        lambda: K.col2im(self.gcol.reshape(B, m, n, Z), self.x.shape, (r, c), pad, stride, out=self.gx, stream=s),
-                        4 * (nelem(self.x) + nelem(self.col)), "hbm"))
-        st.append(Stage("gemm_wgrad_TN", "sgemm_kernel", lambda: K.mul22(self.gc2, self.col2, True, False, out=self.gf, stream=self._wgrad_stream),
-                        2 * Bmn * L * Z, "mfma", gemm_bytes))
+        col2im = Stage("col2im", "col2im_stream_kernel",
+                       lambda: K.col2im(self.gcol.reshape(B, m, n, Z), self.x.shape, (r, c), pad, stride, out=self.gx, stream=s),
+                       4 * (nelem(self.x) + nelem(self.col)), "hbm")
+        if fused_col:       # both gradient products read the NCHW cotangent themselves
+            self.overlap = False
+            gcol4, gf4 = self.gcol.reshape(B, m, n, Z), self.gf.reshape(L, C, r, c)
+            st.append(Stage("gemm_dgrad", "sgemm_kernel", lambda: K.conv_col_bwd_data(self.gy, self.f, out=gcol4, stream=s),
+                            2 * Bmn * L * Z, "mfma", gemm_bytes))
+            st.append(col2im)
+            st.append(Stage("gemm_wgrad", "sgemm_kernel", lambda: K.conv_col_bwd_filter(self.gy, self.col, self.f.shape, out=gf4, stream=s),
+                            2 * Bmn * L * Z, "mfma", gemm_bytes))
+        else:
+            self.gc = empty((B, m, n, L))
+            self.gc2 = self.gc.reshape(Bmn, L)
+            st.append(Stage("transpose_0231", "thin_transpose_kernel or batched_transpose_kernel", lambda: K.transpose4(self.gy, (0, 2, 3, 1), out=self.gc, stream=s),
+                            2 * 4 * nelem(self.y), "hbm"))
+            st.append(Stage("gemm_dgrad_NN", "sgemm_kernel", lambda: K.mul22(self.gc2, self.f_LZ, False, False, out=self.gcol, stream=s),
+                            2 * Bmn * L * Z, "mfma", gemm_bytes))
+            st.append(col2im)
+            st.append(Stage("gemm_wgrad_TN", "sgemm_kernel", lambda: K.mul22(self.gc2, self.col2, True, False, out=self.gf, stream=self._wgrad_stream),
+                            2 * Bmn * L * Z, "mfma", gemm_bytes))
         self.stages = st
         self.conv_flops = 6 * Bmn * L * Z
         # The glue a SpatialConvolution training step adds around this layer
@@ -519,6 +539,8 @@ def check_against_oracle(cfg):
     y = K.conv2d(to_gpu(x), to_gpu(f), pad, stride).get()
     y64 = O.conv2d(x.astype(np.float64), f.astype(np.float64), pad, stride)
     err = float(np.linalg.norm(y - y64) / np.linalg.norm(y64))
+    y = K.conv_col_fwd(col, to_gpu(f)).get()        # the fused product over the same column buffer
+    err = max(err, float(np.linalg.norm(y - y64) / np.linalg.norm(y64)))
     return {"im2col_bit_exact": bool(ok), "conv2d_rel_fro": err, "ok": bool(ok and err <= 1e-4)}
 
 
@@ -690,8 +712,9 @@ def measure(workload, args, primary):
               "schedule": ("one stream" if not getattr(layer, "overlap", False) else
                            "weight-gradient GEMM on a second stream beside col2im")}
     if algo:
-        config["conv_algo"] = ("fused ops, no column buffer (pad -> GEMM over the padded image -> NCHW)" if algo == "direct"
-                               else "im2col -> Mul22 -> transpose; transpose -> Mul22 -> col2im, Mul22")
+        config["conv_algo"] = {"direct": "fused ops, no column buffer (pad -> GEMM over the padded image -> NCHW)",
+                               "col": "im2col -> fused products over the column buffer (NCHW written / read by the GEMMs) -> col2im",
+                               "im2col": "im2col -> Mul22 -> transpose; transpose -> Mul22 -> col2im, Mul22"}[algo]
     if is_gemm:
         config["value_is"] = "flops of Mul22 4096^3 x {NN,NT,TN,TT} + BatchedMul22 64x512^3 / step time"
     elif cfg.get("lrn"):
@@ -741,9 +764,10 @@ def main():
     ap.add_argument("--no-op-api", action="store_true", help="skip timing the same step through the Op API")
     ap.add_argument("--no-check", action="store_true",
                     help="skip the parity gate (profiling runs: keeps its small launches out of the kernel statistics)")
-    ap.add_argument("--conv-algo", default="auto", choices=["auto", "im2col"],
-                    help="auto: the fused convolution ops where they apply (what nn.conv2d builds); im2col: always the "
-                         "im2col -> Mul22 composition")
+    ap.add_argument("--conv-algo", default="auto", choices=["auto", "col", "im2col"],
+                    help="auto: what nn.conv2d builds (the fused ops without a column buffer where they apply, else "
+                         "im2col + the fused products over the column buffer); col: the latter for every layer; "
+                         "im2col: always the literal im2col -> Mul22 -> transpose composition")
     ap.add_argument("--only", action="store_true",
                     help="measure --workload alone (profiling runs); by default the headline workload is followed by "
                          "the other configurations, reported under `workloads`")

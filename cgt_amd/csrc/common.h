@@ -25,14 +25,18 @@ enum WorkspaceUser { kWsGemm = 0, kWsSum = 1, kWsConvFilter = 2, kWsUsers = 3 };
 float* stream_workspace(void* stream, WorkspaceUser user, size_t bytes, const char* what);
 void release_stream_workspaces(void* stream);
 
-// GEMM over an operand read straight from a zero-padded image (gemm.hip): the products of
-// a stride-1 convolution with pad = (kernel - 1) / 2, without a column buffer.
+// The GEMMs of a convolution layer with the layer's layouts built in (gemm.hip).
+// Over an operand read straight from a zero-padded image -- stride 1, pad = (kernel - 1) / 2,
+// no column buffer:
 //   mode 2: out[M][taps * C] = sum over (b, q) of A[b][m][q] * img[b][c][q + tapoff]
 //   mode 3: out[b][m][h][w] = sum over (c, tap) of Wk[m][c/16][tap][c%16] * img[b][c][q + tapoff] (+ bias[m], rectify),
 //           q = h*Wp + w: the pixels of the padded grid are the columns, tpi tiles of 128 per image
+// Over a column buffer col[B * plane][C] (any geometry), with the NCHW side read / written in place:
+//   mode 1: out[b][m][p] = sum over z of W[m][z] * col[b * plane + p][z] (+ bias[m], rectify); C = patch length
+//   mode 4: out[M][N] = sum over (b, p) of A[b][m][p] * col[b * plane + p][n]   (A = the NCHW cotangent)
 struct ConvGemm {
     int mode;
-    long B, C, plane;      // images, channels of `img`, floats per padded plane
+    long B, C, plane;      // images; channels of `img` (mode 1: patch length); floats per padded plane (modes 1, 4: pixels per image)
     int wp, kh, kw;        // padded width, kernel
     long tpi, spi;         // mode 3: pixel tiles (of 128) per image; mode 2: K slices (of 16) per image
     long H, W;             // mode 3: image extents

@@ -228,3 +228,48 @@ CGT_API int cgt_amd_conv_same_bwd_filter_f32(const float* gypad, const float* xp
     const int ax[4] = {0, 3, 1, 2};
     return cgt_amd_transpose4_f32(wk, ws, ax, gf, stream);
 }
+
+// ---- any geometry, over the column buffer of im2col: the three products of conv2d with the
+// NCHW side read and written in place (no [B*m*n, L] intermediate, no transposes).
+//   col [B * P][Z] (P = m * n output pixels per image, Z = C * kh * kw), f [L][Z] (= [L,C,kh,kw]),
+//   y / gy [B][L][P]
+
+CGT_API int cgt_amd_conv_col_fwd_f32(const float* col, const float* f, const float* bias, int relu, long B, long P,
+                                     long Z, long L, float* y, signed char* mask, void* stream) {
+    CGT_ARG_CHECK(B >= 0 && P >= 0 && Z >= 0 && L >= 0, "conv_col_fwd: negative extent");
+    if (B == 0 || P == 0 || L == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(y && (Z == 0 || (col && f)), "conv_col_fwd: null pointer");
+    CGT_ARG_CHECK(B * P < (1L << 31) - 128, "conv_col_fwd: too many output pixels");
+    // y[b][l][p] = sum_z f[l][z] col[b * P + p][z]: rows are filters, so a wavefront's store covers
+    // consecutive pixels of one channel plane
+    ConvGemm cv = {1, B, Z, P, 0, 1, 1, 0, 0, 0, 0, bias, relu, mask};
+    return sgemm_conv(cv, L, B * P, f, col, y, B * P, stream);
+}
+
+// gcol[b * P + p][z] = sum_l gy[b][l][p] f[l][z]: per image a product with the transposed
+// cotangent plane block as its first operand
+CGT_API int cgt_amd_conv_col_bwd_data_f32(const float* gy, const float* f, long B, long P, long Z, long L,
+                                          float* gcol, void* stream) {
+    CGT_ARG_CHECK(B >= 0 && P >= 0 && Z >= 0 && L >= 0, "conv_col_bwd_data: negative extent");
+    if (B == 0 || P == 0 || Z == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(gcol && (L == 0 || (gy && f)), "conv_col_bwd_data: null pointer");
+    int rc = CGT_AMD_OK;
+    for (long b0 = 0; b0 < B && rc == CGT_AMD_OK; b0 += 32768) {     // the batched product takes fewer than 65536 at a time
+        const long nb = std::min(B - b0, 32768L);
+        rc = cgt_amd_sgemm_batched(1, 0, nb, P, Z, L, gy + b0 * L * P, P, L * P, f, Z, 0, gcol + b0 * P * Z, Z, P * Z, stream);
+    }
+    return rc;
+}
+
+// gf[l][z] = sum over (b, p) of gy[b][l][p] col[b * P + p][z]
+CGT_API int cgt_amd_conv_col_bwd_filter_f32(const float* gy, const float* col, long B, long P, long Z, long L,
+                                            float* gf, void* stream) {
+    CGT_ARG_CHECK(B >= 0 && P >= 0 && Z >= 0 && L >= 0, "conv_col_bwd_filter: negative extent");
+    if (L == 0 || Z == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(gf, "conv_col_bwd_filter: null pointer");
+    if (B == 0 || P == 0) return cgt_amd_fill_u32(gf, 0u, L * Z, stream);
+    CGT_ARG_CHECK(gy && col, "conv_col_bwd_filter: null pointer");
+    CGT_ARG_CHECK(B * P < (1L << 31) - 128, "conv_col_bwd_filter: too many output pixels");
+    ConvGemm cv = {4, B, Z, P, 0, 1, 1, 0, 0, 0, 0, nullptr, 0, nullptr};
+    return sgemm_conv(cv, L, Z, gy, col, gf, Z, stream);
+}

@@ -115,6 +115,14 @@ struct GemmArgs {
     const float* cv_bias;                             // mode 3: per-row (output channel) bias or null
     signed char* cv_mask;                             // mode 3: where (x >= 0) goes as int8, or null
     long cv_plane, cv_imgA, cv_imgB;                  // plane stride and per-image strides (floats)
+    //   mode 1 (forward over a column buffer): a plain NT product C[l][n] = sum_z W[l][z] * col[n][z]
+    //     whose columns n = (image, pixel) are written as out[image][l][pixel] (cv_plane =
+    //     pixels per image), with the same optional bias / rectify / mask as mode 3.
+    // K cut per image (weight gradient from an NCHW cotangent, plain kernel): split s is piece
+    // s % kspi of image s / kspi; the image's K range is [img * kimg, (img + 1) * kimg) and
+    // its A operand starts aimg floats further per image (A is [image][M][kimg], k-contiguous).
+    int kimg, kspi;
+    long aimg;
 };
 
 // One ROWS x KT operand tile, moved with 16-byte accesses.
@@ -277,9 +285,9 @@ __device__ __forceinline__ int xcd_remap(int id, int n) {
 template <bool AKC, bool BKC, bool PIPE, int WGM, int WGN, int TM, int TN, bool DEEP = false, int CONV = 0>
 __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmArgs a) {
     static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
-    static_assert(CONV == 0 || ((CONV == 2 || CONV == 3) && !PIPE && !DEEP && AKC && BKC == (CONV == 2)),
-                  "implicit convolution: plain loop; the image operand is B, row-contiguous in mode 3; "
-                  "both operands k-contiguous in mode 2");
+    static_assert(CONV == 0 || (CONV >= 1 && CONV <= 3 && !PIPE && !DEEP && AKC && BKC == (CONV != 3)),
+                  "convolution products: plain loop; the image operand is B, row-contiguous in mode 3; "
+                  "both operands k-contiguous in modes 1 and 2");
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
     typedef OperandTile<AKC, BM> TileA;
     typedef OperandTile<BKC, BN> TileB;
@@ -322,10 +330,16 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
     const int tm = first_m + in_group % gsz, tn = in_group / gsz;
     const int m0 = tm * BM, n0 = tn * BN;
 
-    const int kbeg = split * kchunk;
-    const int kend = min(a.K, kbeg + kchunk);
+    int kbeg = split * kchunk;
+    int kend = min(a.K, kbeg + kchunk);
     const float* A = a.A + batch * a.sA;
     const float* B = a.B + batch * a.sB;
+    if (CONV == 0 && a.kimg) {      // K cut per image: this split is one piece of one image
+        const int img = split / a.kspi, piece = split - img * a.kspi;
+        kbeg = img * a.kimg + piece * kchunk;
+        kend = min((img + 1) * a.kimg, kbeg + kchunk);
+        A += (long)img * a.aimg;
+    }
 
     v16f acc[TM][TN];
 #pragma unroll
@@ -387,8 +401,8 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
     // whole (an edge tile in N still streams A untested) and the tested ones
     // otherwise; a ragged last K slice is tested for both.
     constexpr int kFast = 0, kMixed = 1;
-    const bool wholeA = CONV != 0 || (m0 + BM <= a.M && !a.wide), wholeB = CONV != 0 || (n0 + BN <= a.N && !a.wide);
-    const bool ragged_k = CONV == 0 && (kend - kbeg) % KT != 0;
+    const bool wholeA = CONV >= 2 || (m0 + BM <= a.M && !a.wide), wholeB = CONV >= 2 || (n0 + BN <= a.N && !a.wide);
+    const bool ragged_k = CONV <= 1 && (kend - kbeg) % KT != 0;
     const char* originA = reinterpret_cast<const char*>(A + (AKC ? (long)m0 * a.lda + kbeg : (long)kbeg * a.lda + m0));
     const char* originB = reinterpret_cast<const char*>(B + (BKC ? (long)n0 * a.ldb + kbeg : (long)kbeg * a.ldb + n0));
     const long stepA = (AKC ? (long)KT : (long)KT * a.lda) * 4, stepB = (BKC ? (long)KT : (long)KT * a.ldb) * 4;
@@ -544,7 +558,7 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                 // iteration kt-1, which every wavefront left through the barrier.
                 const int wave_u = __builtin_amdgcn_readfirstlane(wave);
                 if (nk > 0) {
-                    if constexpr (CONV != 0) {
+                    if constexpr (CONV >= 2) {
                         const char *oa, *ob;
                         conv_next(oa, ob);
                         ta.load_direct(oa, ta.goff, As[0], wave_u);
@@ -559,7 +573,7 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                 for (int kt = 0; kt < nk; ++kt) {
                     const int cur = kt & 1;
                     if (kt + 1 < nk) {
-                        if constexpr (CONV != 0) {
+                        if constexpr (CONV >= 2) {
                             const char *oa, *ob;
                             conv_next(oa, ob);
                             ta.load_direct(oa, ta.goff, As[cur ^ 1], wave_u);
@@ -628,8 +642,8 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
         if (wholeA) ta.init_offsets(a.lda);
         if (wholeB) tb.init_offsets(a.ldb);
     }
-    if constexpr (CONV != 0) {
-        main_loop(std::integral_constant<int, kFast>{});      // the host sends whole tiles and whole slices only
+    if constexpr (CONV >= 2) {
+        main_loop(std::integral_constant<int, kFast>{});      // the host sends whole slices only; rows past the end are clamped
     } else {
         if (wholeA && wholeB && !ragged_k) main_loop(std::integral_constant<int, kFast>{});
         else main_loop(std::integral_constant<int, kMixed>{});
@@ -657,6 +671,50 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                 const int h = q / a.cv_wp, w = q - h * a.cv_wp;
                 if (h < a.cv_h && w < a.cv_w) {
                     unsigned lane_off = (unsigned)((4 * half * HW + (long)h * a.cv_w + w) * 4);
+                    char* row = base;
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            asm volatile("" : "+v"(lane_off));
+                            const int r = i * 32 + 8 * (e / 4) + (e % 4);
+                            if (WHOLE || r < rows_left) {
+                                float v = acc[i][j][e];
+                                if (a.cv_bias) v += a.cv_bias[r0 + r + 4 * half];
+                                if (a.cv_mask)      // same element index as in the float array: byte offset / 4
+                                    a.cv_mask[((row - reinterpret_cast<char*>(a.C)) + lane_off) >> 2] = v >= 0.0f ? 1 : 0;
+                                if (a.cv_relu) v = v * (v >= 0.0f ? 1.0f : 0.0f);
+                                *reinterpret_cast<float*>(row + lane_off) = v;
+                            }
+                            row += (e % 4 == 3) ? step5 : step1;
+                        }
+                }
+            }
+        };
+        if (m0 + BM <= a.M) store_tile(std::true_type{});
+        else store_tile(std::false_type{});
+        return;
+    }
+    if (CONV == 1 && tail_piece < 0) {
+        // Rows are output channels, columns (image, pixel) pairs: the tile goes straight into
+        // out[image][channel][pixel].  A tile of columns may straddle images, so the image is
+        // part of the lane's offset (relative to the image of the tile's first column).
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+        const int wm_u = wave_u / WGN, wn_u = wave_u % WGN;
+        const int HW = (int)a.cv_plane;
+        const int img0 = n0 / HW;
+        const int r0 = m0 + wm_u * TM * 32;
+        char* base = reinterpret_cast<char*>(a.C + ((long)img0 * a.M + r0) * HW);
+        const long step1 = (long)HW * 4, step5 = (long)HW * 20;
+        const int rows_left = a.M - r0 - 4 * half;
+        auto store_tile = [&](auto wholec) {
+            constexpr bool WHOLE = decltype(wholec)::value;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int n = n0 + (wn_u * TN + j) * 32 + l32;
+                if (n < a.N) {
+                    const int img = n / HW, p = n - img * HW;
+                    unsigned lane_off = (unsigned)(((long)(img - img0) * a.M * HW + 4 * half * (long)HW + p) * 4);
                     char* row = base;
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
@@ -774,9 +832,10 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restric
         if (n0 + c + j < a.N) dst[j] = o[j];
 }
 
-// The same for a mode-3 convolution product: tile rows are output channels, tile columns
-// pixels of the padded grid; the sums go to out[image][channel][h][w], junk pixels dropped,
-// with the optional bias and rectify of the in-place epilogue.
+// The same for a convolution product that writes NCHW itself (modes 1 and 3): tile rows are
+// output channels, tile columns pixels (mode 3: of the padded grid, junk pixels dropped; mode
+// 1: (image, pixel) pairs); the sums go to out[image][channel][pixel] with the optional bias
+// and rectify of the in-place epilogue.
 __global__ __launch_bounds__(256) void tail_reduce_conv_kernel(const float* __restrict__ ws, GemmArgs a, int bm, int bn) {
     const int lid = a.main_wgs + blockIdx.y;
     constexpr int GM = 8;
@@ -801,21 +860,28 @@ __global__ __launch_bounds__(256) void tail_reduce_conv_kernel(const float* __re
     const int r = i / bn, c = i - r * bn;
     const int row = tm * bm + r;                         // output channel
     if (row >= a.M) return;
-    const int img = tn / a.cv_tpi, t = tn - img * a.cv_tpi;
-    const long HW = (long)a.cv_h * a.cv_w;
-    float* dst = a.C + ((long)img * a.M + row) * HW;
     const float bias = a.cv_bias ? a.cv_bias[row] : 0.0f;
     const float o[4] = {s.x, s.y, s.z, s.w};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const int q = t * bn + c + j;
-        const int h = q / a.cv_wp, w = q - h * a.cv_wp;
-        if (h < a.cv_h && w < a.cv_w) {
+        long at = -1;                                     // where column c + j of the tile goes, if anywhere
+        if (a.conv == 3) {
+            const int img = tn / a.cv_tpi, t = tn - img * a.cv_tpi;
+            const int q = t * bn + c + j;
+            const int h = q / a.cv_wp, w = q - h * a.cv_wp;
+            if (h < a.cv_h && w < a.cv_w) at = ((long)img * a.M + row) * ((long)a.cv_h * a.cv_w) + (long)h * a.cv_w + w;
+        } else {
+            const int n = tn * bn + c + j;
+            const int HW = (int)a.cv_plane;
+            const int img = n / HW;
+            if (n < a.N) at = ((long)img * a.M + row) * HW + (n - img * HW);
+        }
+        if (at >= 0) {
             float x = o[j];
             if (a.cv_bias) x += bias;
-            if (a.cv_mask) a.cv_mask[(dst - a.C) + (long)h * a.cv_w + w] = x >= 0.0f ? 1 : 0;
+            if (a.cv_mask) a.cv_mask[at] = x >= 0.0f ? 1 : 0;
             if (a.cv_relu) x = x * (x >= 0.0f ? 1.0f : 0.0f);
-            dst[(long)h * a.cv_w + w] = x;
+            a.C[at] = x;
         }
     }
 }
@@ -931,7 +997,8 @@ struct TileShape {
 };
 
 // Tile shapes on offer; the 128x128 default comes first and wins ties.
-static const TileShape kShapes[] = {{128, 128}, {128, 96}, {128, 64}, {128, 32}, {96, 128}, {64, 128}};
+static const TileShape kShapes[] = {{128, 128}, {128, 96}, {128, 64}, {128, 32}, {96, 128}, {64, 128}, {32, 128}};
+constexpr int kPlainShapes = 6;      // the last shape exists for the column-buffer forward product only
 
 template <bool AKC, bool BKC, bool PIPE>
 static void launch_shape(int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
@@ -949,7 +1016,14 @@ static void launch_shape(int shape, dim3 grid, hipStream_t st, const GemmArgs& a
 // implicit-convolution variants
 static void launch_conv(int mode, int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
     dim3 block(kGemmThreads);
-    if (mode == 3) {
+    if (mode == 1) {
+        switch (shape) {
+            case 0: sgemm_kernel<true, true, false, 2, 2, 2, 2, false, 1><<<grid, block, 0, st>>>(a); break;
+            case 4: sgemm_kernel<true, true, false, 1, 4, 3, 1, false, 1><<<grid, block, 0, st>>>(a); break;
+            case 5: sgemm_kernel<true, true, false, 1, 4, 2, 1, false, 1><<<grid, block, 0, st>>>(a); break;
+            default: sgemm_kernel<true, true, false, 1, 4, 1, 1, false, 1><<<grid, block, 0, st>>>(a); break;    // 32 x 128
+        }
+    } else if (mode == 3) {
         switch (shape) {
             case 0: sgemm_kernel<true, false, false, 2, 2, 2, 2, false, 3><<<grid, block, 0, st>>>(a); break;
             case 4: sgemm_kernel<true, false, false, 1, 4, 3, 1, false, 3><<<grid, block, 0, st>>>(a); break;    // 96 x 128
@@ -973,13 +1047,13 @@ static void launch_conv(int mode, int shape, dim3 grid, hipStream_t st, const Ge
 //   mode 3: `rows` output channels x 128 pixels per tile; the K slices need whole blocks of 16 channels;
 //   mode 2: `rows` filters x `cols` = taps * channels.
 static int conv_shape(int mode, long rows, long cols, long channels) {
-    if (channels % KT != 0 || rows < 1) return -1;
+    if ((mode != 1 && channels % KT != 0) || rows < 1) return -1;
     int best = -1;
     double best_work = 0;
-    for (int i = 0; i < (int)(sizeof(kShapes) / sizeof(kShapes[0])); ++i) {
-        if (mode == 3 && kShapes[i].bn != 128) continue;
+    for (int i = 0; i < (mode == 1 ? kPlainShapes + 1 : kPlainShapes); ++i) {
+        if (mode != 2 && kShapes[i].bn != 128) continue;
         const double work = (double)(cdiv(rows, kShapes[i].bm) * kShapes[i].bm) *
-                            (mode == 3 ? 1.0 : (double)(cdiv(cols, kShapes[i].bn) * kShapes[i].bn));
+                            (mode != 2 ? 1.0 : (double)(cdiv(cols, kShapes[i].bn) * kShapes[i].bn));
         if (best < 0 || work < best_work * 0.97) {
             best = i;
             best_work = work;
@@ -1024,7 +1098,7 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     // tile shape: least padded work, ties to the earlier (larger) shape
     int shape = 0;
     double best = 0;
-    for (int i = 0; i < (int)(sizeof(kShapes) / sizeof(kShapes[0])); ++i) {
+    for (int i = 0; i < kPlainShapes; ++i) {
         const double work = (double)(cdiv(M, kShapes[i].bm) * kShapes[i].bm) *
                             (double)(cdiv(N, kShapes[i].bn) * kShapes[i].bn);
         if (i == 0 || work < best * 0.97) {
@@ -1047,16 +1121,24 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
         if (!p) ws_rc = CGT_AMD_ERR_HIP;
         return p;
     };
-    if (cv) {
+    const bool per_image_k = cv && cv->mode == 4;     // plain kernel, K cut per image
+    const bool conv_kernel = cv && !per_image_k;
+    const bool writes_nchw = cv && (cv->mode == 1 || cv->mode == 3);
+    if (conv_kernel) {
         shape = conv_shape(cv->mode, M, N, cv->C);
         CGT_ARG_CHECK(cv->mode != 3 || (long)cv->tpi * cv->B * 128 == N, "sgemm_conv: mode 3 takes whole tiles of pixels");
         CGT_ARG_CHECK(shape >= 0, "sgemm_conv: the image must have a multiple of 16 channels");
         // lane offsets are 32-bit: a tile's rows (mode 2: the channels of a whole image) span less than 4 GB
-        CGT_ARG_CHECK(cv->plane < (1L << 23) && (cv->mode != 2 || cv->C * cv->plane < (1L << 30)),
+        CGT_ARG_CHECK(cv->mode == 1 || (cv->plane < (1L << 23) && (cv->mode != 2 || cv->C * cv->plane < (1L << 30))),
                       "sgemm_conv: padded planes too large");
+        // mode 1: a lane's offset spans the images a tile of 128 columns touches
+        CGT_ARG_CHECK(cv->mode != 1 || (cv->plane >= 1 && cv->plane < (1L << 31) && cv->B * cv->plane == N &&
+                                        (127 / cv->plane + 2) * M * cv->plane < (1L << 30)),
+                      "sgemm_conv: column-buffer product too large");
     }
     GemmArgs a;
-    a.conv = cv ? cv->mode : 0;
+    a.conv = conv_kernel ? cv->mode : 0;
+    a.kimg = 0; a.kspi = 1; a.aimg = 0;
     if (cv) {
         a.cv_wp = cv->wp; a.cv_kw = cv->kw; a.cv_kh = cv->kh; a.cv_c = (int)cv->C;
         a.cv_tpi = (int)cv->tpi; a.cv_spi = (int)cv->spi;
@@ -1077,8 +1159,43 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     a.splits = 1;
     a.kchunk = (int)(cdiv(std::max(K, 1L), KT) * KT);
     a.ws = nullptr;
-    a.wide = (!cv && (lda >= (1L << 23) || ldb >= (1L << 23))) ? 1 : 0;
-    if (P == 1 && tiles < 512 && K >= 64 * KT && !(cv && cv->mode == 3)) {
+    const bool implicit = cv && (cv->mode == 2 || cv->mode == 3);     // operands read from padded planes
+    a.wide = (!implicit && (lda >= (1L << 23) || ldb >= (1L << 23))) ? 1 : 0;
+    if (per_image_k) {
+        // one split per piece of an image: K = B * kimg, A = [B][M][kimg]
+        const long kimg = cv->plane;
+        CGT_ARG_CHECK(kimg >= 1 && cv->B >= 1 && cv->B * kimg == K && lda == kimg, "sgemm_conv: per-image K does not match the operands");
+        // pieces per image: every CU should get the same number of workgroups, about four (they
+        // are resident together), with at least 8 slices per piece and a workspace <= 256 MiB ...
+        const long cap = (256L << 20) / (M * N * (long)sizeof(float));
+        const long max_pieces = std::max(1L, std::min({kimg / (8 * KT), cap / cv->B, 64L}));
+        long pieces = 1;
+        double best_cost = 0;
+        for (long p = 1; p <= max_pieces; ++p) {
+            const long wgs = tiles * cv->B * p;
+            // time ~ the busiest CU's share of the work; too few workgroups per CU leave latency uncovered;
+            // every piece costs a partial result written and read back
+            const double busiest = (double)cdiv(wgs, kNumCU) * kNumCU / wgs;
+            const double cover = wgs >= 3L * kNumCU ? 1.0 : 1.0 + 0.15 * (3.0 - (double)wgs / kNumCU);
+            const double cost = busiest * cover + 0.01 * p;
+            if (p == 1 || cost < best_cost - 1e-9) {
+                best_cost = cost;
+                pieces = p;
+            }
+        }
+        a.kchunk = (int)(cdiv(cdiv(kimg, pieces), KT) * KT);
+        pieces = cdiv(kimg, a.kchunk);
+        CGT_ARG_CHECK(cv->B * pieces < (1L << 20) && cv->B * pieces * M * N < (1L << 29),   // ... 2 GiB at the very most
+                      "sgemm_conv: too many images for the weight gradient's partial sums");
+        a.kimg = (int)kimg;
+        a.kspi = (int)pieces;
+        a.aimg = (M - 1) * kimg;
+        a.splits = (int)(cv->B * pieces);
+        if (a.splits > 1) {
+            a.ws = workspace((size_t)a.splits * M * N * sizeof(float));
+            if (!a.ws) return ws_rc;
+        }
+    } else if (P == 1 && tiles < 512 && K >= 64 * KT && !writes_nchw) {
         long want = std::max(1L, 1024 / tiles);
         want = std::min(want, K / (8 * KT));                    // at least 8 slices per split
         const long cap = (256L << 20) / (M * N * (long)sizeof(float));  // workspace <= 256 MiB
@@ -1133,7 +1250,7 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     // and load in bursts) with a long K range each
     const long slices = cdiv(a.splits > 1 ? (long)a.kchunk : K, KT);
     const bool deep = !cv && shape == 0 && !(!tA && tB) && wgs <= 4L * kNumCU && slices >= 32;
-    if (cv) launch_conv(cv->mode, shape, grid, st, a);
+    if (conv_kernel) launch_conv(cv->mode, shape, grid, st, a);
     else launch_trans(tA, tB, pipe, deep, shape, grid, st, a);
     CGT_LAUNCH_CHECK("sgemm_kernel");
     if (a.splits > 1) {
@@ -1144,7 +1261,7 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
         if (vec) splitk_reduce_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a.ws, C, MN, (int)N, ldc, a.splits);
         else splitk_reduce_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a.ws, C, MN, (int)N, ldc, a.splits);
         CGT_LAUNCH_CHECK("splitk_reduce_kernel");
-    } else if (tail_tiles > 0 && cv && cv->mode == 3) {
+    } else if (tail_tiles > 0 && writes_nchw) {
         tail_reduce_conv_kernel<<<dim3((unsigned)cdiv(kShapes[shape].bm * kShapes[shape].bn, 1024), (unsigned)tail_tiles), dim3(256), 0, st>>>(
             a.ws, a, kShapes[shape].bm, kShapes[shape].bn);
         CGT_LAUNCH_CHECK("tail_reduce_conv_kernel");
@@ -1159,6 +1276,10 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
 int sgemm_conv(const ConvGemm& cv, long M, long N, const float* A, const float* B, float* C, long ldc,
                void* stream) {
     const long taps = (long)cv.kh * cv.kw;
+    if (cv.mode == 1)   // A = filters [M][K], B = column buffer [N][K] with K = C (the patch length); C is NCHW, written by the kernel
+        return gemm_dispatch(0, 1, 1, M, N, cv.C, A, cv.C, 0, B, cv.C, 0, C, N, 0, stream, false, &cv);
+    if (cv.mode == 4)   // A = cotangent [B][M][plane], B = column buffer [B * plane][N]; C = [M][N]
+        return gemm_dispatch(0, 0, 1, M, N, cv.B * cv.plane, A, cv.plane, 0, B, N, 0, C, ldc, 0, stream, false, &cv);
     if (cv.mode == 3)   // A = filters [M][taps * C], B = image (row-contiguous operand); C is NCHW, written by the kernel
         return gemm_dispatch(0, 0, 1, M, N, taps * cv.C, A, taps * cv.C, 0, B, N, 0, C, N, 0, stream, false, &cv);
     // A = cotangent planes [B][M][plane], B = image; K runs over (image, pixel slice)

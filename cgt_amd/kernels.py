@@ -328,3 +328,41 @@ def conv_same_bwd_filter(gypad, xpad, xshape, fshape, out=None, stream=None):
     gf = _out(out, tuple(fshape))
     capi.check(capi.lib().cgt_amd_conv_same_bwd_filter_f32(gypad.ptr, xpad.ptr, B, C, H, W, L, kh, kw, gf.ptr, stream))
     return gf
+
+
+def conv_col_fwd(col, f, bias=None, relu=False, out=None, mask=None, stream=None):
+    """y [B,L,m,n] = conv2d from the column buffer col [B,m,n,Z] and the filters f [L,C,kh,kw]
+    (Z = C*kh*kw), written in NCHW by the product itself; optional fused bias add and rectify."""
+    _f32(col, f)
+    B, m, n, Z = col.shape
+    L = f.shape[0]
+    if int(np.prod(f.shape[1:])) != Z:
+        raise ValueError("filters %s do not match patches of %d" % (tuple(f.shape), Z))
+    y = _out(out, (B, L, m, n))
+    capi.check(capi.lib().cgt_amd_conv_col_fwd_f32(col.ptr, f.ptr, None if bias is None else bias.ptr, int(bool(relu)),
+                                                   B, m * n, Z, L, y.ptr, None if mask is None else mask.ptr, stream))
+    return y
+
+
+def conv_col_bwd_data(gy, f, out=None, stream=None):
+    """gcol [B,m,n,Z] from the NCHW cotangent gy [B,L,m,n] and the filters."""
+    _f32(gy, f)
+    B, L, m, n = gy.shape
+    if f.shape[0] != L:
+        raise ValueError("cotangent has %d channels, the filter bank %d filters" % (L, f.shape[0]))
+    Z = int(np.prod(f.shape[1:]))
+    gcol = _out(out, (B, m, n, Z))
+    capi.check(capi.lib().cgt_amd_conv_col_bwd_data_f32(gy.ptr, f.ptr, B, m * n, Z, L, gcol.ptr, stream))
+    return gcol
+
+
+def conv_col_bwd_filter(gy, col, fshape, out=None, stream=None):
+    """gf [L,C,kh,kw] from the NCHW cotangent gy [B,L,m,n] and the column buffer."""
+    _f32(gy, col)
+    B, L, m, n = gy.shape
+    Z = col.shape[3]
+    if tuple(col.shape[:3]) != (B, m, n) or int(np.prod(fshape)) != L * Z:
+        raise ValueError("cotangent %s, columns %s and filters %s do not match" % (tuple(gy.shape), tuple(col.shape), tuple(fshape)))
+    gf = _out(out, tuple(fshape))
+    capi.check(capi.lib().cgt_amd_conv_col_bwd_filter_f32(gy.ptr, col.ptr, B, m * n, Z, L, gf.ptr, stream))
+    return gf

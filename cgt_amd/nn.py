@@ -1,16 +1,19 @@
 """cgt.nn front end of the CNN hot path (reference cgt/nn.py:85-111).
 
-conv2d keeps the reference's CPU-path composition
+The reference's CPU path composes conv2d as
     im2col -> reshape -> Mul22(False, True) -> reshape -> transpose{0,3,1,2}
-with every op running on the GPU.  Where the reference's devtype == "gpu"
-branch switches to fused convolution ops (cuDNN, cgt/nn.py:88-93), this build
-switches to its own fused ops for the layers they cover -- stride 1, pad =
-(kernel - 1) / 2, channel and filter counts their GEMM tiles fit (nn_ops/
-conv_same.py) -- which need no column buffer; conv_algo("im2col") keeps the
-composition for every layer.
+and its devtype == "gpu" branch switches to fused convolution ops (cuDNN,
+cgt/nn.py:88-93).  This build's GPU branch switches to its own fused ops:
+  * stride 1, pad = (kernel - 1) / 2, channel and filter counts in multiples
+    of 16: products that read a zero-padded copy of the image, no column
+    buffer (nn_ops/conv_same.py);
+  * every other layer: Im2Col, then products that write / read the NCHW
+    arrays themselves, no transposes (nn_ops/conv_col.py) -- conv_algo("col")
+    uses these for every layer;
+conv_algo("im2col") keeps the literal composition, every op on the GPU.
 """
 from . import core
-from .nn_ops import conv_same
+from .nn_ops import conv_col, conv_same
 from .nn_ops.cross_channel_lrn import cross_channel_lrn  # noqa: F401
 from .nn_ops.im2col import im2col
 from .nn_ops.max_pool_2d import MaxPool, PoolInfo
@@ -20,12 +23,14 @@ _CONV_ALGO = "auto"
 
 
 def conv_algo(name=None):
-    """Select how conv2d is built: "auto" (fused ops where they apply) or "im2col"
-    (always the im2col -> Mul22 composition).  Returns the previous setting."""
+    """Select how conv2d is built: "auto" (the fused ops without a column buffer where
+    they apply, those over the column buffer elsewhere), "col" (always the fused ops over
+    the column buffer) or "im2col" (always the literal im2col -> Mul22 -> transpose
+    composition).  Returns the previous setting."""
     global _CONV_ALGO
     old = _CONV_ALGO
     if name is not None:
-        assert name in ("auto", "im2col")
+        assert name in ("auto", "col", "im2col")
         _CONV_ALGO = name
     return old
 
@@ -37,6 +42,8 @@ def conv2d(x_BKRC, f_LKrc, kernelshape, pad=(0, 0), stride=(1, 1)):
     if _CONV_ALGO == "auto" and conv_same.supported(x_BKRC, f_LKrc, kernelshape, pad, stride):
         return conv_same.conv_same(x_BKRC, f_LKrc, kernelshape)
     col_BmnZ = im2col(x_BKRC, kernelshape, pad, stride)
+    if _CONV_ALGO != "im2col":
+        return conv_col.conv_col(col_BmnZ, f_LKrc)
     f_LZ = f_LKrc.reshape([L, K * r * c])
     B, m, n, Z = col_BmnZ.shape
     col_Bmn_Z = col_BmnZ.reshape([B * m * n, Z])
@@ -62,8 +69,12 @@ def rectify(x):
     """ReLU as the reference builds it: x * (x >= 0) (cgt/nn.py:44-45).  On the result of a
     fused convolution it becomes part of that op (same values, same gradient)."""
     x = core.as_node(x)
-    if _CONV_FUSION and isinstance(x.op, conv_same.ConvForward) and not x.op.relu:
-        return conv_same.rectified(x)
+    if _CONV_FUSION and isinstance(x.op, (conv_same.ConvForward, conv_col.ConvColForward)) and not x.op.relu:
+        # the same inputs run again with the rectify in the epilogue.  Nodes are evaluated as
+        # they are built, so this costs a second product while the graph is traced; a compiled
+        # function replays only the fused one (the plain result is no longer reachable from
+        # the outputs)
+        return core.Result(x.op.with_relu(), x.parents)[0]
     return x * (x >= 0)
 
 
@@ -91,6 +102,9 @@ class SpatialConvolution(object):
         if (_CONV_FUSION and _CONV_ALGO == "auto"
                 and conv_same.supported(x, self.weight, self.kernelshape, self.pad, self.stride)):
             return conv_same.conv_same(x, self.weight, self.kernelshape, bias=self.bias)
+        if _CONV_FUSION and _CONV_ALGO != "im2col":
+            col = im2col(x, self.kernelshape, self.pad, self.stride)
+            return conv_col.conv_col(col, self.weight, bias=self.bias)
         tmp = conv2d(x, self.weight, self.kernelshape, self.pad, self.stride)
         return core.broadcast("+", tmp, self.bias, "xxxx,1x11")
 

@@ -86,6 +86,9 @@ class ConvForward(core.Op):
     def __init__(self, info, has_bias=False, relu=False):
         self.info, self.has_bias, self.relu = info, bool(has_bias), bool(relu)
 
+    def with_relu(self):
+        return ConvForward(self.info, self.has_bias, True)
+
     def get_diff(self, _):
         return [True, False, True] + ([True] if self.has_bias else [])
 
@@ -225,13 +228,3 @@ def conv_same(x, f, kernelshape, bias=None, relu=False):
     parents = [x, xpad, f] + ([core.as_node(bias)] if bias is not None else [])
     out = core.Result(ConvForward(info, bias is not None, relu), parents)
     return out[0] if relu else out
-
-
-def rectified(node):
-    """The rectify of a ConvForward result as ONE fused op: the same inputs run again with
-    the rectify in the epilogue.  Nodes are evaluated as they are built, so this costs a
-    second product while the graph is traced; a compiled function replays only the fused
-    one (the plain result is no longer reachable from the outputs)."""
-    op = node.op
-    assert isinstance(op, ConvForward) and not op.relu
-    return core.Result(ConvForward(op.info, op.has_bias, True), node.parents)[0]

@@ -355,6 +355,33 @@ int cgt_amd_conv_same_bwd_data_f32(const float *gypad, const float *f, long B, l
 int cgt_amd_conv_same_bwd_filter_f32(const float *gypad, const float *xpad, long B, long C, long H,
                                      long W, long L, int kh, int kw, float *gf, void *stream);
 
+/* ---------------------------------------------------------------- convolution over the column buffer
+ *
+ * conv2d of any geometry as the reference composes it on the CPU -- im2col,
+ * one GEMM, reshape, Transpose{0,3,1,2} (cgt/nn.py:95-100), and for the
+ * gradients Transpose{0,2,3,1} followed by the NN / TN GEMMs that autodiff
+ * derives (cgt/core.py:2143-2175) -- with the [B*m*n, L] intermediates and
+ * both transposes folded into the GEMMs: each product reads or writes the
+ * NCHW array in place.  Same sums in the same order of z as the composition
+ * (results agree with it to GEMM accuracy; the split of the weight gradient's
+ * K axis differs).  In all three: col [B*P][Z] is cgt_amd_im2col_f32's
+ * result (P = m*n output pixels per image, Z = C*kh*kw), f [L][Z] is the
+ * filter bank [L,C,kh,kw] as it is stored, y / gy are [B,L,m,n]. */
+
+/* y = conv(x, f) from col.  bias / relu / mask as in cgt_amd_conv_same_fwd_f32. */
+int cgt_amd_conv_col_fwd_f32(const float *col, const float *f, const float *bias, int relu,
+                             long B, long P, long Z, long L, float *y, signed char *mask,
+                             void *stream);
+
+/* gcol [B*P][Z] (the argument of cgt_amd_col2im_f32) from the cotangent gy. */
+int cgt_amd_conv_col_bwd_data_f32(const float *gy, const float *f, long B, long P, long Z, long L,
+                                  float *gcol, void *stream);
+
+/* gf [L,C,kh,kw] from the cotangent gy and col.  Uses a workspace owned by
+ * the library (one partial sum per image, or per piece of an image). */
+int cgt_amd_conv_col_bwd_filter_f32(const float *gy, const float *col, long B, long P, long Z, long L,
+                                    float *gf, void *stream);
+
 /* ---------------------------------------------------------------- conv glue */
 
 /* out[i0,i1,i2,i3] = in[...] with out.shape[d] = in.shape[axes[d]].

@@ -330,18 +330,18 @@ class LayerOnGpu(object):
             PH, PW = K.pool_outsize(H, pk[0], pp[0], ps[0]), K.pool_outsize(W, pk[1], pp[1], ps[1])
             self.pool, self.mask = empty((B, L, PH, PW)), empty((B, L, PH, PW), np.int32)
             self.gpool = to_gpu(np.ones((B, L, PH, PW), np.float32))
-            self.gact = empty(self.y.shape)
             st.append(Stage("max_pool_fwd", "max_pool_fwd_kernel", lambda: K.max_pool(act, pk, pp, ps, out=(self.pool, self.mask), stream=s),
                             4 * (nelem(self.y) + 2 * nelem(self.pool)), "hbm"))
-            st.append(Stage("max_pool_bwd", "max_pool_bwd_block_kernel",
-                            lambda: K.max_pool_pullback(self.y.shape, self.mask, self.gpool, pk, pp, ps, out=self.gact, stream=s),
-                            4 * (2 * nelem(self.pool) + nelem(self.y)), "hbm"))
-            gy = self.gact
+            # the pool's pullback writes the padded cotangent itself (what the Op graph builds:
+            # ConvPadPoolPullback in the place of MaxPoolPullback -> ConvPad)
+            st.append(Stage("max_pool_bwd_padded", "max_pool_bwd_padded_kernel",
+                            lambda: K.conv_same_pad_pool_pullback(self.y.shape, self.mask, self.gpool, pk, pp, ps, (r, c),
+                                                                  out=self.gypad, stream=s),
+                            4 * (2 * nelem(self.pool) + nelem(self.gypad)), "hbm"))
         else:
-            gy = to_gpu(np.ones(self.y.shape, np.float32))
-        self.gy = gy
-        st.append(Stage("pad_gy", "pad_planes_kernel", lambda: K.conv_same_pad(self.gy, (r, c), out=self.gypad, stream=s),
-                        4 * (nelem(self.y) + nelem(self.gypad)), "hbm"))
+            self.gy = to_gpu(np.ones(self.y.shape, np.float32))
+            st.append(Stage("pad_gy", "pad_planes_kernel", lambda: K.conv_same_pad(self.gy, (r, c), out=self.gypad, stream=s),
+                            4 * (nelem(self.y) + nelem(self.gypad)), "hbm"))
         st.append(Stage("filter_flip", "flip_filters_kernel",
                         lambda: call(lib.cgt_amd_conv_same_filter_f32, self.f.ptr, L, C, r, c, 1, self.fflip.ptr, s), 8 * L * Z, "hbm"))
         st.append(Stage("gemm_dgrad", "sgemm_kernel",

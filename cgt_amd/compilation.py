@@ -226,6 +226,7 @@ def prebuild_standard_ops():
         (nn_ops.conv_same.ConvForward(cinfo, True, True), [T4, T1, T4, T4]),
         (nn_ops.conv_same.ConvBackwardData(cinfo), [T1, T4, T4]),
         (nn_ops.conv_same.ConvBackwardFilter(cinfo), [T1, T1, T4, T4]),
+        (nn_ops.conv_same.ConvPadPoolPullback(cinfo, pinfo), [T4, T4, I4, T4]),
         (nn_ops.conv_col.ConvColForward(), [T4, T4]),
         (nn_ops.conv_col.ConvColForward(True, True), [T4, T4, T4]),
         (nn_ops.conv_col.ConvColBackwardData(), [T4, T4, T4]),

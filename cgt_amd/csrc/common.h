@@ -48,6 +48,20 @@ int sgemm_conv(const ConvGemm& cv, long M, long N, const float* A, const float* 
 // 1 if sgemm_conv has a tile shape for these extents (output channels of the product, channels of the image)
 bool sgemm_conv_supported(int mode, long filters, long channels);
 
+// The pullback of a max pool (pool.hip) written straight into a convolution's zero-padded
+// layout (conv.hip): what cgt_amd_max_pool_pullback_f32 followed by cgt_amd_conv_same_pad_f32
+// leaves, in one pass.  Plane p of the result: `lead` zeros, then rows of `pitch` floats with
+// the H x W pullback starting at row `top`; `plane` floats per plane (a multiple of 4), then
+// `tail` zero floats after the last plane.  relu_mask (int8 [planes][H][W] or null) multiplies
+// each cell as (float)mask * value.
+struct PaddedPlanes {
+    int lead, top, pitch, plane;
+    long tail;
+};
+int launch_pool_pullback_padded(const int* mask, const float* top_diff, const signed char* relu_mask, long nplanes,
+                                long H, long W, int kh, int kw, int ph, int pw, int sh, int sw, long PH, long PW,
+                                const PaddedPlanes& lay, float* dst, void* stream);
+
 constexpr int kWave = 64;    // CDNA wavefront width
 constexpr int kNumXCD = 8;   // MI355X: 8 accelerator dies, each with its own L2
 constexpr int kNumCU = 256;  // MI355X compute units

@@ -130,6 +130,22 @@ CGT_API int cgt_amd_conv_same_pad_f32(const float* x, long planes, long H, long 
     return CGT_AMD_OK;
 }
 
+// gypad = pad(relu_mask * max_pool_pullback(mask, top_diff)): the cotangent of a convolution whose
+// result went through (a rectify and) a max pool, in the layout the gradient products read, without
+// the unpadded array in between
+CGT_API int cgt_amd_conv_same_pad_pool_pullback_f32(const int* mask, const float* top_diff, const signed char* relu_mask,
+                                                    long planes, long H, long W, int pool_kh, int pool_kw, int pool_ph,
+                                                    int pool_pw, int pool_sh, int pool_sw, long PH, long PW, int kh, int kw,
+                                                    float* gypad, void* stream) {
+    SameGeom g;
+    int rc = check_same("conv_same_pad_pool_pullback", g, 1, 1, H, W, 1, kh, kw);
+    if (rc) return rc;
+    CGT_ARG_CHECK(planes >= 0 && gypad, "conv_same_pad_pool_pullback: bad arguments");
+    const PaddedPlanes lay = {g.pw, g.ph, (int)g.Wp, (int)g.plane, g.tail};
+    return launch_pool_pullback_padded(mask, top_diff, relu_mask, planes, H, W, pool_kh, pool_kw, pool_ph, pool_pw, pool_sh,
+                                       pool_sw, PH, PW, lay, gypad, stream);
+}
+
 // ---- the pieces (each one kernel plus, for the products, the GEMM's own reduce kernel)
 
 CGT_API int cgt_amd_conv_same_filter_f32(const float* f, long L, long C, int kh, int kw, int flipped, float* fk,

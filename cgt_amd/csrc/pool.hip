@@ -321,6 +321,111 @@ __global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_direct_kernel(
     }
 }
 
+// The pullback written into zero-padded planes (see PaddedPlanes): one thread per aligned
+// 16-byte unit of the result.  A unit's four floats are zeros of the padding or pullback cells;
+// a cell gathers the windows that cover it in ascending (ph, pw), as max_pool_bwd_kernel does,
+// straight from global memory (neighbouring threads read neighbouring pooled cells).  With a
+// compile-time geometry the candidate windows of a cell are a fixed-size neighbourhood: all
+// their loads are issued up front, unconditionally (indices of windows that do not exist are
+// clamped to 0 and their values dropped), instead of one dependent load after another.
+template <class G>
+__global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_padded_kernel(
+    G g, const int* __restrict__ mask, const float* __restrict__ top_diff, const signed char* __restrict__ relu_mask,
+    float* __restrict__ dst, int H, int W, int PH, int PW, PaddedPlanes lay, int units_per_plane,
+    long total_units, long tail_units) {
+    const float rPitch = 1.0f / (float)lay.pitch;
+    const int PP = PH * PW, HW = H * W;
+    const int lane = threadIdx.x & 63;
+    // A wavefront takes chunks of kChunk units of one plane at a time, so the plane and with it
+    // the base addresses of its mask / cotangent / output are wave-uniform (scalar registers,
+    // 32-bit lane offsets) -- the kernel is bound by its index arithmetic, not by memory.
+    constexpr int kChunk = 512;
+    const int chunks_per_plane = (units_per_plane + kChunk - 1) / kChunk;
+    const int items = (int)(total_units / units_per_plane) * chunks_per_plane;     // < 2^31: the host checks
+    const int nwaves = (int)gridDim.x * (kPoolThreads / 64);
+    const int wave_id = __builtin_amdgcn_readfirstlane((int)((blockIdx.x * kPoolThreads + threadIdx.x) >> 6));
+    for (long t = (long)blockIdx.x * kPoolThreads + threadIdx.x; t < tail_units; t += (long)gridDim.x * kPoolThreads)
+        stream_store4(dst + (total_units + t) * 4, 0.f, 0.f, 0.f, 0.f);
+    for (int item = wave_id; item < items; item += nwaves) {
+        const long pl = item / chunks_per_plane;
+        const int chunk = item - (int)pl * chunks_per_plane;
+        const int* mk = mask + pl * PP;
+        const float* td = top_diff + pl * PP;
+        const signed char* rmk = relu_mask ? relu_mask + pl * HW : nullptr;
+        float* out = dst + pl * (long)lay.plane;
+        const int uend = min(units_per_plane, (chunk + 1) * kChunk);
+        for (int uu = chunk * kChunk + lane; uu < uend; uu += 64) {
+            float o[4] = {0.f, 0.f, 0.f, 0.f};
+            const int e0 = uu * 4;
+            // element e of a plane is column (e - lead) % pitch of padded row (e - lead) / pitch;
+            // shifted by one row so that it is never negative (lead <= pitch), fixed up exactly
+            const int e1 = e0 - lay.lead + lay.pitch;
+            int hp = fastdiv(e1, rPitch);
+            int wp = e1 - hp * lay.pitch;
+            if (wp < 0) { --hp; wp += lay.pitch; }
+            if (wp >= lay.pitch) { ++hp; wp -= lay.pitch; }
+            if constexpr (G::is_static) {
+                constexpr int NY = (G::kKH + G::kSH - 1) / G::kSH, NX = (G::kKW + G::kSW - 1) / G::kSW;
+                int mv[4][NY][NX], cell[4];
+                float tv[4][NY][NX], rm[4];
+                bool ok[4][NY][NX], inside[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int h = hp - 1 - lay.top;
+                    inside[j] = h >= 0 && h < H && wp < W;
+                    cell[j] = h * W + wp;
+                    const int yb = floordiv(h + g.ph() - g.kh(), g.sh()) + 1, y1 = min(PH - 1, (h + g.ph()) / g.sh());
+                    const int xb = floordiv(wp + g.pw() - g.kw(), g.sw()) + 1, x1 = min(PW - 1, (wp + g.pw()) / g.sw());
+#pragma unroll
+                    for (int dy = 0; dy < NY; ++dy)
+#pragma unroll
+                        for (int dx = 0; dx < NX; ++dx) {
+                            const int y = yb + dy, x = xb + dx;
+                            ok[j][dy][dx] = inside[j] && y >= 0 && y <= y1 && x >= 0 && x <= x1;
+                            const int at = ok[j][dy][dx] ? y * PW + x : 0;
+                            mv[j][dy][dx] = mk[at];
+                            tv[j][dy][dx] = td[at];
+                        }
+                    rm[j] = (rmk && inside[j]) ? (float)rmk[cell[j]] : 1.0f;
+                    if (++wp == lay.pitch) { wp = 0; ++hp; }
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float acc = 0.0f;
+#pragma unroll
+                    for (int dy = 0; dy < NY; ++dy)
+#pragma unroll
+                        for (int dx = 0; dx < NX; ++dx)
+                            acc = (ok[j][dy][dx] && mv[j][dy][dx] == cell[j]) ? acc + tv[j][dy][dx] : acc;
+                    if (rmk) acc = rm[j] * acc;
+                    o[j] = inside[j] ? acc : 0.0f;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int h = hp - 1 - lay.top;
+                    if (h >= 0 && h < H && wp < W) {
+                        const int cell = h * W + wp;
+                        const int y0 = max(0, floordiv(h + g.ph() - g.kh(), g.sh()) + 1), y1 = min(PH - 1, (h + g.ph()) / g.sh());
+                        const int x0 = max(0, floordiv(wp + g.pw() - g.kw(), g.sw()) + 1), x1 = min(PW - 1, (wp + g.pw()) / g.sw());
+                        float acc = 0.0f;
+                        for (int y = y0; y <= y1; ++y)
+                            for (int x = x0; x <= x1; ++x) {
+                                const int m = mk[y * PW + x];
+                                const float t = td[y * PW + x];
+                                acc = (m == cell) ? acc + t : acc;
+                            }
+                        if (rmk) acc = (float)rmk[cell] * acc;
+                        o[j] = acc;
+                    }
+                    if (++wp == lay.pitch) { wp = 0; ++hp; }
+                }
+            }
+            *reinterpret_cast<float4*>(out + e0) = make_float4(o[0], o[1], o[2], o[3]);
+        }
+    }
+}
+
 static int check_pool(const char* what, long N, long C, long H, long W, int kh, int kw, int ph,
                       int pw, int sh, int sw, long PH, long PW) {
     CGT_ARG_CHECK(N >= 0 && C >= 0 && H >= 0 && W >= 0 && PH >= 0 && PW >= 0, "%s: negative shape", what);
@@ -442,6 +547,39 @@ static int launch_pool_bwd(G g, const int* mask, const float* top_diff, long npl
             g, mask, top_diff, bottom_diff, total, (int)H, (int)W, (int)PH, (int)PW);
         CGT_LAUNCH_CHECK("max_pool_bwd_direct_kernel");
     }
+    return CGT_AMD_OK;
+}
+
+int launch_pool_pullback_padded(const int* mask, const float* top_diff, const signed char* relu_mask, long nplanes,
+                                long H, long W, int kh, int kw, int ph, int pw, int sh, int sw, long PH, long PW,
+                                const PaddedPlanes& lay, float* dst, void* stream) {
+    int rc = check_pool("pool_pullback_padded", nplanes, 1, H, W, kh, kw, ph, pw, sh, sw, PH, PW);
+    if (rc) return rc;
+    CGT_ARG_CHECK(dst && reinterpret_cast<uintptr_t>(dst) % 16 == 0, "pool_pullback_padded: the padded buffer must be 16-byte aligned");
+    CGT_ARG_CHECK(lay.plane % 4 == 0 && lay.tail % 4 == 0 && lay.plane < kFastdivLimit && lay.lead <= lay.pitch &&
+                  lay.lead + (lay.top + H) * (long)lay.pitch <= lay.plane && W <= lay.pitch && H * W < (1L << 30),
+                  "pool_pullback_padded: bad padded layout");
+    CGT_ARG_CHECK(nplanes == 0 || PH * PW == 0 || (mask && top_diff), "pool_pullback_padded: null pointer");
+    const long upp = lay.plane / 4, units = nplanes * upp, tail_units = lay.tail / 4;
+    if (units + tail_units == 0) return CGT_AMD_OK;
+    if (PH * PW == 0) return cgt_amd_fill_u32(dst, 0u, (units + tail_units) * 4, stream);     // no windows: all zeros
+    CGT_ARG_CHECK(nplanes * cdiv(upp, 512L) < (1L << 31) - (1L << 19), "pool_pullback_padded: too many planes");
+    // one wavefront per chunk of 512 units of a plane (grid-stride beyond 64 K workgroups)
+    const long blocks = std::max(1L, std::min(cdiv(nplanes * cdiv(upp, 512L), (long)(kPoolThreads / 64)), 1L << 16));
+    hipStream_t st = as_stream(stream);
+#define X(KH, KW, PH_, PW_, SH, SW)                                                                              \
+    if (kh == KH && kw == KW && ph == PH_ && pw == PW_ && sh == SH && sw == SW) {                                \
+        max_pool_bwd_padded_kernel<<<dim3((unsigned)blocks), dim3(kPoolThreads), 0, st>>>(                       \
+            StaticGeom<KH, KW, PH_, PW_, SH, SW>(), mask, top_diff, relu_mask, dst, (int)H, (int)W, (int)PH, (int)PW, lay, (int)upp, \
+            units, tail_units);                                                                                  \
+        CGT_LAUNCH_CHECK("max_pool_bwd_padded_kernel");                                                          \
+        return CGT_AMD_OK;                                                                                       \
+    }
+    CGT_STATIC_POOLS(X)
+#undef X
+    max_pool_bwd_padded_kernel<<<dim3((unsigned)blocks), dim3(kPoolThreads), 0, st>>>(
+        DynGeom{kh, kw, ph, pw, sh, sw}, mask, top_diff, relu_mask, dst, (int)H, (int)W, (int)PH, (int)PW, lay, (int)upp, units, tail_units);
+    CGT_LAUNCH_CHECK("max_pool_bwd_padded_kernel");
     return CGT_AMD_OK;
 }
 

@@ -298,6 +298,23 @@ def conv_same_pad(x, kernel, out=None, stream=None):
     return res
 
 
+def conv_same_pad_pool_pullback(xshape, mask, gtop, pool_kernel, pool_pad, pool_stride, kernel, relu_mask=None,
+                                out=None, stream=None):
+    """conv_same_pad(relu_mask * max_pool_pullback(xshape, mask, gtop, ...), kernel) in one pass,
+    bit for bit; relu_mask is an int8 array of shape xshape or None."""
+    _f32(gtop)
+    B, C, H, W = xshape
+    if mask.dtype != np.int32 or tuple(mask.shape) != tuple(gtop.shape) or tuple(mask.shape[:2]) != (B, C):
+        raise ValueError("mask %s / cotangent %s do not fit an input of shape %s" % (tuple(mask.shape), tuple(gtop.shape), tuple(xshape)))
+    if relu_mask is not None and (relu_mask.dtype != np.int8 or tuple(relu_mask.shape) != tuple(xshape)):
+        raise ValueError("the rectify mask must be an int8 array of the input's shape")
+    res = _out(out, (conv_same_padded_size(B * C, H, W, kernel),))
+    capi.check(capi.lib().cgt_amd_conv_same_pad_pool_pullback_f32(
+        mask.ptr, gtop.ptr, None if relu_mask is None else relu_mask.ptr, B * C, H, W, *_geom(pool_kernel, pool_pad, pool_stride),
+        mask.shape[2], mask.shape[3], int(kernel[0]), int(kernel[1]), res.ptr, stream))
+    return res
+
+
 def conv_same_fwd(xpad, f, xshape, bias=None, relu=False, out=None, mask=None, stream=None):
     """conv2d (stride 1, same padding) from the padded input; optional fused bias add and
     rectify; `mask` (int8 array of the output's shape) receives (pre-activation >= 0)."""

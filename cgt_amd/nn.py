@@ -62,6 +62,7 @@ def conv_fusion(on=None):
     old = _CONV_FUSION
     if on is not None:
         _CONV_FUSION = bool(on)
+        conv_same.FUSE_POOL_PULLBACK = bool(on)
     return old
 
 

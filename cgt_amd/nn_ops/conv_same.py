@@ -65,6 +65,57 @@ class ConvPad(core.Op):
                                       gpu_deref_mask=(True,))
 
 
+# Whether the padded cotangent of a convolution that feeds (a rectify and) a max pool is written
+# by the pool's pullback itself (ConvPadPoolPullback) instead of MaxPoolPullback -> (mask *) -> ConvPad
+FUSE_POOL_PULLBACK = True
+
+
+class ConvPadPoolPullback(core.Op):
+    """inputs [x, pool, mask, gpool] (+ [relu_mask]) -> ConvPad(relu_mask * MaxPoolPullback(x, pool, mask, gpool))
+    in one pass, bit for bit: the inputs are MaxPoolPullback's own (cgt/nn_ops/max_pool_2d.py:55-72,
+    only mask and gpool are read), x gives the shape."""
+    available_impls = ("native_gpu",)
+
+    def __init__(self, info, poolinfo, has_relu=False):
+        self.info, self.poolinfo, self.has_relu = info, poolinfo, bool(has_relu)
+
+    def get_diff(self, n):
+        return [False] * n
+
+    def shp_apply(self, inputs):
+        B, C, H, W = core.shape(inputs[0])
+        return [padded_size(B * C, H, W, self.info)]
+
+    def typ_apply(self, input_types):
+        return core.TensorType("f4", 1)
+
+    def get_native_compile_info(self, input_types, devtype):
+        assert devtype == "gpu"
+        from .max_pool_2d import info2closure as pool_closure
+        code = r"""
+            CGT_EXPORT_C void $function($closure* cl, cgtArray** reads, cgtArray* write) {
+                cgtArray *x = reads[0], *mask = reads[2], *gpool = reads[3], *rmask = cl->has_relu ? reads[4] : NULL;
+                const long* s = x->shape();
+                long need = cgt_amd_conv_same_padded_size(s[0] * s[1], s[2], s[3], cl->conv_kernel_h, cl->conv_kernel_w);
+                cgt_check(write->size() == need, "ConvPadPoolPullback: output has %ld floats, the geometry needs %ld", write->size(), need);
+                cgt_check(gpool->size() == mask->size() && mask->shape()[0] == s[0] && mask->shape()[1] == s[1] &&
+                          (!rmask || (rmask->size() == x->size() && rmask->dtype() == cgt_i1)),
+                          "ConvPadPoolPullback: mask, cotangent or rectify mask do not fit the input's shape");
+                if (cgtGlobalStatus != cgtStatusOK) return;
+                int rc = cgt_amd_conv_same_pad_pool_pullback_f32((const int*)mask->data(), (const float*)gpool->data(),
+                    rmask ? (const signed char*)rmask->data() : NULL, s[0] * s[1], s[2], s[3],
+                    cl->kernel_h, cl->kernel_w, cl->pad_h, cl->pad_w, cl->stride_h, cl->stride_w,
+                    mask->shape()[2], mask->shape()[3], cl->conv_kernel_h, cl->conv_kernel_w,
+                    (float*)write->data(), cgt_get_stream());
+                cgt_check(rc == CGT_AMD_OK, "ConvPadPoolPullback: %s", cgt_amd_last_error());
+            }"""
+        triples = pool_closure(self.poolinfo) + [("conv_kernel_h", ctypes.c_int, self.info.kernel_h),
+                                                 ("conv_kernel_w", ctypes.c_int, self.info.kernel_w),
+                                                 ("has_relu", ctypes.c_int, int(self.has_relu))]
+        return core.NativeCompileInfo(code, includes=["cgt_amd.h"], closure_triples=triples,
+                                      gpu_deref_mask=(False, False, True, True) + ((True,) if self.has_relu else ()))
+
+
 _CHECK_PADDED = r"""
                 long need = cgt_amd_conv_same_padded_size(%s, H, W, cl->kernel_h, cl->kernel_w);
                 cgt_check(%s->size() == need, "%s: padded operand has %%ld floats, the geometry needs %%ld", %s->size(), need);
@@ -105,18 +156,28 @@ class ConvForward(core.Op):
         return self.pullback_wanted(inputs, output, goutput, self.get_diff(len(inputs)))
 
     def pullback_wanted(self, inputs, output, goutput, wanted):
+        from .max_pool_2d import MaxPoolPullback
         x, xpad, f = inputs[:3]
-        if self.relu:
-            _y, mask = core.unpack(output)
-            gy = core.elwise_binary("*", mask, goutput[0])     # what x * (x >= 0) hands back: (x >= 0) * gz
-        else:
-            gy = goutput
+        gz = goutput[0] if self.relu else goutput
+        mask = core.unpack(output)[1] if self.relu else None
+        want_bias = self.has_bias and wanted[3]
+        # the cotangent comes out of a max pool and nothing but the padded copy needs it: the
+        # pool's pullback writes the padded copy itself (rectify mask applied on the way)
+        fuse_pool = FUSE_POOL_PULLBACK and isinstance(gz.op, MaxPoolPullback) and not want_bias
+        gy = None
+        if not fuse_pool:
+            # what x * (x >= 0) hands back: (x >= 0) * gz
+            gy = core.elwise_binary("*", mask, gz) if self.relu else gz
         gbias = None
-        if self.has_bias and wanted[3]:
+        if want_bias:
             gbias = core.sum(gy, axis=(0, 2, 3), keepdims=True)  # the pullback of the bias' Repeat
         gx = gf = None
         if wanted[0] or wanted[2]:
-            gypad = core.Result(ConvPad(self.info), [gy])
+            if fuse_pool:
+                gypad = core.Result(ConvPadPoolPullback(self.info, gz.op.info, self.relu),
+                                    list(gz.parents) + ([mask] if self.relu else []))
+            else:
+                gypad = core.Result(ConvPad(self.info), [gy])
             gx = core.Result(ConvBackwardData(self.info), [gypad, f, x]) if wanted[0] else None
             gf = core.Result(ConvBackwardFilter(self.info), [gypad, xpad, f, x]) if wanted[2] else None
         return [gx, None, gf] + ([gbias] if self.has_bias else [])

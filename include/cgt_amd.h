@@ -318,6 +318,19 @@ long cgt_amd_conv_same_padded_size(long planes, long H, long W, int kh, int kw);
 int cgt_amd_conv_same_pad_f32(const float *x, long planes, long H, long W, int kh, int kw,
                               float *xpad, void *stream);
 
+/* gypad = pad(relu_mask * max_pool_pullback(mask, top_diff)) in one pass: the
+ * padded cotangent of a convolution whose result went through a max pool
+ * (cgt_amd_max_pool_pullback_f32, bit for bit, written in the padded layout
+ * instead of [planes][H][W]), optionally multiplied by the int8 mask of a
+ * rectify in between ((float)mask * value, as the Op graph's mask * gy;
+ * relu_mask may be NULL).  Pool geometry and PH, PW as for
+ * cgt_amd_max_pool_pullback_f32; kh, kw are the convolution's kernel. */
+int cgt_amd_conv_same_pad_pool_pullback_f32(const int *mask, const float *top_diff,
+                                            const signed char *relu_mask, long planes, long H, long W,
+                                            int pool_kh, int pool_kw, int pool_ph, int pool_pw,
+                                            int pool_sh, int pool_sw, long PH, long PW,
+                                            int kh, int kw, float *gypad, void *stream);
+
 /* y [B,L,H,W] = conv(x, f), f [L,C,kh,kw], from the padded x.  `bias` (L floats,
  * may be NULL) is added per channel and, if relu != 0, the result is replaced by
  * v * (v >= 0) -- the bias add and rectify of SpatialConvolution + nn.rectify

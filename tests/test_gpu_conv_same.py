@@ -151,6 +151,9 @@ def test_nn_conv2d_takes_the_fused_ops_and_grad_goes_through_them(K):
     y, loss, gx, gf = graph(xn, fn)
     assert isinstance(y.op, conv_same.ConvForward) and isinstance(gx.op, conv_same.ConvBackwardData)
     assert isinstance(gf.op, conv_same.ConvBackwardFilter)
+    # the cotangent comes out of the pool: its pullback writes the padded copy itself, rectify mask included
+    assert isinstance(gx.parents[0].op, conv_same.ConvPadPoolPullback) and gx.parents[0].op.has_relu
+    assert gf.parents[0] is gx.parents[0]
     d = np.float64
     y64 = O.conv2d(x.astype(d), f.astype(d), (1, 1), (1, 1))
     r64 = y64 * (y64 >= 0)
@@ -224,6 +227,74 @@ def test_spatial_convolution_bias_and_rectify_fused_have_the_bits_of_the_separat
     x2 = rs.randn(5, 64, 11, 9).astype(np.float32)
     for a, u in zip(f_fused(x2), f_unfused(x2)):
         assert np.array_equal(a.view(np.uint32), u.view(np.uint32))
+
+
+POOLS = [((2, 2), (0, 0), (2, 2)), ((3, 3), (0, 0), (2, 2)), ((3, 3), (1, 1), (2, 2)), ((4, 3), (1, 0), (3, 2)),
+         ((2, 2), (0, 0), (1, 1)), ((1, 1), (0, 0), (2, 3))]
+
+
+@pytest.mark.parametrize("pk,pp,ps", POOLS)
+@pytest.mark.parametrize("shape,kernel", [((3, 5, 14, 12), (3, 3)), ((2, 3, 55, 55), (5, 5)), ((1, 7, 9, 31), (1, 7)), ((2, 4, 6, 5), (7, 3))])
+def test_pool_pullback_written_into_the_padded_layout_is_bit_exact(K, pk, pp, ps, shape, kernel):
+    # one pass instead of MaxPoolPullback -> (rectify mask *) -> ConvPad: the same bits, every float of
+    # the padded buffer written (it starts out poisoned)
+    from cgt_amd.gpuarray import to_gpu
+    rs = np.random.RandomState(sum(shape) + pk[0] * 7 + ps[1])
+    act = rs.randn(*shape).astype(np.float32)
+    act *= (act >= 0)                                   # ties at zero, as after a rectify
+    top, mask = K.max_pool(to_gpu(act), pk, pp, ps)
+    if top.size == 0:
+        pytest.skip("the pool has no output for this shape")
+    gtop = to_gpu((rs.randn(*top.shape) * 10.0 ** rs.randint(-3, 4, top.shape)).astype(np.float32))
+    rmask = to_gpu((rs.rand(*shape) < 0.6).astype(np.int8))
+    want_plain = K.conv_same_pad(K.max_pool_pullback(shape, mask, gtop, pk, pp, ps), kernel).get()
+    want_relu = K.conv_same_pad(K.elwise_binary("*", rmask, K.max_pool_pullback(shape, mask, gtop, pk, pp, ps)), kernel).get()
+    # what the oracle says the unpadded pullback is
+    assert np.array_equal(K.max_pool_pullback(shape, mask, gtop, pk, pp, ps).get().view(np.uint32),
+                          O.max_pool_pullback(shape, mask.get(), gtop.get()).view(np.uint32))
+    poison = to_gpu(np.full(want_plain.shape, np.nan, np.float32))
+    got = K.conv_same_pad_pool_pullback(shape, mask, gtop, pk, pp, ps, kernel, out=poison).get()
+    assert np.array_equal(got.view(np.uint32), want_plain.view(np.uint32))
+    poison = to_gpu(np.full(want_plain.shape, np.nan, np.float32))
+    got = K.conv_same_pad_pool_pullback(shape, mask, gtop, pk, pp, ps, kernel, relu_mask=rmask, out=poison).get()
+    assert np.array_equal(got.view(np.uint32), want_relu.view(np.uint32))
+
+
+def test_pool_pullback_fusion_leaves_the_gradients_bit_identical(K):
+    # conv -> rectify -> pool: gradients through ConvPadPoolPullback against the graph with the
+    # separate MaxPoolPullback, mask multiply and ConvPad; and the compiled function is shorter
+    import cgt_amd as cgt
+    from cgt_amd import nn
+    from cgt_amd.nn_ops import conv_same
+    rs = np.random.RandomState(21)
+    x = rs.randn(3, 32, 13, 14).astype(np.float32)
+    f = (rs.randn(48, 32, 3, 3) / 17).astype(np.float32)
+
+    def graph(xn, fn, relu):
+        y = nn.conv2d(xn, fn, (3, 3), pad=(1, 1))
+        pooled = nn.max_pool_2d(nn.rectify(y) if relu else y, (3, 3), (0, 0), (2, 2))
+        gx, gf = cgt.grad(cgt.sum(pooled * pooled), [xn, fn])
+        return [pooled, gx, gf]
+
+    for relu in (True, False):
+        xn, fn = cgt.constant(x), cgt.constant(f)
+        fused = graph(xn, fn, relu)
+        assert isinstance(fused[1].parents[0].op, conv_same.ConvPadPoolPullback)
+        conv_same.FUSE_POOL_PULLBACK = False
+        try:
+            xu, fu = cgt.constant(x), cgt.constant(f)
+            plain = graph(xu, fu, relu)
+            assert isinstance(plain[1].parents[0].op, conv_same.ConvPad)
+        finally:
+            conv_same.FUSE_POOL_PULLBACK = True
+        for a, u in zip(fused, plain):
+            assert np.array_equal(a.get().view(np.uint32), u.get().view(np.uint32))
+        f_fused, f_plain = cgt.function([xn], fused), cgt.function([xu], plain)
+        launches = lambda fun: sum(1 for s in fun.plan_steps() if s[0] == "byref")      # noqa: E731
+        assert launches(f_fused) == launches(f_plain) - (2 if relu else 1)
+        x2 = rs.randn(5, 32, 13, 14).astype(np.float32)
+        for a, u in zip(f_fused(x2), f_plain(x2)):
+            assert np.array_equal(a.view(np.uint32), u.view(np.uint32))
 
 
 def test_vgg_layer_full_size_through_the_fused_ops(K):

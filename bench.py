@@ -240,7 +240,10 @@ class LayerOnGpu(object):
             self.gy_lrn = empty(self.y.shape)
             g_in = gy
             st.append(Stage("lrn_bwd", "lrn_bwd_kernel",
-                            lambda: K.lrn_bwd(self.y, self.top, self.scale, g_in, size, alpha, beta, out=self.gy_lrn, stream=s),
+                            # as the Op's closure calls it: `top` is formed again from x and scale, not read.
+                            # The stage's bytes stay the five arrays of the reference's algorithm (x, top,
+                            # scale, cotangent in; one out), the unit the metric is quoted in; the kernel moves four
+                            lambda: K.lrn_bwd(self.y, None, self.scale, g_in, size, alpha, beta, out=self.gy_lrn, stream=s),
                             5 * 4 * nelem(self.y), "hbm"))
             gy = self.gy_lrn
         self.gy = gy

@@ -203,7 +203,10 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_fwd_generic_kernel(
     }
 }
 
-template <int SIZE, bool DOWN>
+// RECOMP: `top` is not read; top[c] = x[c] * scale[c]^-beta is formed again from x and scale
+// with the operations of the forward kernels (same bits as the array they wrote), so the
+// kernel streams four arrays instead of five.
+template <int SIZE, bool DOWN, bool RECOMP>
 __device__ __forceinline__ void lrn_bwd_run(const float* __restrict__ x, const float* __restrict__ top,
                                             const float* __restrict__ scale, const float* __restrict__ top_diff,
                                             float* __restrict__ bottom_diff, int C, int HW, const LrnBlock& blk,
@@ -226,24 +229,35 @@ __device__ __forceinline__ void lrn_bwd_run(const float* __restrict__ x, const f
 
     float tr[U + SIZE - 1];   // tr[j] = (td*top/scale)[c0 - PRE + j]
     float dr[U + POST];       // dr[j] = td[c0 + j]
-    float sr[U + POST];       // sr[j] = scale[c0 + j]
+    float sr[U + POST];       // sr[j] = scale[c0 + j]; RECOMP: scale[c0 + j]^-beta
+    float xr[U + POST];       // RECOMP: x[c0 + j]
 #pragma unroll
     for (int j = 0; j < SIZE - 1; ++j) {
         const int c = cs - PRE + j;
-        float d = 0.0f, sc = 1.0f, t = 0.0f;
+        float d = 0.0f, sc = 1.0f, t = 0.0f;      // t: top, or x when it is formed here
         if (c >= 0 && c < C) {
             d = dp[c * hs];
             sc = sp[c * hs];
-            t = tp[c * hs];
+            t = RECOMP ? xp[c * hs] : tp[c * hs];
         }
-        tr[j] = d * t / sc;
-        if (j >= PRE) {           // channel >= cs: also a centre later on
-            dr[j - PRE] = d;
-            sr[j - PRE] = sc;
+        if constexpr (RECOMP) {
+            const float pw = pow_neg_beta(sc, nbeta);
+            tr[j] = d * (t * pw) / sc;
+            if (j >= PRE) {
+                dr[j - PRE] = d;
+                sr[j - PRE] = pw;
+                xr[j - PRE] = t;
+            }
+        } else {
+            tr[j] = d * t / sc;
+            if (j >= PRE) {           // channel >= cs: also a centre later on
+                dr[j - PRE] = d;
+                sr[j - PRE] = sc;
+            }
         }
     }
     for (int c0 = cs; c0 < ce; c0 += U) {
-        float xc[U], tn[U];
+        float xc[U], tn[U], sn[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int ch = c0 + POST + u;
@@ -251,22 +265,37 @@ __device__ __forceinline__ void lrn_bwd_run(const float* __restrict__ x, const f
             if (ch < C) {
                 d = dp[ch * hs];
                 sc = sp[ch * hs];
-                t = tp[ch * hs];
+                t = RECOMP ? xp[ch * hs] : tp[ch * hs];
             }
             dr[POST + u] = d;
-            sr[POST + u] = sc;
+            sn[u] = sc;
             tn[u] = t;
-            xc[u] = (c0 + u < ce) ? xp[(c0 + u) * hs] : 0.0f;
+            if constexpr (!RECOMP) {
+                sr[POST + u] = sc;
+                xc[u] = (c0 + u < ce) ? xp[(c0 + u) * hs] : 0.0f;
+            }
         }
+        if constexpr (RECOMP) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) tr[SIZE - 1 + u] = dr[POST + u] * tn[u] / sr[POST + u];
+            for (int u = 0; u < U; ++u) {
+                const float pw = pow_neg_beta(sn[u], nbeta);
+                sr[POST + u] = pw;
+                xr[POST + u] = tn[u];
+                tr[SIZE - 1 + u] = dr[POST + u] * (tn[u] * pw) / sn[u];
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u) tr[SIZE - 1 + u] = dr[POST + u] * tn[u] / sn[u];
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             float acc = 0.0f;
 #pragma unroll
             for (int j = 0; j < SIZE; ++j) acc += tr[u + j];
-            if (c0 + u < ce)
-                bp[(c0 + u) * hs] = dr[u] * pow_neg_beta(sr[u], nbeta) - ratio * xc[u] * acc;
+            if (c0 + u < ce) {
+                if constexpr (RECOMP) bp[(c0 + u) * hs] = dr[u] * sr[u] - ratio * xr[u] * acc;
+                else bp[(c0 + u) * hs] = dr[u] * pow_neg_beta(sr[u], nbeta) - ratio * xc[u] * acc;
+            }
         }
 #pragma unroll
         for (int j = 0; j < SIZE - 1; ++j) tr[j] = tr[U + j];
@@ -274,18 +303,19 @@ __device__ __forceinline__ void lrn_bwd_run(const float* __restrict__ x, const f
         for (int j = 0; j < POST; ++j) {
             dr[j] = dr[U + j];
             sr[j] = sr[U + j];
+            if constexpr (RECOMP) xr[j] = xr[U + j];
         }
     }
 }
 
-template <int SIZE>
+template <int SIZE, bool RECOMP>
 __global__ __launch_bounds__(kLrnThreads) void lrn_bwd_kernel(
     const float* __restrict__ x, const float* __restrict__ top, const float* __restrict__ scale,
     const float* __restrict__ top_diff, float* __restrict__ bottom_diff, int C, int HW, int crun,
     float nbeta, float ratio) {
     const LrnBlock blk = lrn_block(HW, C, crun);
-    if (blk.run & 1) lrn_bwd_run<SIZE, true>(x, top, scale, top_diff, bottom_diff, C, HW, blk, crun, nbeta, ratio);
-    else lrn_bwd_run<SIZE, false>(x, top, scale, top_diff, bottom_diff, C, HW, blk, crun, nbeta, ratio);
+    if (blk.run & 1) lrn_bwd_run<SIZE, true, RECOMP>(x, top, scale, top_diff, bottom_diff, C, HW, blk, crun, nbeta, ratio);
+    else lrn_bwd_run<SIZE, false, RECOMP>(x, top, scale, top_diff, bottom_diff, C, HW, blk, crun, nbeta, ratio);
 }
 
 __global__ __launch_bounds__(kLrnThreads) void lrn_bwd_generic_kernel(
@@ -304,7 +334,8 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_bwd_generic_kernel(
         const int lo = max(0, c - pre), hi = min(C - 1, c + post);
         for (int cc = lo; cc <= hi; ++cc) {
             const long i = base + (long)cc * HW;
-            acc += top_diff[i] * top[i] / scale[i];
+            const float t = top ? top[i] : x[i] * pow_neg_beta(scale[i], nbeta);      // top == nullptr: formed again
+            acc += top_diff[i] * t / scale[i];
         }
         const long i = base + (long)c * HW;
         bottom_diff[i] = top_diff[i] * pow_neg_beta(scale[i], nbeta) - ratio * x[i] * acc;
@@ -374,22 +405,22 @@ CGT_API int cgt_amd_lrn_fwd_f32(const float* x, long N, long C, long H, long W, 
     return CGT_AMD_OK;
 }
 
-CGT_API int cgt_amd_lrn_bwd_f32(const float* x, const float* top, const float* scale,
-                                const float* top_diff, long N, long C, long H, long W, int size,
-                                double alpha, double beta, float* bottom_diff, void* stream) {
+// top == nullptr: top is formed again from x and scale (cgt_amd_lrn_bwd_recompute_f32)
+static int lrn_bwd(const float* x, const float* top, const float* scale, const float* top_diff, long N, long C, long H,
+                   long W, int size, double alpha, double beta, float* bottom_diff, void* stream) {
     if (N * C * H * W == 0 && N >= 0 && C >= 0 && H >= 0 && W >= 0 && size >= 1) return CGT_AMD_OK;
     int rc = check_lrn("lrn_bwd", N, C, H, W, size);
     if (rc) return rc;
-    CGT_ARG_CHECK(x && top && scale && top_diff && bottom_diff, "lrn_bwd: null pointer");
+    CGT_ARG_CHECK(x && scale && top_diff && bottom_diff, "lrn_bwd: null pointer");
     const int HW = (int)(H * W);
     const int crun = pick_crun(N, (int)C, HW, size);
     dim3 grid((unsigned)(cdiv(HW, kLrnThreads) * cdiv(C, crun) * N)), block(kLrnThreads);
     hipStream_t st = as_stream(stream);
     const float nbeta = (float)(-beta), ratio = (float)(2. * alpha * beta / size);
-#define LRN_BWD_CASE(S)                                                                      \
-    case S:                                                                                  \
-        lrn_bwd_kernel<S><<<grid, block, 0, st>>>(x, top, scale, top_diff, bottom_diff, (int)C, \
-                                                  HW, crun, nbeta, ratio);                   \
+#define LRN_BWD_CASE(S)                                                                                       \
+    case S:                                                                                                   \
+        if (top) lrn_bwd_kernel<S, false><<<grid, block, 0, st>>>(x, top, scale, top_diff, bottom_diff, (int)C, HW, crun, nbeta, ratio); \
+        else lrn_bwd_kernel<S, true><<<grid, block, 0, st>>>(x, top, scale, top_diff, bottom_diff, (int)C, HW, crun, nbeta, ratio);      \
         break;
     switch (size) {
         LRN_BWD_CASE(1) LRN_BWD_CASE(2) LRN_BWD_CASE(3) LRN_BWD_CASE(4) LRN_BWD_CASE(5)
@@ -401,4 +432,17 @@ CGT_API int cgt_amd_lrn_bwd_f32(const float* x, const float* top, const float* s
 #undef LRN_BWD_CASE
     CGT_LAUNCH_CHECK("lrn_bwd_kernel");
     return CGT_AMD_OK;
+}
+
+CGT_API int cgt_amd_lrn_bwd_f32(const float* x, const float* top, const float* scale,
+                                const float* top_diff, long N, long C, long H, long W, int size,
+                                double alpha, double beta, float* bottom_diff, void* stream) {
+    CGT_ARG_CHECK(top || N * C * H * W == 0, "lrn_bwd: null pointer");
+    return lrn_bwd(x, top, scale, top_diff, N, C, H, W, size, alpha, beta, bottom_diff, stream);
+}
+
+CGT_API int cgt_amd_lrn_bwd_recompute_f32(const float* x, const float* scale, const float* top_diff, long N, long C,
+                                          long H, long W, int size, double alpha, double beta, float* bottom_diff,
+                                          void* stream) {
+    return lrn_bwd(x, nullptr, scale, top_diff, N, C, H, W, size, alpha, beta, bottom_diff, stream);
 }

@@ -107,15 +107,20 @@ def lrn_fwd(x, size, alpha, beta, k=1.0, out=None, stream=None):
 
 
 def lrn_bwd(x, top, scale, gtop, size, alpha, beta, out=None, stream=None):
-    """CrossChannelLRNBackward op (reference cgt/nn_ops/cross_channel_lrn.py:65-104)."""
-    _f32(x, top, scale, gtop)
+    """CrossChannelLRNBackward op (reference cgt/nn_ops/cross_channel_lrn.py:65-104).
+    top=None: top = x * scale^-beta is formed again inside the kernel (the bits lrn_fwd wrote)."""
+    _f32(x, scale, gtop)
     N, C, H, W = x.shape
-    for a in (top, scale, gtop):
-        if a.shape != x.shape:
-            raise ValueError("LRN backward operands must share x's shape")
+    for a in (scale, gtop) + (() if top is None else (top,)):
+        if a.shape != x.shape or a.dtype != np.float32:
+            raise ValueError("LRN backward operands must be float32 arrays of x's shape")
     gb = _out(out, x.shape)
-    capi.check(capi.lib().cgt_amd_lrn_bwd_f32(x.ptr, top.ptr, scale.ptr, gtop.ptr, N, C, H, W, int(size),
-                                              float(alpha), float(beta), gb.ptr, stream))
+    if top is None:
+        capi.check(capi.lib().cgt_amd_lrn_bwd_recompute_f32(x.ptr, scale.ptr, gtop.ptr, N, C, H, W, int(size),
+                                                            float(alpha), float(beta), gb.ptr, stream))
+    else:
+        capi.check(capi.lib().cgt_amd_lrn_bwd_f32(x.ptr, top.ptr, scale.ptr, gtop.ptr, N, C, H, W, int(size),
+                                                  float(alpha), float(beta), gb.ptr, stream))
     return gb
 
 

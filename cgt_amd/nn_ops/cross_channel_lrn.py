@@ -70,19 +70,24 @@ class CrossChannelLRNBackward(core.Op):
         assert devtype == "gpu" and input_types[0].dtype == "f4"
         code = r"""
             CGT_EXPORT_C void $function($closure* cldata, cgtArray** reads, cgtArray* bottom_diff) {
-                cgtArray *X=reads[0], *top=reads[1], *scaling=reads[2], *top_diff=reads[3];
+                // reads[1], the forward op's `top`, is not read: top = X * scaling^-beta is formed
+                // again from X and scaling with the forward kernel's own operations (same bits)
+                cgtArray *X=reads[0], *scaling=reads[2], *top_diff=reads[3];
                 long num_img = X->shape()[0],
                      channels = X->shape()[1],
                      height = X->shape()[2],
                      width = X->shape()[3];
-                int rc = cgt_amd_lrn_bwd_f32((const float*)X->data(), (const float*)top->data(),
+                cgt_check(scaling->size() == X->size() && top_diff->size() == X->size() && bottom_diff->size() == X->size(),
+                          "CrossChannelLRNBackward: operands do not share the input's shape");
+                if (cgtGlobalStatus != cgtStatusOK) return;
+                int rc = cgt_amd_lrn_bwd_recompute_f32((const float*)X->data(),
                     (const float*)scaling->data(), (const float*)top_diff->data(),
                     num_img, channels, height, width, cldata->localsize, cldata->alpha, cldata->beta,
                     (float*)bottom_diff->data(), cgt_get_stream());
                 cgt_check(rc == CGT_AMD_OK, "CrossChannelLRNBackward: %s", cgt_amd_last_error());
             }"""
         return core.NativeCompileInfo(code, closure_triples=make_closure(self.info),
-                                      includes=["cgt_amd.h"], gpu_deref_mask=(True, True, True, True))
+                                      includes=["cgt_amd.h"], gpu_deref_mask=(True, False, True, True))
 
     def shp_apply(self, inputs):
         return core.shape(inputs[0])

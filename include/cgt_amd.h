@@ -245,6 +245,16 @@ int cgt_amd_lrn_bwd_f32(const float *x, const float *top, const float *scale,
                         int size, double alpha, double beta,
                         float *bottom_diff, void *stream);
 
+/* The same without the `top` operand: top = x * scale^(-beta) is formed again
+ * from x and scale with the forward kernels' own operations, so for the
+ * (top, scale) pair cgt_amd_lrn_fwd_f32 wrote the result has the bits of
+ * cgt_amd_lrn_bwd_f32 while one array less is streamed from memory (four
+ * instead of five).  What CrossChannelLRNBackward's closure calls: its `top`
+ * input is always the forward op's output. */
+int cgt_amd_lrn_bwd_recompute_f32(const float *x, const float *scale, const float *top_diff,
+                                  long N, long C, long H, long W, int size, double alpha,
+                                  double beta, float *bottom_diff, void *stream);
+
 /* ---------------------------------------------------------------- GEMM */
 
 /* Row-major C[M,N] = op(A) . op(B), alpha = 1, beta = 0, true fp32 (MFMA

@@ -238,6 +238,16 @@ def test_lrn_vs_oracle(K, shape, size, alpha, beta, k):
         gb = K.lrn_bwd(gpu(x), gpu(rtop), gpu(rscale), gpu(g), size, alpha, beta).get()
         assert relfro(gb, rgb) <= TOL
         assert relfro(gb, tgb) <= 1e-5
+    # the variant that does not read `top` (what the Op's closure calls): top is formed again from
+    # x and scale, so on the pair the forward kernel wrote it has the bits of the five-array kernel
+    g = rs.rand(*shape).astype(np.float32)
+    xg, gg = gpu(x), gpu(g)
+    dtop, dscale = K.lrn_fwd(xg, size, alpha, beta, k)
+    with_top = K.lrn_bwd(xg, dtop, dscale, gg, size, alpha, beta).get()
+    recomputed = K.lrn_bwd(xg, None, dscale, gg, size, alpha, beta).get()
+    assert np.array_equal(recomputed.view(np.uint32), with_top.view(np.uint32))
+    tgb = O.lrn_bwd(x64, ttop, tscale, g.astype(np.float64), size, alpha, beta)
+    assert relfro(recomputed, tgb) <= 1e-5
 
 
 @pytest.mark.parametrize("shape,size", [((5, 7, 701, 685), 5), ((5, 7, 701, 685), 4), ((2, 9, 1024, 1024), 3)])

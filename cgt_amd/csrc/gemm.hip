@@ -311,9 +311,13 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
         split = grp * kNumXCD + r % in_grp;
         lid = r / in_grp;
     } else if ((int)blockIdx.x < a.main_wgs) {
+        // each XCD gets a contiguous range of (batch, tile) pairs: the tiles of one product, which
+        // share its operands, meet in one L2 (remapped inside each batch, the three column tiles of
+        // an AlexNet data-gradient image sat on three XCDs and its cotangent was fetched three times)
         const int per_batch = a.main_wgs / a.batch;        // == tiles unless there is a tail (batch 1)
-        batch = blockIdx.x / per_batch;
-        lid = xcd_remap(blockIdx.x - batch * per_batch, per_batch);
+        const int g = xcd_remap(blockIdx.x, a.main_wgs);
+        batch = g / per_batch;
+        lid = g - batch * per_batch;
     } else {
         tail_piece = blockIdx.x - a.main_wgs;
         lid = a.main_wgs + tail_piece / a.tail_splits;

@@ -187,26 +187,33 @@ class LayerOnGpu(object):
         # products over the column buffer ("col"); "im2col" is the literal composition with Mul22 and
         # the two transposes
         if algo == "auto":
-            self.algo = "direct" if K.conv_same_supported(C, L, (r, c), pad, stride) else "col"
+            self.algo = ("direct" if K.conv_same_supported(C, L, (r, c), pad, stride) else
+                         "patch" if C < 16 and K.conv_patch_supported(x.shape, (r, c), pad, stride) else "col")
         else:
             self.algo = algo
-        fused_col = self.algo == "col"
+        patch = self.algo == "patch"          # no column buffer for the forward product and the weight gradient
+        fused_col = self.algo in ("col", "patch")
         if self.algo == "direct":
             self.overlap = False
             self.glue = glue
             self._direct_stages(K, cfg, nelem)
             return
-        self.col = empty((B, m, n, Z))
-        self.col2 = self.col.reshape(Bmn, Z)
+        self.col = None if patch else empty((B, m, n, Z))
+        self.col2 = None if patch else self.col.reshape(Bmn, Z)
         self.y_mnL = None if fused_col else empty((Bmn, L))
         self.y = empty((B, L, m, n))
         act = self.y
         st = []
         s = stream
         gemm_bytes = 4 * (Bmn * Z + L * Z + Bmn * L)      # the three conv products touch the same three matrices
-        st.append(Stage("im2col", "im2col_linear_kernel or im2col_pipe_kernel", lambda: K.im2col(self.x, (r, c), pad, stride, out=self.col, stream=s),
-                        4 * (nelem(self.x) + nelem(self.col)), "hbm"))
-        if fused_col:       # the product writes [B,L,m,n] itself
+        if not patch:
+            st.append(Stage("im2col", "im2col_linear_kernel or im2col_pipe_kernel", lambda: K.im2col(self.x, (r, c), pad, stride, out=self.col, stream=s),
+                            4 * (nelem(self.x) + nelem(self.col)), "hbm"))
+        patch_bytes = 4 * (nelem(self.x) + L * Z + Bmn * L)      # image + filters + result
+        if patch:           # the product gathers the patches from x and writes [B,L,m,n] itself
+            st.append(Stage("gemm_fwd", "sgemm_kernel", lambda: K.conv_patch_fwd(self.x, self.f, pad, stride, out=self.y, stream=s),
+                            2 * Bmn * L * Z, "mfma", patch_bytes))
+        elif fused_col:     # the product writes [B,L,m,n] itself
             st.append(Stage("gemm_fwd", "sgemm_kernel", lambda: K.conv_col_fwd(self.col, self.f, out=self.y, stream=s),
                             2 * Bmn * L * Z, "mfma", gemm_bytes))
         else:
@@ -252,15 +259,19 @@ class LayerOnGpu(object):
         self.gf = empty((L, Z))
         col2im = Stage("col2im", "col2im_stream_kernel",
                        lambda: K.col2im(self.gcol.reshape(B, m, n, Z), self.x.shape, (r, c), pad, stride, out=self.gx, stream=s),
-                       4 * (nelem(self.x) + nelem(self.col)), "hbm")
+                       4 * (nelem(self.x) + nelem(self.gcol)), "hbm")
         if fused_col:       # both gradient products read the NCHW cotangent themselves
             self.overlap = False
             gcol4, gf4 = self.gcol.reshape(B, m, n, Z), self.gf.reshape(L, C, r, c)
             st.append(Stage("gemm_dgrad", "sgemm_kernel", lambda: K.conv_col_bwd_data(self.gy, self.f, out=gcol4, stream=s),
                             2 * Bmn * L * Z, "mfma", gemm_bytes))
             st.append(col2im)
-            st.append(Stage("gemm_wgrad", "sgemm_kernel", lambda: K.conv_col_bwd_filter(self.gy, self.col, self.f.shape, out=gf4, stream=s),
-                            2 * Bmn * L * Z, "mfma", gemm_bytes))
+            if patch:
+                st.append(Stage("gemm_wgrad", "sgemm_kernel", lambda: K.conv_patch_bwd_filter(self.gy, self.x, self.f.shape, pad, stride, out=gf4, stream=s),
+                                2 * Bmn * L * Z, "mfma", patch_bytes))
+            else:
+                st.append(Stage("gemm_wgrad", "sgemm_kernel", lambda: K.conv_col_bwd_filter(self.gy, self.col, self.f.shape, out=gf4, stream=s),
+                                2 * Bmn * L * Z, "mfma", gemm_bytes))
         else:
             self.gc = empty((B, m, n, L))
             self.gc2 = self.gc.reshape(Bmn, L)
@@ -544,6 +555,9 @@ def check_against_oracle(cfg):
     err = float(np.linalg.norm(y - y64) / np.linalg.norm(y64))
     y = K.conv_col_fwd(col, to_gpu(f)).get()        # the fused product over the same column buffer
     err = max(err, float(np.linalg.norm(y - y64) / np.linalg.norm(y64)))
+    if K.conv_patch_supported(x.shape, (r, c), pad, stride):      # and with the patches gathered from x
+        y = K.conv_patch_fwd(to_gpu(x), to_gpu(f), pad, stride).get()
+        err = max(err, float(np.linalg.norm(y - y64) / np.linalg.norm(y64)))
     return {"im2col_bit_exact": bool(ok), "conv2d_rel_fro": err, "ok": bool(ok and err <= 1e-4)}
 
 
@@ -717,6 +731,8 @@ def measure(workload, args, primary):
     if algo:
         config["conv_algo"] = {"direct": "fused ops, no column buffer (pad -> GEMM over the padded image -> NCHW)",
                                "col": "im2col -> fused products over the column buffer (NCHW written / read by the GEMMs) -> col2im",
+                               "patch": "forward product and weight gradient gather their patches from the image (no column buffer, "
+                                        "NCHW written / read by the GEMMs); data gradient over a column buffer -> col2im",
                                "im2col": "im2col -> Mul22 -> transpose; transpose -> Mul22 -> col2im, Mul22"}[algo]
     if is_gemm:
         config["value_is"] = "flops of Mul22 4096^3 x {NN,NT,TN,TT} + BatchedMul22 64x512^3 / step time"
@@ -767,7 +783,7 @@ def main():
     ap.add_argument("--no-op-api", action="store_true", help="skip timing the same step through the Op API")
     ap.add_argument("--no-check", action="store_true",
                     help="skip the parity gate (profiling runs: keeps its small launches out of the kernel statistics)")
-    ap.add_argument("--conv-algo", default="auto", choices=["auto", "col", "im2col"],
+    ap.add_argument("--conv-algo", default="auto", choices=["auto", "patch", "col", "im2col"],
                     help="auto: what nn.conv2d builds (the fused ops without a column buffer where they apply, else "
                          "im2col + the fused products over the column buffer); col: the latter for every layer; "
                          "im2col: always the literal im2col -> Mul22 -> transpose composition")

@@ -72,6 +72,9 @@ PROTOTYPES = {
     "cgt_amd_conv_same_bwd_filter_f32": (c_int, [c_void_p, c_void_p] + [c_long] * 5 + [c_int, c_int, c_void_p, c_void_p]),
     "cgt_amd_conv_same_pad_pool_pullback_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_long, c_long, c_long] + [c_int] * 6 +
                                                 [c_long, c_long, c_int, c_int, c_void_p, c_void_p]),
+    "cgt_amd_conv_patch_supported": (c_int, [c_long] * 4 + [c_int] * 6),
+    "cgt_amd_conv_patch_fwd_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int] + [c_long] * 5 + [c_int] * 6 + [c_void_p, c_void_p, c_void_p]),
+    "cgt_amd_conv_patch_bwd_filter_f32": (c_int, [c_void_p, c_void_p] + [c_long] * 5 + [c_int] * 6 + [c_void_p, c_void_p]),
     "cgt_amd_conv_col_fwd_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int] + [c_long] * 4 + [c_void_p, c_void_p, c_void_p]),
     "cgt_amd_conv_col_bwd_data_f32": (c_int, [c_void_p, c_void_p] + [c_long] * 4 + [c_void_p, c_void_p]),
     "cgt_amd_conv_col_bwd_filter_f32": (c_int, [c_void_p, c_void_p] + [c_long] * 4 + [c_void_p, c_void_p]),

@@ -231,6 +231,10 @@ def prebuild_standard_ops():
         (nn_ops.conv_col.ConvColForward(True, True), [T4, T4, T4]),
         (nn_ops.conv_col.ConvColBackwardData(), [T4, T4, T4]),
         (nn_ops.conv_col.ConvColBackwardFilter(), [T4, T4, T4]),
+        (nn_ops.conv_col.ConvPatchForward(info), [T4, T4]),
+        (nn_ops.conv_col.ConvPatchForward(info, True, True), [T4, T4, T4]),
+        (nn_ops.conv_col.ConvPatchBackwardData(info), [T4, T4, T4]),
+        (nn_ops.conv_col.ConvPatchBackwardFilter(info), [T4, T4, T4]),
         (core.Transport("gpu"), [T4]),
         # conv-layer glue: the closure code is generic over element type and
         # rank, so one library per op class serves every use

@@ -21,7 +21,7 @@ inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 // stream -- it is retired and released with the stream (cgt_amd_stream_destroy).
 // Growth while the stream is being captured is refused (an allocation would break the
 // capture): returns nullptr with the message set.
-enum WorkspaceUser { kWsGemm = 0, kWsSum = 1, kWsConvFilter = 2, kWsUsers = 3 };
+enum WorkspaceUser { kWsGemm = 0, kWsSum = 1, kWsConvFilter = 2, kWsConvTable = 3, kWsConvData = 4, kWsUsers = 5 };
 float* stream_workspace(void* stream, WorkspaceUser user, size_t bytes, const char* what);
 void release_stream_workspaces(void* stream);
 
@@ -34,6 +34,13 @@ void release_stream_workspaces(void* stream);
 // Over a column buffer col[B * plane][C] (any geometry), with the NCHW side read / written in place:
 //   mode 1: out[b][m][p] = sum over z of W[m][z] * col[b * plane + p][z] (+ bias[m], rectify); C = patch length
 //   mode 4: out[M][N] = sum over (b, p) of A[b][m][p] * col[b * plane + p][n]   (A = the NCHW cotangent)
+// Modes 1 and 4 without a column buffer: col[b * plane + p][z] is read from the image x
+// [B][C][H][W] where im2col would have copied it from (zero outside the image); OH x OW = plane
+// output pixels per image, z = (c * kh + ho) * kw + wo.
+struct PatchGeom {
+    const float* x;
+    int C, H, W, kh, kw, ph, pw, sh, sw, OH, OW;
+};
 struct ConvGemm {
     int mode;
     long B, C, plane;      // images; channels of `img` (mode 1: patch length); floats per padded plane (modes 1, 4: pixels per image)
@@ -43,6 +50,7 @@ struct ConvGemm {
     const float* bias;     // mode 3: per-output-channel bias or null
     int relu;              // mode 3: x * (x >= 0) on the way out
     signed char* mask;     // mode 3: (x >= 0) as int8, same shape as the output, or null
+    const PatchGeom* patch = nullptr;      // modes 1, 4: gather the column buffer's elements from the image
 };
 int sgemm_conv(const ConvGemm& cv, long M, long N, const float* A, const float* B, float* C, long ldc, void* stream);
 // 1 if sgemm_conv has a tile shape for these extents (output channels of the product, channels of the image)

@@ -289,3 +289,55 @@ CGT_API int cgt_amd_conv_col_bwd_filter_f32(const float* gy, const float* col, l
     ConvGemm cv = {4, B, Z, P, 0, 1, 1, 0, 0, 0, 0, nullptr, 0, nullptr};
     return sgemm_conv(cv, L, Z, gy, col, gf, Z, stream);
 }
+
+// ---- any geometry, no column buffer for the forward product and the weight gradient: the two
+// products above with col's elements gathered from the image as the GEMM loads its operand tile
+// (im2col's index rule applied inside the loader, zero outside the image).  The data gradient
+// keeps the column buffer: its result has to be scattered back (cgt_amd_conv_col_bwd_data_f32
+// + cgt_amd_col2im_f32), and with a handful of input channels there is no GEMM to gather into.
+
+static bool patch_geom(PatchGeom& pg, const float* x, long C, long H, long W, int kh, int kw, int ph, int pw, int sh, int sw) {
+    if (C < 1 || H < 1 || W < 1 || kh < 1 || kw < 1 || ph < 0 || pw < 0 || sh < 1 || sw < 1) return false;
+    if (H + 2L * ph < kh || W + 2L * pw < kw) return false;
+    const long OH = (H + 2L * ph - kh) / sh + 1, OW = (W + 2L * pw - kw) / sw + 1;
+    if (H >= 32768 || W >= 32768 || kh >= 32768 || kw >= 32768 || ph >= 32768 || pw >= 32768 || C >= (1L << 20) ||
+        OH * OW >= (1L << 21) || C * kh * kw >= (1L << 31) - 128)
+        return false;
+    pg = PatchGeom{x, (int)C, (int)H, (int)W, kh, kw, ph, pw, sh, sw, (int)OH, (int)OW};
+    return true;
+}
+
+CGT_API int cgt_amd_conv_patch_supported(long B, long C, long H, long W, int kh, int kw, int ph, int pw, int sh, int sw) {
+    PatchGeom pg;
+    if (B < 0 || !patch_geom(pg, nullptr, C, H, W, kh, kw, ph, pw, sh, sw)) return 0;
+    return B * C * H * W < (1L << 29) && B * pg.OH * pg.OW < (1L << 31) - 128 ? 1 : 0;
+}
+
+CGT_API int cgt_amd_conv_patch_fwd_f32(const float* x, const float* f, const float* bias, int relu, long B, long C,
+                                       long H, long W, long L, int kh, int kw, int ph, int pw, int sh, int sw,
+                                       float* y, signed char* mask, void* stream) {
+    CGT_ARG_CHECK(B >= 0 && L >= 0, "conv_patch_fwd: negative extent");
+    PatchGeom pg;
+    CGT_ARG_CHECK(patch_geom(pg, x, C, H, W, kh, kw, ph, pw, sh, sw) && cgt_amd_conv_patch_supported(B, C, H, W, kh, kw, ph, pw, sh, sw),
+                  "conv_patch_fwd: geometry out of range (use im2col + cgt_amd_conv_col_fwd_f32)");
+    const long P = (long)pg.OH * pg.OW, Z = C * kh * kw;
+    if (B == 0 || L == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(x && f && y, "conv_patch_fwd: null pointer");
+    ConvGemm cv = {1, B, Z, P, 0, 1, 1, 0, 0, 0, 0, bias, relu, mask, &pg};
+    return sgemm_conv(cv, L, B * P, f, x, y, B * P, stream);
+}
+
+CGT_API int cgt_amd_conv_patch_bwd_filter_f32(const float* gy, const float* x, long B, long C, long H, long W, long L,
+                                              int kh, int kw, int ph, int pw, int sh, int sw, float* gf, void* stream) {
+    CGT_ARG_CHECK(B >= 0 && L >= 0, "conv_patch_bwd_filter: negative extent");
+    PatchGeom pg;
+    CGT_ARG_CHECK(patch_geom(pg, x, C, H, W, kh, kw, ph, pw, sh, sw) && cgt_amd_conv_patch_supported(B, C, H, W, kh, kw, ph, pw, sh, sw),
+                  "conv_patch_bwd_filter: geometry out of range (use im2col + cgt_amd_conv_col_bwd_filter_f32)");
+    const long P = (long)pg.OH * pg.OW, Z = C * kh * kw;
+    if (L == 0) return CGT_AMD_OK;
+    CGT_ARG_CHECK(gf, "conv_patch_bwd_filter: null pointer");
+    if (B == 0) return cgt_amd_fill_u32(gf, 0u, L * Z, stream);
+    CGT_ARG_CHECK(gy && x, "conv_patch_bwd_filter: null pointer");
+    ConvGemm cv = {4, B, Z, P, 0, 1, 1, 0, 0, 0, 0, nullptr, 0, nullptr, &pg};
+    return sgemm_conv(cv, L, Z, gy, x, gf, Z, stream);
+}

@@ -123,6 +123,17 @@ struct GemmArgs {
     // its A operand starts aimg floats further per image (A is [image][M][kimg], k-contiguous).
     int kimg, kspi;
     long aimg;
+    // Patch gather (GATHER != 0): the B operand is not a column buffer but the image itself,
+    // [images][g_C][g_H][g_W]; element (pixel n, patch index z) of the column buffer is read
+    // from g_x where im2col would have copied it from (0 outside the image).
+    //   GATHER 1 (forward): B is k-contiguous, rows = pixels n, k = z.  g_koff[k] = byte offset of
+    //     patch element k inside an image, 4 * ((c * H + ho) * W + wo), -1 for k past the patch length
+    //     (the table is padded to a multiple of 16); g_khw[k] = (ho << 16) | wo (padded layers).
+    //   GATHER 2 (weight gradient): B is row-contiguous, rows = patch elements z, k = pixels.
+    const float* g_x;
+    const int* g_koff;
+    const int* g_khw;
+    int g_C, g_H, g_W, g_kh, g_kw, g_ph, g_pw, g_sh, g_sw, g_OW, g_P;   // g_P = output pixels per image
 };
 
 // One ROWS x KT operand tile, moved with 16-byte accesses.
@@ -282,8 +293,11 @@ __device__ __forceinline__ int xcd_remap(int id, int n) {
 // WGM x WGN wavefronts, each TM x TN blocks of 32x32.
 // PIPE selects the software-pipelined main loop (k-contiguous operands only).
 // DEEP (plain loop only) keeps two K slices of global loads in flight instead of one.
-template <bool AKC, bool BKC, bool PIPE, int WGM, int WGN, int TM, int TN, bool DEEP = false, int CONV = 0>
+template <bool AKC, bool BKC, bool PIPE, int WGM, int WGN, int TM, int TN, bool DEEP = false, int CONV = 0, int GATHER = 0,
+          bool GPAD = false>
 __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmArgs a) {
+    static_assert(GATHER == 0 || (!PIPE && !DEEP && AKC && ((GATHER == 1 && BKC && CONV == 1) || (GATHER == 2 && !BKC && CONV == 0))),
+                  "patch gather: forward = NT with the NCHW epilogue, weight gradient = NN with K cut per image");
     static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
     static_assert(CONV == 0 || (CONV >= 1 && CONV <= 3 && !PIPE && !DEEP && AKC && BKC == (CONV != 3)),
                   "convolution products: plain loop; the image operand is B, row-contiguous in mode 3; "
@@ -338,8 +352,10 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
     int kend = min(a.K, kbeg + kchunk);
     const float* A = a.A + batch * a.sA;
     const float* B = a.B + batch * a.sB;
+    int gimg = 0;                   // GATHER 2: the image this workgroup's K range lies in
     if (CONV == 0 && a.kimg) {      // K cut per image: this split is one piece of one image
         const int img = split / a.kspi, piece = split - img * a.kspi;
+        gimg = img;
         kbeg = img * a.kimg + piece * kchunk;
         kend = min((img + 1) * a.kimg, kbeg + kchunk);
         A += (long)img * a.aimg;
@@ -405,7 +421,8 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
     // whole (an edge tile in N still streams A untested) and the tested ones
     // otherwise; a ragged last K slice is tested for both.
     constexpr int kFast = 0, kMixed = 1;
-    const bool wholeA = CONV >= 2 || (m0 + BM <= a.M && !a.wide), wholeB = CONV >= 2 || (n0 + BN <= a.N && !a.wide);
+    const bool wholeA = CONV >= 2 || (m0 + BM <= a.M && !a.wide);
+    const bool wholeB = GATHER == 0 && (CONV >= 2 || (n0 + BN <= a.N && !a.wide));     // gathered tiles go through registers
     const bool ragged_k = CONV <= 1 && (kend - kbeg) % KT != 0;
     const char* originA = reinterpret_cast<const char*>(A + (AKC ? (long)m0 * a.lda + kbeg : (long)kbeg * a.lda + m0));
     const char* originB = reinterpret_cast<const char*>(B + (BKC ? (long)n0 * a.ldb + kbeg : (long)kbeg * a.ldb + n0));
@@ -471,6 +488,120 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
             else ra.load_checked(A, a.lda, m0, a.M, k0, kend);
             if (wholeB && !tested) rb.load_fast(originB + slice * stepB, tb.goff);
             else rb.load_checked(B, a.ldb, n0, a.N, k0, kend);
+        }
+    };
+
+    // Patch gather: what each of this thread's 16-byte pieces of the B tile is made of.
+    // The piece's position inside the tile is fixed, so whatever depends on it alone is
+    // worked out once: for the forward product the pixel of its row (byte offset of the
+    // patch's corner), for the weight gradient the four patch elements of its columns.  All
+    // offsets are bytes from g_x (< 2^33 / 2: the host checks), added to the uniform base by
+    // the load itself.  The per-slice work is then one add per element where every element
+    // exists (layers without padding, all but a ragged last slice); bounds tests otherwise.
+    constexpr int GNV = GATHER != 0 ? TileB::NV : 1;
+    unsigned g_base[GNV];                          // GATHER 1: corner of the row's patch; GATHER 2: of the current pixel's
+    int g_corner[GNV], g_k4[GNV];                  // GATHER 1; g_corner = (h0 << 16) | (w0 & 0xffff)
+    unsigned g_zoff[GNV][4];                       // GATHER 2: patch element -> byte offset from the corner
+    int g_zhw[GNV][4], g_ow[GNV], g_h0[GNV], g_w0[GNV];
+    const char* gx = reinterpret_cast<const char*>(a.g_x);
+    if constexpr (GATHER == 1) {
+#pragma unroll
+        for (int i = 0; i < GNV; ++i) {
+            const int idx = threadIdx.x + i * kGemmThreads;
+            const int row = idx >> 2;
+            const int n = min(n0 + row, a.N - 1);            // rows past the end repeat the last pixel; they are never stored
+            const int b = n / a.g_P, p = n - b * a.g_P;
+            const int oh = p / a.g_OW, ow = p - oh * a.g_OW;
+            const int h0 = oh * a.g_sh - a.g_ph, w0 = ow * a.g_sw - a.g_pw;
+            g_base[i] = (unsigned)(((b * a.g_C * a.g_H + h0) * a.g_W + w0) * 4);
+            g_corner[i] = (h0 << 16) | (w0 & 0xffff);
+            g_k4[i] = chunk_pos(row, idx & 3) * 4;
+        }
+    } else if constexpr (GATHER == 2) {
+        const int KK = a.g_kh * a.g_kw;
+#pragma unroll
+        for (int i = 0; i < GNV; ++i) {
+            const int idx = threadIdx.x + i * kGemmThreads;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int z = min(n0 + (idx % (BN / 4)) * 4 + j, a.N - 1);     // columns past the end: never stored
+                const int c = z / KK, r = z - c * KK;
+                const int ho = r / a.g_kw, wo = r - ho * a.g_kw;
+                g_zoff[i][j] = (unsigned)(((c * a.g_H + ho) * a.g_W + wo) * 4);
+                g_zhw[i][j] = (ho << 16) | wo;
+            }
+            // the pixel of this piece's K row in the first slice; gather_b steps it by KT pixels per slice
+            const int p = min(kbeg + idx / (BN / 4), kend - 1) - gimg * a.g_P;
+            const int oh = p / a.g_OW;
+            g_ow[i] = p - oh * a.g_OW;
+            g_h0[i] = oh * a.g_sh - a.g_ph;
+            g_w0[i] = g_ow[i] * a.g_sw - a.g_pw;
+            g_base[i] = (unsigned)(((gimg * a.g_C * a.g_H + g_h0[i]) * a.g_W + g_w0[i]) * 4);
+        }
+    }
+    // One K slice of the gathered operand into tb's registers (parked in LDS after the multiply);
+    // called once per slice, in ascending order.  Every load is issued, from a clamped address;
+    // what does not exist is zeroed afterwards.  `last`: the slice may end past the K range.
+    auto gather_b = [&](int k0, bool last) {
+        if constexpr (GATHER == 1) {
+#pragma unroll
+            for (int i = 0; i < GNV; ++i) {
+                if (!TileB::has(i)) continue;
+                const int k = k0 + g_k4[i];
+                const int4 off = *reinterpret_cast<const int4*>(a.g_koff + k);      // bytes; negative past the patch length
+                const int o[4] = {off.x, off.y, off.z, off.w};
+                if (!GPAD && !last) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) tb.v[i * 4 + j] = *reinterpret_cast<const float*>(gx + (g_base[i] + (unsigned)o[j]));
+                } else {
+                    int hw[4] = {0, 0, 0, 0};
+                    if constexpr (GPAD) {
+                        const int4 t = *reinterpret_cast<const int4*>(a.g_khw + k);
+                        hw[0] = t.x; hw[1] = t.y; hw[2] = t.z; hw[3] = t.w;
+                    }
+                    const int h0 = g_corner[i] >> 16, w0 = (int)(short)(g_corner[i] & 0xffff);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        bool ok = o[j] >= 0;
+                        if constexpr (GPAD)
+                            ok = ok && (unsigned)(h0 + (hw[j] >> 16)) < (unsigned)a.g_H && (unsigned)(w0 + (hw[j] & 0xffff)) < (unsigned)a.g_W;
+                        const float v = *reinterpret_cast<const float*>(gx + (ok ? g_base[i] + (unsigned)o[j] : 0u));
+                        tb.v[i * 4 + j] = ok ? v : 0.0f;
+                    }
+                }
+            }
+        } else if constexpr (GATHER == 2) {
+#pragma unroll
+            for (int i = 0; i < GNV; ++i) {
+                if (!TileB::has(i)) continue;
+                if (!GPAD && !last) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) tb.v[i * 4 + j] = *reinterpret_cast<const float*>(gx + (g_base[i] + g_zoff[i][j]));
+                } else {
+                    const bool inside = k0 + (int)((threadIdx.x + i * kGemmThreads) / (BN / 4)) < kend;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        bool ok = inside;
+                        if constexpr (GPAD)
+                            ok = ok && (unsigned)(g_h0[i] + (g_zhw[i][j] >> 16)) < (unsigned)a.g_H &&
+                                 (unsigned)(g_w0[i] + (g_zhw[i][j] & 0xffff)) < (unsigned)a.g_W;
+                        const float v = *reinterpret_cast<const float*>(gx + (ok ? g_base[i] + g_zoff[i][j] : 0u));
+                        tb.v[i * 4 + j] = ok ? v : 0.0f;
+                    }
+                }
+                // on to the pixel KT further (rows of the output wrap; a slice never leaves the image
+                // except past kend, where nothing is read)
+                int ow = g_ow[i] + KT, wraps = 0;
+                while (ow >= a.g_OW) {
+                    ow -= a.g_OW;
+                    ++wraps;
+                }
+                const int dh = wraps * a.g_sh, dw = (ow - g_ow[i]) * a.g_sw;
+                g_ow[i] = ow;
+                g_h0[i] += dh;
+                g_w0[i] += dw;
+                g_base[i] += (unsigned)((dh * a.g_W + dw) * 4);
+            }
         }
     };
 
@@ -606,7 +737,8 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                     const int k0 = kbeg + slice * KT;
                     if (wholeA && !tested) ta.load_direct(originA + slice * stepA, ta.goff, as, wave_u);
                     else ta.load_checked(A, a.lda, m0, a.M, k0, kend);
-                    if (wholeB && !tested) tb.load_direct(originB + slice * stepB, tb.goff, bs, wave_u);
+                    if constexpr (GATHER != 0) gather_b(k0, slice == nk - 1);
+                    else if (wholeB && !tested) tb.load_direct(originB + slice * stepB, tb.goff, bs, wave_u);
                     else tb.load_checked(B, a.ldb, n0, a.N, k0, kend);
                 };
                 auto park = [&](int slice, float* as, float* bs) {
@@ -648,6 +780,8 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
     }
     if constexpr (CONV >= 2) {
         main_loop(std::integral_constant<int, kFast>{});      // the host sends whole slices only; rows past the end are clamped
+    } else if constexpr (GATHER != 0) {
+        main_loop(std::integral_constant<int, kMixed>{});     // the gathered operand always goes through registers
     } else {
         if (wholeA && wholeB && !ragged_k) main_loop(std::integral_constant<int, kFast>{});
         else main_loop(std::integral_constant<int, kMixed>{});
@@ -1045,6 +1179,40 @@ static void launch_conv(int mode, int shape, dim3 grid, hipStream_t st, const Ge
     }
 }
 
+// patch-gather variants: forward (NT, NCHW epilogue, shapes with 128 columns) and weight gradient (NN)
+template <bool GPAD>
+static void launch_gather(int which, int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
+    dim3 block(kGemmThreads);
+    if (which == 1) {
+        switch (shape) {
+            case 0: sgemm_kernel<true, true, false, 2, 2, 2, 2, false, 1, 1, GPAD><<<grid, block, 0, st>>>(a); break;
+            case 4: sgemm_kernel<true, true, false, 1, 4, 3, 1, false, 1, 1, GPAD><<<grid, block, 0, st>>>(a); break;
+            case 5: sgemm_kernel<true, true, false, 1, 4, 2, 1, false, 1, 1, GPAD><<<grid, block, 0, st>>>(a); break;
+            default: sgemm_kernel<true, true, false, 1, 4, 1, 1, false, 1, 1, GPAD><<<grid, block, 0, st>>>(a); break;
+        }
+    } else {
+        switch (shape) {
+            case 0: sgemm_kernel<true, false, false, 2, 2, 2, 2, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;
+            case 1: sgemm_kernel<true, false, false, 4, 1, 1, 3, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;
+            case 2: sgemm_kernel<true, false, false, 4, 1, 1, 2, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;
+            case 3: sgemm_kernel<true, false, false, 4, 1, 1, 1, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;
+            case 4: sgemm_kernel<true, false, false, 1, 4, 3, 1, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;
+            default: sgemm_kernel<true, false, false, 1, 4, 2, 1, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;
+        }
+    }
+}
+
+// g_koff / g_khw of the forward gather: one entry per patch element, padded to whole K slices
+__global__ void patch_table_kernel(int* __restrict__ koff, int* __restrict__ khw, int K, int Kpad, int kh, int kw, int H, int W) {
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= Kpad) return;
+    const int KK = kh * kw;
+    const int c = k / KK, r = k - c * KK;
+    const int ho = r / kw, wo = r - ho * kw;
+    koff[k] = k < K ? ((c * H + ho) * W + wo) * 4 : -1;      // bytes
+    khw[k] = (ho << 16) | wo;
+}
+
 // tile shape (index into kShapes) of an implicit-convolution product, -1 if none fits: the
 // shape with the least padded work; rows past the end of the result (filters that do not
 // fill the last tile) are computed from repeated operand rows and never stored.
@@ -1143,6 +1311,32 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     GemmArgs a;
     a.conv = conv_kernel ? cv->mode : 0;
     a.kimg = 0; a.kspi = 1; a.aimg = 0;
+    const PatchGeom* pg = cv ? cv->patch : nullptr;       // B operand gathered from the image
+    bool gpad = false;
+    if (pg) {
+        CGT_ARG_CHECK(cv->mode == 1 || cv->mode == 4, "sgemm_conv: patch gather goes with the column-buffer products");
+        const long P = (long)pg->OH * pg->OW, Z = (long)pg->C * pg->kh * pg->kw;
+        CGT_ARG_CHECK(pg->x && P == cv->plane && Z == (cv->mode == 1 ? K : N) && P < (1L << 21) &&
+                      cv->B * pg->C * pg->H * pg->W < (1L << 29) && pg->H < 32768 && pg->W < 32768 &&
+                      pg->kh < 32768 && pg->kw < 32768 && pg->ph < 32768 && pg->pw < 32768,
+                      "sgemm_conv: image too large for the patch gather");
+        // every patch lies inside the image: no bounds tests
+        gpad = !(pg->ph == 0 && pg->pw == 0 && (pg->OH - 1) * pg->sh + pg->kh <= pg->H && (pg->OW - 1) * pg->sw + pg->kw <= pg->W);
+        a.g_x = pg->x;
+        a.g_koff = a.g_khw = nullptr;
+        a.g_C = pg->C; a.g_H = pg->H; a.g_W = pg->W; a.g_kh = pg->kh; a.g_kw = pg->kw; a.g_ph = pg->ph; a.g_pw = pg->pw;
+        a.g_sh = pg->sh; a.g_sw = pg->sw; a.g_OW = pg->OW; a.g_P = (int)P;
+        if (cv->mode == 1) {
+            const long Kpad = cdiv(K, KT) * KT;
+            int* tab = reinterpret_cast<int*>(stream_workspace(stream, kWsConvTable, (size_t)Kpad * 2 * sizeof(int), "sgemm_conv"));
+            if (!tab) return CGT_AMD_ERR_NOMEM;
+            patch_table_kernel<<<dim3((unsigned)cdiv(Kpad, 256L)), dim3(256), 0, as_stream(stream)>>>(
+                tab, tab + Kpad, (int)K, (int)Kpad, pg->kh, pg->kw, pg->H, pg->W);
+            CGT_LAUNCH_CHECK("patch_table_kernel");
+            a.g_koff = tab;
+            a.g_khw = tab + Kpad;
+        }
+    }
     if (cv) {
         a.cv_wp = cv->wp; a.cv_kw = cv->kw; a.cv_kh = cv->kh; a.cv_c = (int)cv->C;
         a.cv_tpi = (int)cv->tpi; a.cv_spi = (int)cv->spi;
@@ -1254,7 +1448,9 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     // and load in bursts) with a long K range each
     const long slices = cdiv(a.splits > 1 ? (long)a.kchunk : K, KT);
     const bool deep = !cv && shape == 0 && !(!tA && tB) && wgs <= 4L * kNumCU && slices >= 32;
-    if (conv_kernel) launch_conv(cv->mode, shape, grid, st, a);
+    if (pg && gpad) launch_gather<true>(cv->mode == 1 ? 1 : 2, shape, grid, st, a);
+    else if (pg) launch_gather<false>(cv->mode == 1 ? 1 : 2, shape, grid, st, a);
+    else if (conv_kernel) launch_conv(cv->mode, shape, grid, st, a);
     else launch_trans(tA, tB, pipe, deep, shape, grid, st, a);
     CGT_LAUNCH_CHECK("sgemm_kernel");
     if (a.splits > 1) {

@@ -388,3 +388,38 @@ def conv_col_bwd_filter(gy, col, fshape, out=None, stream=None):
     gf = _out(out, tuple(fshape))
     capi.check(capi.lib().cgt_amd_conv_col_bwd_filter_f32(gy.ptr, col.ptr, B, m * n, Z, L, gf.ptr, stream))
     return gf
+
+
+def conv_patch_supported(xshape, kernel, pad, stride):
+    B, C, H, W = (int(s) for s in xshape)
+    return bool(capi.lib().cgt_amd_conv_patch_supported(B, C, H, W, *_geom(kernel, pad, stride)))
+
+
+def conv_patch_fwd(x, f, pad, stride, bias=None, relu=False, out=None, mask=None, stream=None):
+    """y [B,L,m,n] = conv2d(x, f) with the patches gathered from x inside the product (no column
+    buffer); optional fused bias add and rectify as in conv_col_fwd."""
+    _f32(x, f)
+    B, C, H, W = x.shape
+    L, C2, kh, kw = f.shape
+    if C2 != C:
+        raise ValueError("filter channels %d != input channels %d" % (C2, C))
+    g = _geom((kh, kw), pad, stride)
+    m, n = conv_outsize(H, g[0], g[2], g[4]), conv_outsize(W, g[1], g[3], g[5])
+    y = _out(out, (B, L, m, n))
+    capi.check(capi.lib().cgt_amd_conv_patch_fwd_f32(x.ptr, f.ptr, None if bias is None else bias.ptr, int(bool(relu)),
+                                                     B, C, H, W, L, *g, y.ptr, None if mask is None else mask.ptr, stream))
+    return y
+
+
+def conv_patch_bwd_filter(gy, x, fshape, pad, stride, out=None, stream=None):
+    """gf [L,C,kh,kw] from the NCHW cotangent gy and the image x (no column buffer)."""
+    _f32(gy, x)
+    B, C, H, W = x.shape
+    L, C2, kh, kw = (int(s) for s in fshape)
+    g = _geom((kh, kw), pad, stride)
+    m, n = conv_outsize(H, g[0], g[2], g[4]), conv_outsize(W, g[1], g[3], g[5])
+    if C2 != C or tuple(gy.shape) != (B, L, m, n):
+        raise ValueError("cotangent %s does not fit x %s and filters %s" % (tuple(gy.shape), tuple(x.shape), tuple(fshape)))
+    gf = _out(out, (L, C, kh, kw))
+    capi.check(capi.lib().cgt_amd_conv_patch_bwd_filter_f32(gy.ptr, x.ptr, B, C, H, W, L, *g, gf.ptr, stream))
+    return gf

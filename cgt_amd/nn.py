@@ -7,9 +7,14 @@ cgt/nn.py:88-93).  This build's GPU branch switches to its own fused ops:
   * stride 1, pad = (kernel - 1) / 2, channel and filter counts in multiples
     of 16: products that read a zero-padded copy of the image, no column
     buffer (nn_ops/conv_same.py);
-  * every other layer: Im2Col, then products that write / read the NCHW
-    arrays themselves, no transposes (nn_ops/conv_col.py) -- conv_algo("col")
-    uses these for every layer;
+  * layers with few input channels (the first layer of a network: 1 or 3
+    channels, any stride): products that gather their patches from the image
+    and write / read the NCHW arrays themselves -- no column buffer for the
+    forward product and the weight gradient, no transposes (nn_ops/conv_col.py,
+    ConvPatch*);
+  * every other layer: Im2Col, then the same products over the column
+    buffer (nn_ops/conv_col.py, ConvCol*) -- conv_algo("col") uses these for
+    every layer;
 conv_algo("im2col") keeps the literal composition, every op on the GPU.
 """
 from . import core
@@ -41,6 +46,8 @@ def conv2d(x_BKRC, f_LKrc, kernelshape, pad=(0, 0), stride=(1, 1)):
     assert tuple(kernelshape) == (r, c), "kernelshape must match the filter's last two axes"
     if _CONV_ALGO == "auto" and conv_same.supported(x_BKRC, f_LKrc, kernelshape, pad, stride):
         return conv_same.conv_same(x_BKRC, f_LKrc, kernelshape)
+    if _CONV_ALGO == "auto" and conv_col.patch_supported(x_BKRC, kernelshape, pad, stride):
+        return conv_col.conv_patch(x_BKRC, f_LKrc, kernelshape, pad, stride)
     col_BmnZ = im2col(x_BKRC, kernelshape, pad, stride)
     if _CONV_ALGO != "im2col":
         return conv_col.conv_col(col_BmnZ, f_LKrc)
@@ -70,7 +77,8 @@ def rectify(x):
     """ReLU as the reference builds it: x * (x >= 0) (cgt/nn.py:44-45).  On the result of a
     fused convolution it becomes part of that op (same values, same gradient)."""
     x = core.as_node(x)
-    if _CONV_FUSION and isinstance(x.op, (conv_same.ConvForward, conv_col.ConvColForward)) and not x.op.relu:
+    if (_CONV_FUSION and isinstance(x.op, (conv_same.ConvForward, conv_col.ConvColForward, conv_col.ConvPatchForward))
+            and not x.op.relu):
         # the same inputs run again with the rectify in the epilogue.  Nodes are evaluated as
         # they are built, so this costs a second product while the graph is traced; a compiled
         # function replays only the fused one (the plain result is no longer reachable from
@@ -103,6 +111,8 @@ class SpatialConvolution(object):
         if (_CONV_FUSION and _CONV_ALGO == "auto"
                 and conv_same.supported(x, self.weight, self.kernelshape, self.pad, self.stride)):
             return conv_same.conv_same(x, self.weight, self.kernelshape, bias=self.bias)
+        if _CONV_FUSION and _CONV_ALGO == "auto" and conv_col.patch_supported(x, self.kernelshape, self.pad, self.stride):
+            return conv_col.conv_patch(x, self.weight, self.kernelshape, self.pad, self.stride, bias=self.bias)
         if _CONV_FUSION and _CONV_ALGO != "im2col":
             col = im2col(x, self.kernelshape, self.pad, self.stride)
             return conv_col.conv_col(col, self.weight, bias=self.bias)

@@ -405,6 +405,26 @@ int cgt_amd_conv_col_bwd_data_f32(const float *gy, const float *f, long B, long 
 int cgt_amd_conv_col_bwd_filter_f32(const float *gy, const float *col, long B, long P, long Z, long L,
                                     float *gf, void *stream);
 
+/* The forward product and the weight gradient of the same composition without
+ * the column buffer: the element col[b*P + p][z] is read from x where
+ * cgt_amd_im2col_f32 would have copied it from (zero outside the image) while
+ * the GEMM loads its operand tile.  Any kernel, padding and stride; results
+ * agree with the products over col to rounding (same sums, same order of z;
+ * the forward product bit for bit).  x [B,C,H,W], f / gf [L,C,kh,kw], y / gy
+ * [B,L,m,n] with m = (H + 2 ph - kh) / sh + 1.  The data gradient keeps the
+ * column buffer (cgt_amd_conv_col_bwd_data_f32 + cgt_amd_col2im_f32). */
+
+/* 1 if the two entry points below take this layer (m*n < 2^21, extents and
+ * kernel < 32768, B*C*H*W < 2^29: byte offsets into x are 32-bit). */
+int cgt_amd_conv_patch_supported(long B, long C, long H, long W, int kh, int kw, int ph, int pw,
+                                 int sh, int sw);
+int cgt_amd_conv_patch_fwd_f32(const float *x, const float *f, const float *bias, int relu,
+                               long B, long C, long H, long W, long L, int kh, int kw, int ph,
+                               int pw, int sh, int sw, float *y, signed char *mask, void *stream);
+int cgt_amd_conv_patch_bwd_filter_f32(const float *gy, const float *x, long B, long C, long H,
+                                      long W, long L, int kh, int kw, int ph, int pw, int sh,
+                                      int sw, float *gf, void *stream);
+
 /* ---------------------------------------------------------------- conv glue */
 
 /* out[i0,i1,i2,i3] = in[...] with out.shape[d] = in.shape[axes[d]].

@@ -102,9 +102,10 @@ def test_default_workload_prints_the_contract_line():
     assert alex["config"]["lrn"]["k"] == 2.0
     names = [r["stage"] for r in alex["stages"]]
     assert "lrn_fwd" in names and "lrn_bwd" in names and "max_pool_bwd" in names
-    # a strided layer: im2col, then products that write / read NCHW themselves -- no transposes
-    assert names[:2] == ["im2col", "gemm_fwd"] and not any(n.startswith("transpose") for n in names)
-    assert "column buffer" in alex["config"]["conv_algo"]
+    # a strided layer with 3 input channels: the forward product and the weight gradient gather their
+    # patches from the image and write / read NCHW themselves -- no im2col, no transposes
+    assert names[0] == "gemm_fwd" and "im2col" not in names and not any(n.startswith("transpose") for n in names)
+    assert "col2im" in names and "no column buffer" in alex["config"]["conv_algo"]
     assert all(r["ms_in_step"] > 0 for r in alex["stages"])
     assert len(w["raw_gemm_4096_and_batched_64x512"]["stages"]) == 5
     for name in ("cifar_conv1_5x5_3x32x32_b128", "mnist_conv3x3_1x28x28_b64"):

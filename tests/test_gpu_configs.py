@@ -63,9 +63,12 @@ def test_mnist_block_full_batch(cgt):
     # conv against the float64 oracle
     h64 = O.conv2d(xval.astype(np.float64), wval.astype(np.float64), (1, 1), (1, 1))
     assert relfro(hv, h64) <= TOL
-    # im2col inside the conv is a copy: bit-exact
-    col = h.parents[0]
-    assert type(col.op).__name__ == "Im2Col" and col.shape == (64, 28, 28, 9)
+    # one input channel: the products gather their patches from x, no column buffer in the graph
+    assert type(h.op).__name__ == "ConvPatchForward" and h.parents[0] is x
+    # the Im2Col op on the same input is a copy: bit-exact
+    from cgt_amd.nn_ops.im2col import im2col
+    col = im2col(x, (3, 3), (1, 1), (1, 1))
+    assert col.shape == (64, 28, 28, 9)
     assert np.array_equal(col.get(), O.im2col(xval, (3, 3), (1, 1), (1, 1)))
     # ReLU as the reference spells it, on the same fp32 input: bit-exact (signs of zero included)
     want_r = O.rectify(hv)

@@ -39,6 +39,8 @@ CASES = [
     (1, 4, 5, 5, 7, (5, 5), (0, 0), (1, 1)),            # one pixel per image
     (12, 16, 56, 56, 64, (5, 5), (2, 2), (1, 1)),       # 294 column tiles: the last 38 go through the tail split
     (2, 24, 30, 30, 48, (3, 3), (1, 1), (1, 1)),
+    (5, 3, 20, 17, 33, (4, 6), (3, 5), (3, 2)),         # padding wider than half the kernel, patches hanging over every edge
+    (2, 6, 40, 40, 200, (7, 7), (3, 3), (2, 2)),
 ]
 
 
@@ -69,6 +71,13 @@ def test_conv_col_products_vs_oracle(K, B, C, H, W, L, kernel, pad, stride):
     assert relfro(gf.get(), gf64) <= TOL
     gx_lit, gf_lit = K.conv2d_pullback(xg, fg, gyg, pad, stride)
     assert relfro(gf.get(), gf_lit.get()) <= 2e-6 and relfro(gx.get(), gx_lit.get()) <= 2e-6
+    # the same two products with the patches gathered from x inside the GEMM (no column buffer):
+    # the same operand values in the same order, so the same bits
+    assert K.conv_patch_supported(x.shape, kernel, pad, stride)
+    y_p = K.conv_patch_fwd(xg, fg, pad, stride)
+    assert np.array_equal(y_p.get().view(np.uint32), y.get().view(np.uint32))
+    gf_p = K.conv_patch_bwd_filter(gyg, xg, f.shape, pad, stride)
+    assert np.array_equal(gf_p.get().view(np.uint32), gf.get().view(np.uint32))
     # a second call into the same (reused, uncleared) outputs gives the same bits
     first = (y.get(), gcol.get(), gf.get())
     K.conv_col_fwd(col, fg, out=y)
@@ -95,6 +104,10 @@ def test_conv_col_fused_bias_and_rectify_match_the_separate_ops(K, B, C, H, W, L
     assert np.array_equal(mask.get(), (pre >= 0).astype(np.int8))
     only_bias = K.conv_col_fwd(col, to_gpu(f), bias=to_gpu(b)).get()
     assert np.array_equal(only_bias.view(np.uint32), pre.view(np.uint32))
+    # and without the column buffer
+    mask2 = empty(plain.shape, np.int8)
+    fused2 = K.conv_patch_fwd(to_gpu(x), to_gpu(f), pad, stride, bias=to_gpu(b), relu=True, mask=mask2).get()
+    assert np.array_equal(fused2.view(np.uint32), want.view(np.uint32)) and np.array_equal(mask2.get(), mask.get())
 
 
 def test_conv_col_full_size_alexnet_conv1(K):
@@ -117,6 +130,8 @@ def test_conv_col_full_size_alexnet_conv1(K):
     gcol = K.conv_col_bwd_data(gyg, fg)
     gx = K.col2im(gcol, x.shape, (11, 11), (0, 0), (4, 4)).get()
     gf = K.conv_col_bwd_filter(gyg, col, f.shape).get()
+    assert np.array_equal(K.conv_patch_fwd(xg, fg, (0, 0), (4, 4)).get().view(np.uint32), yh.view(np.uint32))
+    assert np.array_equal(K.conv_patch_bwd_filter(gyg, xg, f.shape, (0, 0), (4, 4)).get().view(np.uint32), gf.view(np.uint32))
     del gcol
     gf64 = np.zeros(f.shape, d)
     for b in (3, 126):
@@ -130,7 +145,7 @@ def test_conv_col_full_size_alexnet_conv1(K):
 
 
 def test_nn_conv2d_builds_the_column_buffer_ops_for_a_strided_layer():
-    # a layer the padded-image products do not cover (stride 2, 3 channels): Im2Col stays, one
+    # a layer the padded-image products do not cover (stride 2, 20 channels): Im2Col stays, one
     # fused op follows it, grad walks its pullback and Im2Col's own (Col2Im); a compiled function
     # replays the same closures and serves another batch size; the literal composition agrees
     import cgt_amd as cgt
@@ -138,8 +153,8 @@ def test_nn_conv2d_builds_the_column_buffer_ops_for_a_strided_layer():
     from cgt_amd.nn_ops import conv_col
     capi.require_gpu()
     rs = np.random.RandomState(4)
-    x = rs.randn(3, 3, 23, 19).astype(np.float32)
-    f = (rs.randn(40, 3, 5, 5) / 9).astype(np.float32)
+    x = rs.randn(3, 20, 23, 19).astype(np.float32)
+    f = (rs.randn(40, 20, 5, 5) / 22).astype(np.float32)
 
     def graph(xn, fn):
         y = nn.conv2d(xn, fn, (5, 5), pad=(1, 2), stride=(2, 2))
@@ -171,7 +186,7 @@ def test_nn_conv2d_builds_the_column_buffer_ops_for_a_strided_layer():
     fun = cgt.function([xn], [y, loss, gx, gf])
     for got, node in zip(fun(x), (y, loss, gx, gf)):
         assert np.array_equal(got.view(np.uint32), node.get().view(np.uint32))
-    x5 = rs.randn(5, 3, 23, 19).astype(np.float32)
+    x5 = rs.randn(5, 20, 23, 19).astype(np.float32)
     fresh = graph(cgt.constant(x5), fn)
     for got, node in zip(fun(x5), fresh):
         assert np.array_equal(got.view(np.uint32), node.get().view(np.uint32))
@@ -185,10 +200,10 @@ def test_spatial_convolution_over_the_column_buffer_fuses_bias_and_rectify():
     from cgt_amd.nn_ops import conv_col
     capi.require_gpu()
     rs = np.random.RandomState(9)
-    x = rs.randn(4, 3, 21, 21).astype(np.float32)
-    w = (rs.randn(24, 3, 7, 7) / 12).astype(np.float32)
+    x = rs.randn(4, 17, 21, 21).astype(np.float32)
+    w = (rs.randn(24, 17, 7, 7) / 29).astype(np.float32)
     b = (0.3 * rs.randn(1, 24, 1, 1)).astype(np.float32)
-    layer = nn.SpatialConvolution(3, 24, (7, 7), (0, 0), stride=(2, 2), weight_init=w, bias_init=b)
+    layer = nn.SpatialConvolution(17, 24, (7, 7), (0, 0), stride=(2, 2), weight_init=w, bias_init=b)
 
     def graph(xn):
         act = nn.rectify(layer(xn))
@@ -221,6 +236,60 @@ def test_spatial_convolution_over_the_column_buffer_fuses_bias_and_rectify():
     f_fused, f_unfused = cgt.function([xn], fused), cgt.function([xu], unfused)
     launches = lambda f: sum(1 for s in f.plan_steps() if s[0] == "byref")      # noqa: E731
     assert launches(f_fused) <= launches(f_unfused) - 4          # Repeat, +, >=, * are gone
-    x2 = rs.randn(6, 3, 21, 21).astype(np.float32)
+    x2 = rs.randn(6, 17, 21, 21).astype(np.float32)
     for a, u in zip(f_fused(x2), f_unfused(x2)):
+        assert np.array_equal(a.view(np.uint32), u.view(np.uint32))
+
+
+def test_nn_conv2d_gathers_patches_for_a_layer_with_few_channels():
+    # 3 input channels, stride 2, padding: no Im2Col in the graph -- the forward product and the
+    # weight gradient read x themselves, the data gradient goes through the column buffer's
+    # cotangent and Col2Im.  Values and gradients have the bits of the graph over the column buffer
+    # (the same products on the same operand values), SpatialConvolution's bias and a rectify ride
+    # in the epilogue, and the compiled function serves another batch size.
+    import cgt_amd as cgt
+    from cgt_amd import capi, nn
+    from cgt_amd.nn_ops import conv_col
+    capi.require_gpu()
+    rs = np.random.RandomState(14)
+    x = rs.randn(4, 3, 29, 23).astype(np.float32)
+    w = (rs.randn(40, 3, 5, 7) / 10).astype(np.float32)
+    b = (0.3 * rs.randn(1, 40, 1, 1)).astype(np.float32)
+    layer = nn.SpatialConvolution(3, 40, (5, 7), (2, 1), stride=(2, 3), weight_init=w, bias_init=b)
+
+    def graph(xn):
+        act = nn.rectify(layer(xn))
+        pooled = nn.max_pool_2d(act, (2, 2), (0, 0), (2, 2))
+        loss = cgt.sum(pooled * pooled)
+        gx, gw, gb = cgt.grad(loss, [xn, layer.weight, layer.bias])
+        return [act, loss, gx, gw, gb]
+
+    xn = cgt.constant(x)
+    patch = graph(xn)
+    producer = patch[0].parents[0].op
+    assert isinstance(producer, conv_col.ConvPatchForward) and producer.relu and producer.has_bias
+    assert type(patch[2].op).__name__ == "Col2Im" and isinstance(patch[2].parents[0].op, conv_col.ConvPatchBackwardData)
+    assert isinstance(patch[3].op, conv_col.ConvPatchBackwardFilter)
+    old = nn.conv_algo("col")
+    try:
+        xc = cgt.constant(x)
+        col = graph(xc)
+        assert isinstance(col[0].parents[0].op, conv_col.ConvColForward)
+    finally:
+        nn.conv_algo(old)
+    for a, u in zip(patch, col):
+        assert np.array_equal(a.get().view(np.uint32), u.get().view(np.uint32))
+    d = np.float64
+    pre = O.conv2d(x.astype(d), w.astype(d), (2, 1), (2, 3)) + b
+    act64 = pre * (pre >= 0)
+    p64, mask = O.max_pool(act64, (2, 2), (0, 0), (2, 2))
+    gpre = O.max_pool_pullback(act64.shape, mask, 2 * p64) * (pre >= 0)
+    gx64, gw64 = O.conv2d_pullback(x.astype(d), w.astype(d), gpre, (2, 1), (2, 3))
+    assert relfro(patch[0].get(), act64) <= TOL and relfro(patch[2].get(), gx64) <= TOL
+    assert relfro(patch[3].get(), gw64) <= TOL and relfro(patch[4].get(), gpre.sum((0, 2, 3), keepdims=True)) <= TOL
+    f_patch, f_col = cgt.function([xn], patch), cgt.function([xc], col)
+    launches = lambda f: sum(1 for s in f.plan_steps() if s[0] == "byref")      # noqa: E731
+    assert launches(f_patch) == launches(f_col) - 1              # no Im2Col
+    x2 = rs.randn(7, 3, 29, 23).astype(np.float32)
+    for a, u in zip(f_patch(x2), f_col(x2)):
         assert np.array_equal(a.view(np.uint32), u.view(np.uint32))

@@ -65,8 +65,20 @@ DEFAULT_WORKLOAD = "vgg_mid_conv3x3_128x56x56_b64"
 # headline layer once more as the im2col -> Mul22 -> col2im composition, which is how
 # layers the fused ops do not cover run and where the VGG-sized im2col / col2im figures are
 IM2COL_SUFFIX = "/im2col"
-EXTRA_WORKLOADS = [DEFAULT_WORKLOAD + IM2COL_SUFFIX, "alexnet_conv1_11x11s4_3x227x227_b128", GEMM_WORKLOAD,
+# ... and AlexNet conv1 once more over a column buffer ("/col": im2col + the fused products over it), which is
+# where the AlexNet-sized im2col figure is now that the layer itself runs without one
+COL_SUFFIX = "/col"
+EXTRA_WORKLOADS = [DEFAULT_WORKLOAD + IM2COL_SUFFIX, "alexnet_conv1_11x11s4_3x227x227_b128",
+                   "alexnet_conv1_11x11s4_3x227x227_b128" + COL_SUFFIX, GEMM_WORKLOAD,
                    "cifar_conv1_5x5_3x32x32_b128", "mnist_conv3x3_1x28x28_b64"]
+
+
+def split_workload(workload):
+    """(base workload, forced conv algorithm or None) of a name with an algorithm suffix."""
+    for suffix, algo in ((IM2COL_SUFFIX, "im2col"), (COL_SUFFIX, "col")):
+        if workload.endswith(suffix):
+            return workload[:-len(suffix)], algo
+    return workload, None
 
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries of this script, per workload
 PROFILE_PREFIX = {
@@ -97,10 +109,10 @@ def _pmc_rows(path):
 
 
 def profile_prefix(workload, algo):
-    base = workload[:-len(IM2COL_SUFFIX)] if workload.endswith(IM2COL_SUFFIX) else workload
+    base, _ = split_workload(workload)
     prefix = PROFILE_PREFIX.get(base)
-    if prefix is None:
-        return None
+    if prefix is None or (base != DEFAULT_WORKLOAD and algo not in (None, "patch")):
+        return None             # AlexNet conv1: the summaries are of the layer as nn.conv2d builds it
     return prefix + ("_im2col" if algo == "im2col" and base == DEFAULT_WORKLOAD else "")
 
 
@@ -652,9 +664,10 @@ def measure(workload, args, primary):
         layer = GemmOnGpu()
         parity = {"ok": True, "skipped": True} if args.no_check else check_gemm_against_oracle()
     else:
-        cfg = WORKLOADS[workload[:-len(IM2COL_SUFFIX)] if workload.endswith(IM2COL_SUFFIX) else workload]
+        base, forced = split_workload(workload)
+        cfg = WORKLOADS[base]
         layer = LayerOnGpu(cfg, overlap=primary and args.overlap and not args.no_overlap, glue=primary and args.glue,
-                           algo="im2col" if workload.endswith(IM2COL_SUFFIX) else args.conv_algo)
+                           algo=forced or args.conv_algo)
         parity = {"ok": True, "skipped": True} if args.no_check else check_against_oracle(cfg)
 
     for _ in range(args.warmup):

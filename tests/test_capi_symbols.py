@@ -105,3 +105,31 @@ def test_argument_errors_are_reported_not_fatal():
     assert rc == 1 and "size" in capi.last_error()
     rc = lib.cgt_amd_sgemm(0, 0, 4, 4, 4, None, 2, None, 4, None, 4, None)
     assert rc == 1
+
+
+def test_conv_col_and_patch_host_side_rules():
+    # the column-buffer and patch-gather products validate on the host before any launch
+    from cgt_amd import capi
+    lib = capi.lib()
+    ok = lambda B, C, H, W, k, p, s: lib.cgt_amd_conv_patch_supported(B, C, H, W, k, k, p, p, s, s)      # noqa: E731
+    assert ok(128, 3, 227, 227, 11, 0, 4) and ok(64, 1, 28, 28, 3, 1, 1) and ok(1, 3, 5, 5, 5, 0, 1)
+    assert not ok(1, 3, 4, 4, 5, 0, 1)                  # kernel larger than the padded image
+    assert not ok(1, 1, 3000, 3000, 3, 1, 1)            # 9 M output pixels per image: beyond the gather's pixel walk
+    assert not ok(4096, 64, 64, 64, 3, 1, 1)            # 2^30 floats: byte offsets into x would not fit 32 bits
+    assert not ok(1, 3, 40000, 8, 3, 1, 1) and not ok(1, 3, 8, 8, 3, 1, 0)
+    rc = lib.cgt_amd_conv_patch_fwd_f32(None, None, None, 0, 2, 3, 9, 9, 8, 3, 3, 1, 1, 1, 1, None, None, None)
+    assert rc == 1 and "null" in capi.last_error()
+    rc = lib.cgt_amd_conv_patch_fwd_f32(None, None, None, 0, 2, 3, 2, 2, 8, 3, 3, 0, 0, 1, 1, None, None, None)
+    assert rc == 1 and "out of range" in capi.last_error()
+    rc = lib.cgt_amd_conv_patch_bwd_filter_f32(None, None, 2, 3, 9, 9, 8, 3, 3, 1, 1, 1, 1, None, None)
+    assert rc == 1 and "null" in capi.last_error()
+    # empty batches and empty filter banks are not errors and launch nothing
+    assert lib.cgt_amd_conv_patch_fwd_f32(None, None, None, 0, 0, 3, 9, 9, 8, 3, 3, 1, 1, 1, 1, None, None, None) == 0
+    assert lib.cgt_amd_conv_col_fwd_f32(None, None, None, 0, 0, 49, 27, 8, None, None, None) == 0
+    assert lib.cgt_amd_conv_col_bwd_data_f32(None, None, 0, 49, 27, 8, None, None) == 0
+    rc = lib.cgt_amd_conv_col_fwd_f32(None, None, None, 0, 2, 49, 27, 8, None, None, None)
+    assert rc == 1 and "null" in capi.last_error()
+    rc = lib.cgt_amd_conv_col_bwd_filter_f32(None, None, 2, 49, 27, 8, None, None)
+    assert rc == 1 and "null" in capi.last_error()
+    rc = lib.cgt_amd_conv_col_fwd_f32(None, None, None, 0, -1, 49, 27, 8, None, None, None)
+    assert rc == 1 and "negative" in capi.last_error()

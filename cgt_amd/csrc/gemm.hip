@@ -491,116 +491,152 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
         }
     };
 
-    // Patch gather: what each of this thread's 16-byte pieces of the B tile is made of.
-    // The piece's position inside the tile is fixed, so whatever depends on it alone is
-    // worked out once: for the forward product the pixel of its row (byte offset of the
-    // patch's corner), for the weight gradient the four patch elements of its columns.  All
-    // offsets are bytes from g_x (< 2^33 / 2: the host checks), added to the uniform base by
-    // the load itself.  The per-slice work is then one add per element where every element
-    // exists (layers without padding, all but a ragged last slice); bounds tests otherwise.
-    constexpr int GNV = GATHER != 0 ? TileB::NV : 1;
-    unsigned g_base[GNV];                          // GATHER 1: corner of the row's patch; GATHER 2: of the current pixel's
-    int g_corner[GNV], g_k4[GNV];                  // GATHER 1; g_corner = (h0 << 16) | (w0 & 0xffff)
-    unsigned g_zoff[GNV][4];                       // GATHER 2: patch element -> byte offset from the corner
-    int g_zhw[GNV][4], g_ow[GNV], g_h0[GNV], g_w0[GNV];
+    // Patch gather: the B tile is filled from the image, through registers, with as much of the
+    // address arithmetic as possible done once per tile.  Offsets are bytes from g_x (< 2^31: the
+    // host checks), added to the uniform base by the load itself.  Where every element exists
+    // (layers without padding, all but a ragged last slice) a slice costs a thread its 8
+    // four-byte loads and at most one add per element; bounds tests otherwise.
+    //   GATHER 1 (forward, BN = 128): a thread fills the two 16-byte pieces of the k-contiguous
+    //     tile that the plain register path gives it (row = pixel, 4 consecutive k).  Fixed per
+    //     tile: its rows' pixels -> byte offset of the patch corner.  Per slice: the patch
+    //     offsets of its 4 k's, one 16-byte load from the table g_koff.  (Lanes as rows with the
+    //     table in scalar registers needs no vector arithmetic at all and measured SLOWER, 0.301
+    //     against 0.267 ms on AlexNet conv1: the scalar loads share the LDS wait counter.)
+    //   GATHER 2 (weight gradient, BN = 128 or 64): wavefront w takes the K rows (pixels)
+    //     4w..4w+3 of the slice, a lane BN / 64 adjacent columns (patch elements, fixed per tile);
+    //     the four pixels are wave-uniform and walked KT positions per slice in scalar registers,
+    //     so an element's address is scalar pointer + lane offset (0.295 -> 0.276 ms against one
+    //     pixel walk per lane).
+    constexpr int ZPL = BN / 64;                   // GATHER 2: columns per lane
+    static_assert(GATHER != 1 || BN == 128, "forward gather: 128 pixels per tile");
+    static_assert(GATHER != 2 || BN == 128 || BN == 64, "weight-gradient gather: 128 or 64 columns per tile");
     const char* gx = reinterpret_cast<const char*>(a.g_x);
+    const int gwave = __builtin_amdgcn_readfirstlane(wave);
+    unsigned g_lane[2] = {0u, 0u};                 // byte offsets: GATHER 1 the patch corners of the thread's two rows, GATHER 2 its columns
+    int g_lh[2] = {0, 0}, g_lw[2] = {0, 0};        // padded layers: (h0, w0) of those corners / (ho, wo) of those columns
+    int g_k4[2] = {0, 0};                          // GATHER 1: first k (inside a slice) of the thread's two pieces
+    unsigned gp_base[4] = {0u, 0u, 0u, 0u};        // GATHER 2: byte offset of the four pixels' patch corners (uniform)
+    int gp_ow[4] = {0, 0, 0, 0}, gp_h0[4] = {0, 0, 0, 0}, gp_w0[4] = {0, 0, 0, 0};
     if constexpr (GATHER == 1) {
 #pragma unroll
-        for (int i = 0; i < GNV; ++i) {
+        for (int i = 0; i < 2; ++i) {
             const int idx = threadIdx.x + i * kGemmThreads;
             const int row = idx >> 2;
             const int n = min(n0 + row, a.N - 1);            // rows past the end repeat the last pixel; they are never stored
             const int b = n / a.g_P, p = n - b * a.g_P;
             const int oh = p / a.g_OW, ow = p - oh * a.g_OW;
-            const int h0 = oh * a.g_sh - a.g_ph, w0 = ow * a.g_sw - a.g_pw;
-            g_base[i] = (unsigned)(((b * a.g_C * a.g_H + h0) * a.g_W + w0) * 4);
-            g_corner[i] = (h0 << 16) | (w0 & 0xffff);
+            g_lh[i] = oh * a.g_sh - a.g_ph;
+            g_lw[i] = ow * a.g_sw - a.g_pw;
+            g_lane[i] = (unsigned)(((b * a.g_C * a.g_H + g_lh[i]) * a.g_W + g_lw[i]) * 4);
             g_k4[i] = chunk_pos(row, idx & 3) * 4;
         }
     } else if constexpr (GATHER == 2) {
         const int KK = a.g_kh * a.g_kw;
 #pragma unroll
-        for (int i = 0; i < GNV; ++i) {
-            const int idx = threadIdx.x + i * kGemmThreads;
+        for (int q = 0; q < ZPL; ++q) {
+            const int z = min(n0 + lane * ZPL + q, a.N - 1);         // columns past the end: never stored
+            const int c = z / KK, r = z - c * KK;
+            g_lh[q] = r / a.g_kw;
+            g_lw[q] = r - g_lh[q] * a.g_kw;
+            g_lane[q] = (unsigned)(((c * a.g_H + g_lh[q]) * a.g_W + g_lw[q]) * 4);
+        }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int z = min(n0 + (idx % (BN / 4)) * 4 + j, a.N - 1);     // columns past the end: never stored
-                const int c = z / KK, r = z - c * KK;
-                const int ho = r / a.g_kw, wo = r - ho * a.g_kw;
-                g_zoff[i][j] = (unsigned)(((c * a.g_H + ho) * a.g_W + wo) * 4);
-                g_zhw[i][j] = (ho << 16) | wo;
-            }
-            // the pixel of this piece's K row in the first slice; gather_b steps it by KT pixels per slice
-            const int p = min(kbeg + idx / (BN / 4), kend - 1) - gimg * a.g_P;
+        for (int j = 0; j < 4; ++j) {
+            const int p = min(kbeg + gwave * 4 + j, kend - 1) - gimg * a.g_P;     // in the first slice
             const int oh = p / a.g_OW;
-            g_ow[i] = p - oh * a.g_OW;
-            g_h0[i] = oh * a.g_sh - a.g_ph;
-            g_w0[i] = g_ow[i] * a.g_sw - a.g_pw;
-            g_base[i] = (unsigned)(((gimg * a.g_C * a.g_H + g_h0[i]) * a.g_W + g_w0[i]) * 4);
+            gp_ow[j] = p - oh * a.g_OW;
+            gp_h0[j] = oh * a.g_sh - a.g_ph;
+            gp_w0[j] = gp_ow[j] * a.g_sw - a.g_pw;
+            gp_base[j] = (unsigned)(((gimg * a.g_C * a.g_H + gp_h0[j]) * a.g_W + gp_w0[j]) * 4);
         }
     }
-    // One K slice of the gathered operand into tb's registers (parked in LDS after the multiply);
-    // called once per slice, in ascending order.  Every load is issued, from a clamped address;
-    // what does not exist is zeroed afterwards.  `last`: the slice may end past the K range.
+    // One K slice of the gathered operand into tb's registers; called once per slice, in ascending
+    // order (GATHER 2 advances its pixels).  Every load is issued, from a clamped address; what
+    // does not exist is zeroed afterwards.  `last`: the slice may end past the K range.
     auto gather_b = [&](int k0, bool last) {
+        // the two forms are whole straight-line blocks behind ONE uniform branch: with a branch per
+        // element the compiler's wait-count pass drains the load queue before every load
         if constexpr (GATHER == 1) {
+            int o[8], hw[8];
 #pragma unroll
-            for (int i = 0; i < GNV; ++i) {
-                if (!TileB::has(i)) continue;
-                const int k = k0 + g_k4[i];
-                const int4 off = *reinterpret_cast<const int4*>(a.g_koff + k);      // bytes; negative past the patch length
-                const int o[4] = {off.x, off.y, off.z, off.w};
-                if (!GPAD && !last) {
+            for (int i = 0; i < 2; ++i) {
+                const int4 off = *reinterpret_cast<const int4*>(a.g_koff + k0 + g_k4[i]);    // bytes; negative past the patch length
+                o[i * 4] = off.x; o[i * 4 + 1] = off.y; o[i * 4 + 2] = off.z; o[i * 4 + 3] = off.w;
+            }
+            if (!GPAD && !last) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) tb.v[i * 4 + j] = *reinterpret_cast<const float*>(gx + (g_base[i] + (unsigned)o[j]));
-                } else {
-                    int hw[4] = {0, 0, 0, 0};
-                    if constexpr (GPAD) {
-                        const int4 t = *reinterpret_cast<const int4*>(a.g_khw + k);
-                        hw[0] = t.x; hw[1] = t.y; hw[2] = t.z; hw[3] = t.w;
-                    }
-                    const int h0 = g_corner[i] >> 16, w0 = (int)(short)(g_corner[i] & 0xffff);
+                for (int e = 0; e < 8; ++e) tb.v[e] = *reinterpret_cast<const float*>(gx + (g_lane[e / 4] + (unsigned)o[e]));
+            } else {
+                if constexpr (GPAD) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        bool ok = o[j] >= 0;
-                        if constexpr (GPAD)
-                            ok = ok && (unsigned)(h0 + (hw[j] >> 16)) < (unsigned)a.g_H && (unsigned)(w0 + (hw[j] & 0xffff)) < (unsigned)a.g_W;
-                        const float v = *reinterpret_cast<const float*>(gx + (ok ? g_base[i] + (unsigned)o[j] : 0u));
-                        tb.v[i * 4 + j] = ok ? v : 0.0f;
+                    for (int i = 0; i < 2; ++i) {
+                        const int4 t = *reinterpret_cast<const int4*>(a.g_khw + k0 + g_k4[i]);
+                        hw[i * 4] = t.x; hw[i * 4 + 1] = t.y; hw[i * 4 + 2] = t.z; hw[i * 4 + 3] = t.w;
                     }
                 }
+                bool ok[8];
+                float v[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    ok[e] = o[e] >= 0;
+                    if constexpr (GPAD)
+                        ok[e] = ok[e] && (unsigned)(g_lh[e / 4] + (hw[e] >> 16)) < (unsigned)a.g_H &&
+                                (unsigned)(g_lw[e / 4] + (hw[e] & 0xffff)) < (unsigned)a.g_W;
+                    v[e] = *reinterpret_cast<const float*>(gx + (ok[e] ? g_lane[e / 4] + (unsigned)o[e] : 0u));
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) tb.v[e] = ok[e] ? v[e] : 0.0f;
             }
         } else if constexpr (GATHER == 2) {
+            if (!GPAD && !last) {
 #pragma unroll
-            for (int i = 0; i < GNV; ++i) {
-                if (!TileB::has(i)) continue;
-                if (!GPAD && !last) {
+                for (int j = 0; j < 4; ++j)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) tb.v[i * 4 + j] = *reinterpret_cast<const float*>(gx + (g_base[i] + g_zoff[i][j]));
-                } else {
-                    const bool inside = k0 + (int)((threadIdx.x + i * kGemmThreads) / (BN / 4)) < kend;
+                    for (int q = 0; q < ZPL; ++q)
+                        tb.v[j * ZPL + q] = *reinterpret_cast<const float*>(gx + gp_base[j] + g_lane[q]);
+            } else {
+                bool ok[4 * ZPL];
+                float v[4 * ZPL];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        bool ok = inside;
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int q = 0; q < ZPL; ++q) {
+                        bool in = k0 + gwave * 4 + j < kend;
                         if constexpr (GPAD)
-                            ok = ok && (unsigned)(g_h0[i] + (g_zhw[i][j] >> 16)) < (unsigned)a.g_H &&
-                                 (unsigned)(g_w0[i] + (g_zhw[i][j] & 0xffff)) < (unsigned)a.g_W;
-                        const float v = *reinterpret_cast<const float*>(gx + (ok ? g_base[i] + g_zoff[i][j] : 0u));
-                        tb.v[i * 4 + j] = ok ? v : 0.0f;
+                            in = in && (unsigned)(gp_h0[j] + g_lh[q]) < (unsigned)a.g_H && (unsigned)(gp_w0[j] + g_lw[q]) < (unsigned)a.g_W;
+                        ok[j * ZPL + q] = in;
+                        v[j * ZPL + q] = *reinterpret_cast<const float*>(gx + (in ? gp_base[j] + g_lane[q] : 0u));
                     }
-                }
-                // on to the pixel KT further (rows of the output wrap; a slice never leaves the image
-                // except past kend, where nothing is read)
-                int ow = g_ow[i] + KT, wraps = 0;
+#pragma unroll
+                for (int e = 0; e < 4 * ZPL; ++e) tb.v[e] = ok[e] ? v[e] : 0.0f;
+            }
+            // on to the pixels KT further (rows of the output wrap; a slice never leaves the image
+            // except past kend, where nothing is read)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                int ow = gp_ow[j] + KT, wraps = 0;
                 while (ow >= a.g_OW) {
                     ow -= a.g_OW;
                     ++wraps;
                 }
-                const int dh = wraps * a.g_sh, dw = (ow - g_ow[i]) * a.g_sw;
-                g_ow[i] = ow;
-                g_h0[i] += dh;
-                g_w0[i] += dw;
-                g_base[i] += (unsigned)((dh * a.g_W + dw) * 4);
+                const int dh = wraps * a.g_sh, dw = (ow - gp_ow[j]) * a.g_sw;
+                gp_ow[j] = ow;
+                gp_h0[j] += dh;
+                gp_w0[j] += dw;
+                gp_base[j] += (unsigned)((dh * a.g_W + dw) * 4);
+            }
+        }
+    };
+    // ... and from the registers into the LDS tile, in the layout the fragment reads expect
+    auto gather_park = [&](float* bs) {
+        if constexpr (GATHER == 1) {
+            tb.store(bs);                                           // the plain register path's pieces
+        } else if constexpr (GATHER == 2) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float* dst = bs + (gwave * 4 + j) * TileB::LDM + lane * ZPL;
+                if constexpr (ZPL == 2) *reinterpret_cast<float2*>(dst) = make_float2(tb.v[j * 2], tb.v[j * 2 + 1]);
+                else *dst = tb.v[j];
             }
         }
     };
@@ -744,7 +780,8 @@ __global__ __launch_bounds__(kGemmThreads, PIPE ? 3 : 4) void sgemm_kernel(GemmA
                 auto park = [&](int slice, float* as, float* bs) {
                     const bool tested = ragged_k && slice == nk - 1;
                     if (!wholeA || tested) ta.store(as);
-                    if (!wholeB || tested) tb.store(bs);
+                    if constexpr (GATHER != 0) gather_park(bs);
+                    else if (!wholeB || tested) tb.store(bs);
                 };
                 if (nk > 0) {
                     issue(0, As[0], Bs[0]);
@@ -1193,11 +1230,9 @@ static void launch_gather(int which, int shape, dim3 grid, hipStream_t st, const
     } else {
         switch (shape) {
             case 0: sgemm_kernel<true, false, false, 2, 2, 2, 2, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;
-            case 1: sgemm_kernel<true, false, false, 4, 1, 1, 3, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;
-            case 2: sgemm_kernel<true, false, false, 4, 1, 1, 2, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;
-            case 3: sgemm_kernel<true, false, false, 4, 1, 1, 1, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;
-            case 4: sgemm_kernel<true, false, false, 1, 4, 3, 1, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;
-            default: sgemm_kernel<true, false, false, 1, 4, 2, 1, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;
+            case 2: sgemm_kernel<true, false, false, 4, 1, 1, 2, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;    // 128 x 64
+            case 4: sgemm_kernel<true, false, false, 1, 4, 3, 1, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;    // 96 x 128
+            default: sgemm_kernel<true, false, false, 1, 4, 2, 1, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;   // 64 x 128
         }
     }
 }
@@ -1270,7 +1305,9 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     // tile shape: least padded work, ties to the earlier (larger) shape
     int shape = 0;
     double best = 0;
+    const bool gather_cols = cv && cv->mode == 4 && cv->patch;     // the gathered weight gradient: tiles of 128 or 64 columns
     for (int i = 0; i < kPlainShapes; ++i) {
+        if (gather_cols && kShapes[i].bn != 128 && kShapes[i].bn != 64) continue;
         const double work = (double)(cdiv(M, kShapes[i].bm) * kShapes[i].bm) *
                             (double)(cdiv(N, kShapes[i].bn) * kShapes[i].bn);
         if (i == 0 || work < best * 0.97) {

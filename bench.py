@@ -70,7 +70,7 @@ IM2COL_SUFFIX = "/im2col"
 COL_SUFFIX = "/col"
 EXTRA_WORKLOADS = [DEFAULT_WORKLOAD + IM2COL_SUFFIX, "alexnet_conv1_11x11s4_3x227x227_b128",
                    "alexnet_conv1_11x11s4_3x227x227_b128" + COL_SUFFIX, GEMM_WORKLOAD,
-                   "cifar_conv1_5x5_3x32x32_b128", "mnist_conv3x3_1x28x28_b64"]
+                   "cifar_conv1_5x5_3x32x32_b128", "cifar_conv2_5x5_32x15x15_b128", "mnist_conv3x3_1x28x28_b64"]
 
 
 def split_workload(workload):

@@ -1173,7 +1173,7 @@ struct TileShape {
 
 // Tile shapes on offer; the 128x128 default comes first and wins ties.
 static const TileShape kShapes[] = {{128, 128}, {128, 96}, {128, 64}, {128, 32}, {96, 128}, {64, 128}, {32, 128}};
-constexpr int kPlainShapes = 6;      // the last shape exists for the column-buffer forward product only
+constexpr int kPlainShapes = 6;      // the last shape exists for the products that write NCHW themselves (32 or fewer filters)
 
 template <bool AKC, bool BKC, bool PIPE>
 static void launch_shape(int shape, dim3 grid, hipStream_t st, const GemmArgs& a) {
@@ -1202,7 +1202,8 @@ static void launch_conv(int mode, int shape, dim3 grid, hipStream_t st, const Ge
         switch (shape) {
             case 0: sgemm_kernel<true, false, false, 2, 2, 2, 2, false, 3><<<grid, block, 0, st>>>(a); break;
             case 4: sgemm_kernel<true, false, false, 1, 4, 3, 1, false, 3><<<grid, block, 0, st>>>(a); break;    // 96 x 128
-            default: sgemm_kernel<true, false, false, 1, 4, 2, 1, false, 3><<<grid, block, 0, st>>>(a); break;   // 64 x 128
+            case 5: sgemm_kernel<true, false, false, 1, 4, 2, 1, false, 3><<<grid, block, 0, st>>>(a); break;    // 64 x 128
+            default: sgemm_kernel<true, false, false, 1, 4, 1, 1, false, 3><<<grid, block, 0, st>>>(a); break;   // 32 x 128
         }
     } else {
         switch (shape) {
@@ -1257,7 +1258,7 @@ static int conv_shape(int mode, long rows, long cols, long channels) {
     if ((mode != 1 && channels % KT != 0) || rows < 1) return -1;
     int best = -1;
     double best_work = 0;
-    for (int i = 0; i < (mode == 1 ? kPlainShapes + 1 : kPlainShapes); ++i) {
+    for (int i = 0; i < (mode != 2 ? kPlainShapes + 1 : kPlainShapes); ++i) {
         if (mode != 2 && kShapes[i].bn != 128) continue;
         const double work = (double)(cdiv(rows, kShapes[i].bm) * kShapes[i].bm) *
                             (mode != 2 ? 1.0 : (double)(cdiv(cols, kShapes[i].bn) * kShapes[i].bn));

@@ -277,7 +277,8 @@ class ConvPatchBackwardData(core.Op):
 
 
 class ConvPatchBackwardFilter(core.Op):
-    """inputs [gy, x, f] -> gf (f gives the shape only)."""
+    """inputs [gy, x, f] -> gf (f gives the shape only): ConvColBackwardFilter's sums with the patches read
+    from x (equal to it to rounding; bit for bit when both products take the same tile shape)."""
     available_impls = ("native_gpu",)
 
     def __init__(self, info):

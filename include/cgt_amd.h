@@ -410,7 +410,8 @@ int cgt_amd_conv_col_bwd_filter_f32(const float *gy, const float *col, long B, l
  * cgt_amd_im2col_f32 would have copied it from (zero outside the image) while
  * the GEMM loads its operand tile.  Any kernel, padding and stride; results
  * agree with the products over col to rounding (same sums, same order of z;
- * the forward product bit for bit).  x [B,C,H,W], f / gf [L,C,kh,kw], y / gy
+ * the forward product bit for bit, the weight gradient bit for bit when both
+ * take the same tile shape and therefore cut K into the same pieces).  x [B,C,H,W], f / gf [L,C,kh,kw], y / gy
  * [B,L,m,n] with m = (H + 2 ph - kh) / sh + 1.  The data gradient keeps the
  * column buffer (cgt_amd_conv_col_bwd_data_f32 + cgt_amd_col2im_f32). */
 

@@ -162,9 +162,12 @@ def make_inputs(cfg, batch=None, seed=0):
 
 
 class Stage(object):
-    def __init__(self, name, kernel, fn, work, bound, operand_bytes=None):
+    def __init__(self, name, kernel, fn, work, bound, operand_bytes=None, ref_bytes=None):
         self.name, self.kernel, self.fn, self.work, self.bound = name, kernel, fn, work, bound
         self.operand_bytes = operand_bytes      # GEMM stages: 4 * (|A| + |B| + |C|), the compulsory traffic
+        # HBM stages whose op moves fewer arrays than the reference's algorithm does (`work` is what
+        # the op as built has to move): the reference algorithm's bytes, the unit its figures are quoted in
+        self.ref_bytes = ref_bytes
         self.ms = self.ms_median = self.ms_min = self.ms_in_step = None
 
 
@@ -236,9 +239,19 @@ class LayerOnGpu(object):
                             2 * 4 * nelem(self.y), "hbm"))
         if cfg["lrn"]:
             size, alpha, beta, k = cfg["lrn"]
-            self.top, self.scale = empty(self.y.shape), empty(self.y.shape)
-            st.append(Stage("lrn_fwd", "lrn_fwd_flat_kernel or lrn_fwd_kernel", lambda: K.lrn_fwd(self.y, size, alpha, beta, k, out=(self.top, self.scale), stream=s),
-                            3 * 4 * nelem(self.y), "hbm"))
+            # what nn.cross_channel_lrn builds beside the fused conv ops: only `top` is stored and the
+            # gradient forms the scale again from x (two arrays forward, three backward); the literal
+            # composition keeps the reference's (top, scale) pair (three forward, four backward: `top`
+            # is formed again).  The reference's algorithm moves three and five.
+            lean_lrn = patch or fused_col
+            self.top = empty(self.y.shape)
+            self.scale = None if lean_lrn else empty(self.y.shape)
+            if lean_lrn:
+                st.append(Stage("lrn_fwd", "lrn_fwd_kernel", lambda: K.lrn_fwd(self.y, size, alpha, beta, k, out=self.top, stream=s, want_scale=False),
+                                2 * 4 * nelem(self.y), "hbm", ref_bytes=3 * 4 * nelem(self.y)))
+            else:
+                st.append(Stage("lrn_fwd", "lrn_fwd_flat_kernel or lrn_fwd_kernel", lambda: K.lrn_fwd(self.y, size, alpha, beta, k, out=(self.top, self.scale), stream=s),
+                                3 * 4 * nelem(self.y), "hbm"))
             act = self.top
         if cfg["pool"]:
             pk, pp, ps = cfg["pool"]
@@ -258,12 +271,14 @@ class LayerOnGpu(object):
         if cfg["lrn"]:
             self.gy_lrn = empty(self.y.shape)
             g_in = gy
-            st.append(Stage("lrn_bwd", "lrn_bwd_kernel",
-                            # as the Op's closure calls it: `top` is formed again from x and scale, not read.
-                            # The stage's bytes stay the five arrays of the reference's algorithm (x, top,
-                            # scale, cotangent in; one out), the unit the metric is quoted in; the kernel moves four
-                            lambda: K.lrn_bwd(self.y, None, self.scale, g_in, size, alpha, beta, out=self.gy_lrn, stream=s),
-                            5 * 4 * nelem(self.y), "hbm"))
+            if lean_lrn:    # x and the cotangent in, one array out
+                st.append(Stage("lrn_bwd", "lrn_bwd_x_kernel",
+                                lambda: K.lrn_bwd_from_x(self.y, g_in, size, alpha, beta, k, out=self.gy_lrn, stream=s),
+                                3 * 4 * nelem(self.y), "hbm", ref_bytes=5 * 4 * nelem(self.y)))
+            else:           # as the Op's closure calls it: `top` is formed again from x and scale, not read
+                st.append(Stage("lrn_bwd", "lrn_bwd_kernel",
+                                lambda: K.lrn_bwd(self.y, None, self.scale, g_in, size, alpha, beta, out=self.gy_lrn, stream=s),
+                                4 * 4 * nelem(self.y), "hbm", ref_bytes=5 * 4 * nelem(self.y)))
             gy = self.gy_lrn
         self.gy = gy
         self.gcol = empty((Bmn, Z))
@@ -713,6 +728,9 @@ def measure(workload, args, primary):
             rate = st.work / (st.ms_in_step * 1e-3) / scale
             row.update({"ms_in_step": round(st.ms_in_step, 4), unit + "_in_step": round(rate, 2),
                         "frac_in_step": round(rate / peak, 4)})
+        if st.bound == "hbm" and getattr(st, "ref_bytes", None):
+            row.update({"bytes_reference_algorithm": st.ref_bytes,
+                        "GBps_in_reference_bytes": round(st.ref_bytes / (clock(st) * 1e-3) / 1e9, 1)})
         if st.bound == "mfma":
             gemm_flops += st.work
             gemm_ms += clock(st)

@@ -54,6 +54,8 @@ PROTOTYPES = {
                             + [c_void_p, c_void_p]),
     "cgt_amd_lrn_bwd_recompute_f32": (c_int, [c_void_p] * 3 + [c_long] * 4 + [c_int, c_double, c_double]
                                       + [c_void_p, c_void_p]),
+    "cgt_amd_lrn_bwd_from_x_f32": (c_int, [c_void_p] * 2 + [c_long] * 4 + [c_int, c_double, c_double, c_double]
+                                   + [c_void_p, c_void_p]),
     "cgt_amd_sgemm": (c_int, [c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p,
                               c_long, c_void_p, c_long, c_void_p]),
     "cgt_amd_sgemm_noalloc": (c_int, [c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p,

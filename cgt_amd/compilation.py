@@ -218,6 +218,8 @@ def prebuild_standard_ops():
         (nn_ops.max_pool_2d.MaxPoolPullback(pinfo), [T4, T4, I4, T4]),
         (nn_ops.cross_channel_lrn.CrossChannelLRNForward(linfo), [T4]),
         (nn_ops.cross_channel_lrn.CrossChannelLRNBackward(linfo), [T4, T4, T4, T4]),
+        (nn_ops.cross_channel_lrn.CrossChannelLRNTop(linfo), [T4]),
+        (nn_ops.cross_channel_lrn.CrossChannelLRNBackwardFromX(linfo), [T4, T4]),
         (core.Mul22(False, True), [T2, T2]),
         (core.BatchedMul22(False, False), [T3, T3]),
         (core.Transpose((0, 3, 1, 2)), [T4]),

@@ -92,7 +92,7 @@ __device__ __forceinline__ void lrn_fwd_run(const float* __restrict__ x, float* 
             for (int j = 0; j < SIZE; ++j) acc += win[u + j] * win[u + j];
             const float s = kconst + acc * aos;
             if (c0 + u < ce) {
-                sp[(c0 + u) * hs] = s;
+                if (scale) sp[(c0 + u) * hs] = s;
                 tp[(c0 + u) * hs] = win[u + PRE] * pow_neg_beta(s, nbeta);
             }
         }
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_fwd_flat_kernel(
         }
         const v4f s = kconst + acc * aos;
         const v4f mid = w[PRE];
-        stream_store4(scale + f, s.x, s.y, s.z, s.w);
+        if (scale) stream_store4(scale + f, s.x, s.y, s.z, s.w);
         stream_store4(top + f, mid.x * pow_neg_beta(s.x, nbeta), mid.y * pow_neg_beta(s.y, nbeta),
                       mid.z * pow_neg_beta(s.z, nbeta), mid.w * pow_neg_beta(s.w, nbeta));
         return;
@@ -174,7 +174,7 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_fwd_flat_kernel(
             }
         }
         const float s = kconst + acc * aos;
-        scale[e] = s;
+        if (scale) scale[e] = s;
         top[e] = x[e] * pow_neg_beta(s, nbeta);
     }
 }
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_fwd_generic_kernel(
             acc += v * v;
         }
         const float s = kconst + acc * aos;
-        scale[base + (long)c * HW] = s;
+        if (scale) scale[base + (long)c * HW] = s;
         top[base + (long)c * HW] = x[base + (long)c * HW] * pow_neg_beta(s, nbeta);
     }
 }
@@ -318,6 +318,148 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_bwd_kernel(
     else lrn_bwd_run<SIZE, false, RECOMP>(x, top, scale, top_diff, bottom_diff, C, HW, blk, crun, nbeta, ratio);
 }
 
+// No stored scale: scale[ch] = k + (alpha/size) * sum of x^2 over the forward window of ch is formed
+// again from x (the window sum the forward kernels take, in the order of the walk), so the kernel
+// streams x and the cotangent in and the result out -- three arrays.  Every channel that enters
+// the ratio window needs its own forward window, so the run's halo of x is 2 (SIZE - 1) channels.
+template <int SIZE, bool DOWN>
+__device__ __forceinline__ void lrn_bwd_x_run(const float* __restrict__ x, const float* __restrict__ top_diff,
+                                              float* __restrict__ bottom_diff, int C, int HW, const LrnBlock& blk,
+                                              int crun, float aos, float nbeta, float kconst, float ratio) {
+    constexpr int PRE0 = SIZE - (SIZE + 1) / 2, POST0 = SIZE - PRE0 - 1, U = kLrnChunk;      // ratio window
+    constexpr int FPRE0 = (SIZE - 1) / 2, FPOST0 = SIZE - FPRE0 - 1;                         // forward window
+    constexpr int PRE = DOWN ? POST0 : PRE0, POST = DOWN ? PRE0 : POST0;
+    constexpr int FPRE = DOWN ? FPOST0 : FPRE0, FPOST = DOWN ? FPRE0 : FPOST0;
+    const int p = blk.px * kLrnThreads + threadIdx.x;
+    if (p >= HW) return;
+    const long n = blk.n;
+    const int cs0 = blk.run * crun, ce0 = min(C, cs0 + crun);
+    const int cs = DOWN ? C - ce0 : cs0, ce = DOWN ? C - cs0 : ce0;
+    const long hs = DOWN ? -(long)HW : (long)HW;
+    const long base = n * C * (long)HW + p + (DOWN ? (long)(C - 1) * HW : 0);
+    const float* xp = x + base;
+    const float* dp = top_diff + base;
+    float* bp = bottom_diff + base;
+
+    float xw[U + SIZE - 1];   // xw[j] = x[c0 + POST - FPRE + j]
+    float tr[U + SIZE - 1];   // tr[j] = (td*top/scale)[c0 - PRE + j]
+    float dr[U + POST];       // dr[j] = td[c0 + j]
+    float sr[U + POST];       // sr[j] = scale[c0 + j]^-beta
+    float xr[U + POST];       // xr[j] = x[c0 + j]
+    {
+        // channels cs - PRE .. cs + POST - 1 fill the window before the first centre
+        float xh[2 * (SIZE - 1) + 1], dh[SIZE];
+#pragma unroll
+        for (int i = 0; i < 2 * (SIZE - 1); ++i) {
+            const int c = cs - PRE - FPRE + i;
+            xh[i] = (c >= 0 && c < C) ? xp[c * hs] : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < SIZE - 1; ++j) {
+            const int c = cs - PRE + j;
+            dh[j] = (c >= 0 && c < C) ? dp[c * hs] : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < SIZE - 1; ++j) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int i = 0; i < SIZE; ++i) acc += xh[j + i] * xh[j + i];
+            const float sc = kconst + acc * aos;
+            const float pw = pow_neg_beta(sc, nbeta);
+            const float xc = xh[j + FPRE];
+            tr[j] = dh[j] * (xc * pw) / sc;
+            if (j >= PRE) {
+                dr[j - PRE] = dh[j];
+                sr[j - PRE] = pw;
+                xr[j - PRE] = xc;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < SIZE - 1; ++j) xw[j] = xh[SIZE - 1 + j];
+    }
+    for (int c0 = cs; c0 < ce; c0 += U) {
+        float dn[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int cx = c0 + POST + FPOST + u, cd = c0 + POST + u;
+            xw[SIZE - 1 + u] = (cx < C) ? xp[cx * hs] : 0.0f;
+            dn[u] = (cd < C) ? dp[cd * hs] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int i = 0; i < SIZE; ++i) acc += xw[u + i] * xw[u + i];
+            const float sc = kconst + acc * aos;
+            const float pw = pow_neg_beta(sc, nbeta);
+            const float xc = xw[u + FPRE];
+            dr[POST + u] = dn[u];
+            sr[POST + u] = pw;
+            xr[POST + u] = xc;
+            tr[SIZE - 1 + u] = dn[u] * (xc * pw) / sc;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int j = 0; j < SIZE; ++j) acc += tr[u + j];
+            if (c0 + u < ce) bp[(c0 + u) * hs] = dr[u] * sr[u] - ratio * xr[u] * acc;
+        }
+#pragma unroll
+        for (int j = 0; j < SIZE - 1; ++j) {
+            tr[j] = tr[U + j];
+            xw[j] = xw[U + j];
+        }
+#pragma unroll
+        for (int j = 0; j < POST; ++j) {
+            dr[j] = dr[U + j];
+            sr[j] = sr[U + j];
+            xr[j] = xr[U + j];
+        }
+    }
+}
+
+template <int SIZE>
+__global__ __launch_bounds__(kLrnThreads) void lrn_bwd_x_kernel(
+    const float* __restrict__ x, const float* __restrict__ top_diff, float* __restrict__ bottom_diff, int C, int HW,
+    int crun, float aos, float nbeta, float kconst, float ratio) {
+    const LrnBlock blk = lrn_block(HW, C, crun);
+    if (blk.run & 1) lrn_bwd_x_run<SIZE, true>(x, top_diff, bottom_diff, C, HW, blk, crun, aos, nbeta, kconst, ratio);
+    else lrn_bwd_x_run<SIZE, false>(x, top_diff, bottom_diff, C, HW, blk, crun, aos, nbeta, kconst, ratio);
+}
+
+// any window length, from x alone
+__global__ __launch_bounds__(kLrnThreads) void lrn_bwd_x_generic_kernel(
+    const float* __restrict__ x, const float* __restrict__ top_diff, float* __restrict__ bottom_diff, int C, int HW,
+    int crun, int size, float aos, float nbeta, float kconst, float ratio) {
+    const int pre = size - (size + 1) / 2, post = size - pre - 1;
+    const int fpre = (size - 1) / 2, fpost = size - fpre - 1;
+    const LrnBlock blk = lrn_block(HW, C, crun);
+    const int p = blk.px * kLrnThreads + threadIdx.x;
+    if (p >= HW) return;
+    const long n = blk.n;
+    const int cs = blk.run * crun, ce = min(C, cs + crun);
+    const long base = n * C * (long)HW + p;
+    auto scale_at = [&](int ch) {
+        float acc = 0.0f;
+        for (int cc = max(0, ch - fpre); cc <= min(C - 1, ch + fpost); ++cc) {
+            const float v = x[base + (long)cc * HW];
+            acc += v * v;
+        }
+        return kconst + acc * aos;
+    };
+    for (int c = cs; c < ce; ++c) {
+        float acc = 0.0f;
+        for (int cc = max(0, c - pre); cc <= min(C - 1, c + post); ++cc) {
+            const long i = base + (long)cc * HW;
+            const float sc = scale_at(cc);
+            acc += top_diff[i] * (x[i] * pow_neg_beta(sc, nbeta)) / sc;
+        }
+        const long i = base + (long)c * HW;
+        bottom_diff[i] = top_diff[i] * pow_neg_beta(scale_at(c), nbeta) - ratio * x[i] * acc;
+    }
+}
+
 __global__ __launch_bounds__(kLrnThreads) void lrn_bwd_generic_kernel(
     const float* __restrict__ x, const float* __restrict__ top, const float* __restrict__ scale,
     const float* __restrict__ top_diff, float* __restrict__ bottom_diff, int C, int HW, int crun,
@@ -374,7 +516,7 @@ CGT_API int cgt_amd_lrn_fwd_f32(const float* x, long N, long C, long H, long W, 
     if (N * C * H * W == 0 && N >= 0 && C >= 0 && H >= 0 && W >= 0 && size >= 1) return CGT_AMD_OK;
     int rc = check_lrn("lrn_fwd", N, C, H, W, size);
     if (rc) return rc;
-    CGT_ARG_CHECK(x && top && scale, "lrn_fwd: null pointer");
+    CGT_ARG_CHECK(x && top, "lrn_fwd: null pointer");          // scale == nullptr: not stored
     CGT_ARG_CHECK(k > 0, "lrn_fwd: k must be positive");
     const int HW = (int)(H * W);
     const int crun = pick_crun(N, (int)C, HW, size);
@@ -383,8 +525,9 @@ CGT_API int cgt_amd_lrn_fwd_f32(const float* x, long N, long C, long H, long W, 
     const float aos = (float)(alpha / size), nbeta = (float)(-beta), kc = (float)k;
     const long total = N * C * HW;
     // the flat kernel wins once the arrays no longer sit in the last-level cache
-    // (measured: 37 M floats 0.066 vs 0.098 ms, 24 M 0.051 vs 0.067, 9 M 0.022 vs 0.017)
-    const bool flat = total >= (16L << 20) && total < (1L << 31) && reinterpret_cast<uintptr_t>(top) % 16 == 0 &&
+    // (measured: 37 M floats 0.066 vs 0.098 ms, 24 M 0.051 vs 0.067, 9 M 0.022 vs 0.017) -- when both
+    // outputs are stored; with top alone the pixel-per-lane kernel is ahead (37 M floats: 0.057 vs 0.071)
+    const bool flat = scale && total >= (16L << 20) && total < (1L << 31) && reinterpret_cast<uintptr_t>(top) % 16 == 0 &&
                       reinterpret_cast<uintptr_t>(scale) % 16 == 0;
     const dim3 flat_grid((unsigned)cdiv(cdiv(total, 4), kLrnThreads));
 #define LRN_FWD_CASE(S)                                                                           \
@@ -445,4 +588,31 @@ CGT_API int cgt_amd_lrn_bwd_recompute_f32(const float* x, const float* scale, co
                                           long H, long W, int size, double alpha, double beta, float* bottom_diff,
                                           void* stream) {
     return lrn_bwd(x, nullptr, scale, top_diff, N, C, H, W, size, alpha, beta, bottom_diff, stream);
+}
+
+CGT_API int cgt_amd_lrn_bwd_from_x_f32(const float* x, const float* top_diff, long N, long C, long H, long W, int size,
+                                       double alpha, double beta, double k, float* bottom_diff, void* stream) {
+    if (N * C * H * W == 0 && N >= 0 && C >= 0 && H >= 0 && W >= 0 && size >= 1) return CGT_AMD_OK;
+    int rc = check_lrn("lrn_bwd_from_x", N, C, H, W, size);
+    if (rc) return rc;
+    CGT_ARG_CHECK(x && top_diff && bottom_diff, "lrn_bwd_from_x: null pointer");
+    CGT_ARG_CHECK(k > 0, "lrn_bwd_from_x: k must be positive");
+    const int HW = (int)(H * W);
+    const int crun = pick_crun(N, (int)C, HW, size);
+    dim3 grid((unsigned)(cdiv(HW, kLrnThreads) * cdiv(C, crun) * N)), block(kLrnThreads);
+    hipStream_t st = as_stream(stream);
+    const float aos = (float)(alpha / size), nbeta = (float)(-beta), kc = (float)k, ratio = (float)(2. * alpha * beta / size);
+#define LRN_BWD_X_CASE(S)                                                                                     \
+    case S:                                                                                                   \
+        lrn_bwd_x_kernel<S><<<grid, block, 0, st>>>(x, top_diff, bottom_diff, (int)C, HW, crun, aos, nbeta, kc, ratio); \
+        break;
+    switch (size) {
+        LRN_BWD_X_CASE(1) LRN_BWD_X_CASE(2) LRN_BWD_X_CASE(3) LRN_BWD_X_CASE(4) LRN_BWD_X_CASE(5)
+        LRN_BWD_X_CASE(6) LRN_BWD_X_CASE(7) LRN_BWD_X_CASE(8) LRN_BWD_X_CASE(9)
+        default:
+            lrn_bwd_x_generic_kernel<<<grid, block, 0, st>>>(x, top_diff, bottom_diff, (int)C, HW, crun, size, aos, nbeta, kc, ratio);
+    }
+#undef LRN_BWD_X_CASE
+    CGT_LAUNCH_CHECK("lrn_bwd_x_kernel");
+    return CGT_AMD_OK;
 }

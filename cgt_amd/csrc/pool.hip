@@ -426,6 +426,61 @@ __global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_padded_kernel(
     }
 }
 
+// Windows that do not overlap (kernel <= stride): a cell has at most one addend, so the pullback
+// is a scatter with no order to keep.  A workgroup builds its planes in LDS -- zeros, then every
+// window's cotangent at the cell its mask names (0 + g, times the rectify mask: the bits the
+// gather form produces) -- and writes them out as one contiguous run of 16-byte units.  The
+// index arithmetic is per window, not per float of the result.
+__global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_padded_scatter_kernel(
+    const int* __restrict__ mask, const float* __restrict__ top_diff, const signed char* __restrict__ relu_mask,
+    float* __restrict__ dst, long nplanes, int HW, int W, int PP, PaddedPlanes lay, int planes_per_wg, long tail_units) {
+    extern __shared__ float tile[];
+    const long p0 = (long)blockIdx.x * planes_per_wg;
+    const long left = nplanes - p0;
+    const int np = left < planes_per_wg ? (int)left : planes_per_wg;
+    const long total_units = nplanes * (long)(lay.plane / 4);
+    for (long t = (long)blockIdx.x * kPoolThreads + threadIdx.x; t < tail_units; t += (long)gridDim.x * kPoolThreads)
+        stream_store4(dst + (total_units + t) * 4, 0.f, 0.f, 0.f, 0.f);
+    const int nunits = np * (lay.plane / 4);
+    float4* t4 = reinterpret_cast<float4*>(tile);
+    for (int u = threadIdx.x; u < nunits; u += kPoolThreads) t4[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    __syncthreads();
+    const int nwin = np * PP;
+    const float rPP = 1.0f / PP, rW = 1.0f / W;
+    const int* mk = mask + p0 * PP;
+    const float* td = top_diff + p0 * PP;
+    for (int base = threadIdx.x; base < nwin; base += kPoolThreads * 4) {
+        int m[4], pl[4];
+        float g[4], r[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int o = base + u * kPoolThreads;
+            m[u] = -1;
+            if (o < nwin) {
+                m[u] = mk[o];
+                g[u] = td[o];
+            }
+            pl[u] = fastdiv(o, rPP);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            m[u] = (unsigned)m[u] < (unsigned)HW ? m[u] : -1;     // -1: a window that saw no value
+            r[u] = (relu_mask && m[u] >= 0) ? (float)relu_mask[(p0 + pl[u]) * (long)HW + m[u]] : 1.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (m[u] >= 0) {
+                const int h = fastdiv(m[u], rW), w = m[u] - h * W;
+                float v = 0.0f + g[u];
+                if (relu_mask) v = r[u] * v;
+                tile[pl[u] * lay.plane + lay.lead + (h + lay.top) * lay.pitch + w] = v;
+            }
+    }
+    __syncthreads();
+    float4* out = reinterpret_cast<float4*>(dst + p0 * (long)lay.plane);
+    for (int u = threadIdx.x; u < nunits; u += kPoolThreads) out[u] = t4[u];
+}
+
 static int check_pool(const char* what, long N, long C, long H, long W, int kh, int kw, int ph,
                       int pw, int sh, int sw, long PH, long PW) {
     CGT_ARG_CHECK(N >= 0 && C >= 0 && H >= 0 && W >= 0 && PH >= 0 && PW >= 0, "%s: negative shape", what);
@@ -502,6 +557,20 @@ static int launch_pool_fwd(G g, const float* bottom, long nplanes, long H, long 
 template <class G>
 static int launch_pool_bwd(G g, const int* mask, const float* top_diff, long nplanes, long H, long W,
                            long PH, long PW, float* bottom_diff, hipStream_t st) {
+    // windows that do not overlap: the scatter form, planes built in LDS and written as one run
+    if (g.kh() <= g.sh() && g.kw() <= g.sw() && (H * W) % 4 == 0 && H * W * (long)sizeof(float) <= 48 * 1024 &&
+        reinterpret_cast<uintptr_t>(bottom_diff) % 16 == 0) {
+        const long plane_bytes = H * W * (long)sizeof(float);
+        long ppw = std::max(1L, std::min((32 * 1024) / plane_bytes, nplanes / 2048));
+        ppw = std::min(ppw, (kFastdivLimit - 1) / (PH * PW));
+        if (ppw >= 1) {
+            const PaddedPlanes lay = {0, 0, (int)W, (int)(H * W), 0};
+            max_pool_bwd_padded_scatter_kernel<<<dim3((unsigned)cdiv(nplanes, ppw)), dim3(kPoolThreads), (size_t)(ppw * plane_bytes), st>>>(
+                mask, top_diff, nullptr, bottom_diff, nplanes, (int)(H * W), (int)W, (int)(PH * PW), lay, (int)ppw, 0);
+            CGT_LAUNCH_CHECK("max_pool_bwd_padded_scatter_kernel");
+            return CGT_AMD_OK;
+        }
+    }
     if constexpr (G::is_static) {
         const long BH = cdiv(H, (long)G::kSH), BW = cdiv(W, (long)G::kSW);
         if (BH * BW <= (1L << 18) && H * W < (1L << 30)) {
@@ -567,6 +636,18 @@ int launch_pool_pullback_padded(const int* mask, const float* top_diff, const si
     // one wavefront per chunk of 512 units of a plane (grid-stride beyond 64 K workgroups)
     const long blocks = std::max(1L, std::min(cdiv(nplanes * cdiv(upp, 512L), (long)(kPoolThreads / 64)), 1L << 16));
     hipStream_t st = as_stream(stream);
+    const long plane_bytes = lay.plane * (long)sizeof(float);
+    if (kh <= sh && kw <= sw && plane_bytes <= 48 * 1024 && H * W < kFastdivLimit) {
+        // planes per workgroup: up to 32 KB of LDS, and enough workgroups for every CU to hold several
+        long ppw = std::max(1L, std::min((32 * 1024) / plane_bytes, nplanes / 2048));
+        ppw = std::min(ppw, (kFastdivLimit - 1) / (PH * PW));
+        if (ppw >= 1) {
+            max_pool_bwd_padded_scatter_kernel<<<dim3((unsigned)cdiv(nplanes, ppw)), dim3(kPoolThreads), (size_t)(ppw * plane_bytes), st>>>(
+                mask, top_diff, relu_mask, dst, nplanes, (int)(H * W), (int)W, (int)(PH * PW), lay, (int)ppw, tail_units);
+            CGT_LAUNCH_CHECK("max_pool_bwd_padded_scatter_kernel");
+            return CGT_AMD_OK;
+        }
+    }
 #define X(KH, KW, PH_, PW_, SH, SW)                                                                              \
     if (kh == KH && kw == KW && ph == PH_ && pw == PW_ && sh == SH && sw == SW) {                                \
         max_pool_bwd_padded_kernel<<<dim3((unsigned)blocks), dim3(kPoolThreads), 0, st>>>(                       \

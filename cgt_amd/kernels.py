@@ -94,16 +94,34 @@ def max_pool_pullback(xshape, mask, gtop, kernel, pad, stride, out=None, stream=
     return gb
 
 
-def lrn_fwd(x, size, alpha, beta, k=1.0, out=None, stream=None):
+def lrn_fwd(x, size, alpha, beta, k=1.0, out=None, stream=None, want_scale=True):
     """CrossChannelLRNForward op (reference cgt/nn_ops/cross_channel_lrn.py:15-63):
-    returns (top, scale).  k=1 is the reference; other k is an extension."""
+    returns (top, scale).  k=1 is the reference; other k is an extension.
+    want_scale=False: the scale array is not stored and only top is returned."""
     _f32(x)
     N, C, H, W = x.shape
+    if not want_scale:
+        top = _out(out, x.shape)
+        capi.check(capi.lib().cgt_amd_lrn_fwd_f32(x.ptr, N, C, H, W, int(size), float(alpha), float(beta),
+                                                  float(k), top.ptr, None, stream))
+        return top
     top = _out(out[0] if out else None, x.shape)
     scale = _out(out[1] if out else None, x.shape)
     capi.check(capi.lib().cgt_amd_lrn_fwd_f32(x.ptr, N, C, H, W, int(size), float(alpha), float(beta),
                                               float(k), top.ptr, scale.ptr, stream))
     return top, scale
+
+
+def lrn_bwd_from_x(x, gtop, size, alpha, beta, k=1.0, out=None, stream=None):
+    """The LRN gradient from x and the cotangent alone (scale and top are formed again in the kernel)."""
+    _f32(x, gtop)
+    N, C, H, W = x.shape
+    if gtop.shape != x.shape:
+        raise ValueError("LRN backward operands must be float32 arrays of x's shape")
+    gb = _out(out, x.shape)
+    capi.check(capi.lib().cgt_amd_lrn_bwd_from_x_f32(x.ptr, gtop.ptr, N, C, H, W, int(size), float(alpha), float(beta),
+                                                     float(k), gb.ptr, stream))
+    return gb
 
 
 def lrn_bwd(x, top, scale, gtop, size, alpha, beta, out=None, stream=None):

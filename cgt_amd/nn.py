@@ -19,6 +19,7 @@ conv_algo("im2col") keeps the literal composition, every op on the GPU.
 """
 from . import core
 from .nn_ops import conv_col, conv_same
+from .nn_ops import cross_channel_lrn as _lrn
 from .nn_ops.cross_channel_lrn import cross_channel_lrn  # noqa: F401
 from .nn_ops.im2col import im2col
 from .nn_ops.max_pool_2d import MaxPool, PoolInfo
@@ -62,14 +63,16 @@ _CONV_FUSION = True
 
 
 def conv_fusion(on=None):
-    """Whether SpatialConvolution's bias add and a rectify that follows a fused convolution
-    go into the convolution's epilogue (default) or stay separate ops.  Returns the
-    previous setting."""
+    """Whether the fusions around the layer's ops are built (default) or every op stays the
+    reference's: SpatialConvolution's bias add and a rectify that follows a fused convolution
+    in the convolution's epilogue, a pool pullback written straight into the padded cotangent,
+    and cross_channel_lrn without a stored scale array.  Returns the previous setting."""
     global _CONV_FUSION
     old = _CONV_FUSION
     if on is not None:
         _CONV_FUSION = bool(on)
         conv_same.FUSE_POOL_PULLBACK = bool(on)
+        _lrn.STORE_TOP_ONLY = bool(on)
     return old
 
 

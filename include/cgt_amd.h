@@ -229,6 +229,9 @@ int cgt_amd_max_pool_pullback_f32(const int *mask, const float *top_diff,
  * pre = (size-1)/2, post = size-pre-1, window clipped to [0,C);
  * top = x * scale^(-beta).  k = 1 is the reference (it has no k parameter).
  * Requires 1 <= size <= C, as the reference kernel does.
+ * scale == NULL: the scale array is not stored (for callers that only keep top,
+ * as cross_channel_lrn() does, cgt/nn_ops/cross_channel_lrn.py:106-108; the
+ * gradient then comes from cgt_amd_lrn_bwd_from_x_f32).
  * Replaces LRNFillScale + LRNComputeOutput (include/lrn.cuh:3-52) and
  * launchker of CrossChannelLRNForward (cgt/nn_ops/cross_channel_lrn.py:27-39). */
 int cgt_amd_lrn_fwd_f32(const float *x, long N, long C, long H, long W,
@@ -254,6 +257,17 @@ int cgt_amd_lrn_bwd_f32(const float *x, const float *top, const float *scale,
 int cgt_amd_lrn_bwd_recompute_f32(const float *x, const float *scale, const float *top_diff,
                                   long N, long C, long H, long W, int size, double alpha,
                                   double beta, float *bottom_diff, void *stream);
+
+/* The same from x and top_diff alone: scale = k + (alpha/size) * window sum of
+ * x^2 and top = x * scale^(-beta) are formed again inside the kernel, so three
+ * arrays are streamed (x, top_diff, bottom_diff) instead of five.  Equal to
+ * cgt_amd_lrn_bwd_f32 on the forward's outputs up to rounding (the window sum
+ * may be taken in another order than the forward kernel took it).  `k` is the
+ * forward's additive constant.  What the gradient of nn.cross_channel_lrn
+ * calls when the scale array was not stored. */
+int cgt_amd_lrn_bwd_from_x_f32(const float *x, const float *top_diff, long N, long C, long H,
+                               long W, int size, double alpha, double beta, double k,
+                               float *bottom_diff, void *stream);
 
 /* ---------------------------------------------------------------- GEMM */
 

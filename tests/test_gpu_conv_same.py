@@ -234,7 +234,9 @@ POOLS = [((2, 2), (0, 0), (2, 2)), ((3, 3), (0, 0), (2, 2)), ((3, 3), (1, 1), (2
 
 
 @pytest.mark.parametrize("pk,pp,ps", POOLS)
-@pytest.mark.parametrize("shape,kernel", [((3, 5, 14, 12), (3, 3)), ((2, 3, 55, 55), (5, 5)), ((1, 7, 9, 31), (1, 7)), ((2, 4, 6, 5), (7, 3))])
+@pytest.mark.parametrize("shape,kernel", [((3, 5, 14, 12), (3, 3)), ((2, 3, 55, 55), (5, 5)), ((1, 7, 9, 31), (1, 7)), ((2, 4, 6, 5), (7, 3)),
+                                          ((41, 101, 6, 5), (3, 3)),        # many small planes: several per workgroup, the last one short
+                                          ((64, 128, 56, 56), (3, 3))])     # the VGG layer at full size
 def test_pool_pullback_written_into_the_padded_layout_is_bit_exact(K, pk, pp, ps, shape, kernel):
     # one pass instead of MaxPoolPullback -> (rectify mask *) -> ConvPad: the same bits, every float of
     # the padded buffer written (it starts out poisoned)
@@ -245,7 +247,9 @@ def test_pool_pullback_written_into_the_padded_layout_is_bit_exact(K, pk, pp, ps
     top, mask = K.max_pool(to_gpu(act), pk, pp, ps)
     if top.size == 0:
         pytest.skip("the pool has no output for this shape")
-    gtop = to_gpu((rs.randn(*top.shape) * 10.0 ** rs.randint(-3, 4, top.shape)).astype(np.float32))
+    gtop_h = (rs.randn(*top.shape) * 10.0 ** rs.randint(-3, 4, top.shape)).astype(np.float32)
+    gtop_h[rs.rand(*top.shape) < 0.05] = -0.0           # 0 + (-0) = +0 in the reference's scatter-add
+    gtop = to_gpu(gtop_h)
     rmask = to_gpu((rs.rand(*shape) < 0.6).astype(np.int8))
     want_plain = K.conv_same_pad(K.max_pool_pullback(shape, mask, gtop, pk, pp, ps), kernel).get()
     want_relu = K.conv_same_pad(K.elwise_binary("*", rmask, K.max_pool_pullback(shape, mask, gtop, pk, pp, ps)), kernel).get()

@@ -248,6 +248,14 @@ def test_lrn_vs_oracle(K, shape, size, alpha, beta, k):
     assert np.array_equal(recomputed.view(np.uint32), with_top.view(np.uint32))
     tgb = O.lrn_bwd(x64, ttop, tscale, g.astype(np.float64), size, alpha, beta)
     assert relfro(recomputed, tgb) <= 1e-5
+    # without a stored scale: top alone has the bits of the pair's top where the same kernel wrote
+    # both; the gradient from x and the cotangent alone forms the scale again (k goes in)
+    top_only = K.lrn_fwd(xg, size, alpha, beta, k, want_scale=False).get()
+    assert relfro(top_only, ttop) <= 5e-6
+    if x.size < (16 << 20):
+        assert np.array_equal(top_only.view(np.uint32), top.view(np.uint32))
+    from_x = K.lrn_bwd_from_x(xg, gg, size, alpha, beta, k).get()
+    assert relfro(from_x, tgb) <= 1e-5 and relfro(from_x, with_top) <= 1e-6
 
 
 @pytest.mark.parametrize("shape,size", [((5, 7, 701, 685), 5), ((5, 7, 701, 685), 4), ((2, 9, 1024, 1024), 3)])
@@ -264,6 +272,9 @@ def test_lrn_forward_large_arrays(K, shape, size):
     assert relfro(scale, rscale) <= 1e-6 and relfro(top, rtop) <= 5e-6
     assert np.max(np.abs(scale - rscale) / rscale) <= 1e-5
     assert np.max(np.abs(top - rtop) / (np.abs(rtop) + 1e-6)) <= 1e-4
+    # top alone (no scale array): the pixel-per-lane kernel at this size too
+    top_only = K.lrn_fwd(gpu(x), size, 0.3, 0.75, 1.0, want_scale=False).get()
+    assert relfro(top_only, rtop) <= 5e-6 and np.max(np.abs(top_only - rtop) / (np.abs(rtop) + 1e-6)) <= 1e-4
 
 
 def test_lrn_rejects_size_above_channels(K):

@@ -78,9 +78,13 @@ def test_im2col(cgt):
         assert abs(lhs - rhs) <= 1e-5 * abs(lhs)
 
 
-def test_lrn(cgt):
-    # cgt/tests/test_imgproc.py:79-97: randn(4,8,16,16), localsize 4, alpha .1, beta .5
+@pytest.mark.parametrize("top_only", [True, False])
+def test_lrn(cgt, top_only, monkeypatch):
+    # cgt/tests/test_imgproc.py:79-97: randn(4,8,16,16), localsize 4, alpha .1, beta .5; as the op
+    # that stores top alone (what cross_channel_lrn builds) and as the reference's tuple-valued op
     from cgt_amd.nn import cross_channel_lrn
+    from cgt_amd.nn_ops import cross_channel_lrn as L
+    monkeypatch.setattr(L, "STORE_TOP_ONLY", top_only)
     np.random.seed(0)
     Xval = np.random.randn(4, 8, 16, 16).astype(np.float32)
     X = cgt.constant(Xval)
@@ -91,6 +95,8 @@ def test_lrn(cgt):
     assert relfro(y.get(), top64) <= TOL
     a = np.random.rand(*y.shape).astype(np.float32)
     g = cgt.grad(y, [X], goutput=a)[0]
+    assert type(y.op).__name__ == ("CrossChannelLRNTop" if top_only else "TupleIndex")
+    assert type(g.op).__name__ == ("CrossChannelLRNBackwardFromX" if top_only else "CrossChannelLRNBackward")
     assert relfro(g.get(), O.lrn_bwd(Xval.astype(np.float64), top64, scale64, a.astype(np.float64), 4, .1, .5)) <= TOL
 
 
@@ -99,9 +105,15 @@ def test_lrn_k_extension(cgt):
     import torch.nn.functional as F
     from cgt_amd.nn import cross_channel_lrn
     Xval = np.random.RandomState(1).randn(2, 16, 5, 6).astype(np.float32)
-    y = cross_channel_lrn(cgt.constant(Xval), 5, 1e-2, .75, k=2.0)
-    ref = F.local_response_norm(torch.from_numpy(Xval).double(), 5, alpha=1e-2, beta=.75, k=2.0).numpy()
-    assert relfro(y.get(), ref) <= TOL
+    X = cgt.constant(Xval)
+    y = cross_channel_lrn(X, 5, 1e-2, .75, k=2.0)
+    xt = torch.from_numpy(Xval).double().requires_grad_(True)
+    ref = F.local_response_norm(xt, 5, alpha=1e-2, beta=.75, k=2.0)
+    assert relfro(y.get(), ref.detach().numpy()) <= TOL
+    # the gradient forms the scale again from X: k goes into it
+    a = np.random.RandomState(2).rand(*Xval.shape).astype(np.float32)
+    ref.backward(torch.from_numpy(a).double())
+    assert relfro(cgt.grad(y, [X], goutput=a)[0].get(), xt.grad.numpy()) <= TOL
 
 
 @pytest.mark.parametrize("tA,tB", [(False, False), (False, True), (True, False), (True, True)])

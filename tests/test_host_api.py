@@ -65,6 +65,7 @@ def test_available_impls_and_masks():
     ops = [I.Im2Col(I.Im2ColInfo(3, 3, 1, 1, 1, 1)), I.Col2Im(I.Im2ColInfo(3, 3, 1, 1, 1, 1)),
            P.MaxPool(P.PoolInfo(2, 2, 0, 0, 2, 2)), P.MaxPoolPullback(P.PoolInfo(2, 2, 0, 0, 2, 2)),
            L.CrossChannelLRNForward(L.LRNInfo(5, 1e-4, .75)), L.CrossChannelLRNBackward(L.LRNInfo(5, 1e-4, .75)),
+           L.CrossChannelLRNTop(L.LRNInfo(5, 1e-4, .75)), L.CrossChannelLRNBackwardFromX(L.LRNInfo(5, 1e-4, .75)),
            core.Mul22(False, True), core.BatchedMul22(False, False)]
     for op in ops:
         assert "native_gpu" in op.available_impls and op.return_type == "byref"
@@ -98,7 +99,7 @@ def test_closure_struct_layouts():
 
 def test_prebuild_standard_ops_exports_call_symbols():
     built = compilation.prebuild_standard_ops()
-    assert len(built) == 31
+    assert len(built) == 33
     for c in built:
         assert c.fptr_address and c.return_type in ("byref", "byval") and c.kind == "native"
     assert [c.return_type for c in built].count("byval") == 2

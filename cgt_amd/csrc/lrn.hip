@@ -59,7 +59,7 @@ constexpr int kLrnChunk = 8;
 template <int SIZE, bool DOWN>
 __device__ __forceinline__ void lrn_fwd_run(const float* __restrict__ x, float* __restrict__ top,
                                             float* __restrict__ scale, int C, int HW, const LrnBlock& blk,
-                                            int crun, float aos, float nbeta, float kconst) {
+                                            int crun, float aos, float nbeta, float kconst, bool stream_out) {
     constexpr int PRE0 = (SIZE - 1) / 2, POST0 = SIZE - PRE0 - 1, U = kLrnChunk;
     constexpr int PRE = DOWN ? POST0 : PRE0, POST = DOWN ? PRE0 : POST0;
     const int p = blk.px * kLrnThreads + threadIdx.x;
@@ -93,7 +93,9 @@ __device__ __forceinline__ void lrn_fwd_run(const float* __restrict__ x, float* 
             const float s = kconst + acc * aos;
             if (c0 + u < ce) {
                 if (scale) sp[(c0 + u) * hs] = s;
-                tp[(c0 + u) * hs] = win[u + PRE] * pow_neg_beta(s, nbeta);
+                const float t = win[u + PRE] * pow_neg_beta(s, nbeta);
+                if (stream_out) __builtin_nontemporal_store(t, &tp[(c0 + u) * hs]);
+                else tp[(c0 + u) * hs] = t;
             }
         }
 #pragma unroll
@@ -104,10 +106,10 @@ __device__ __forceinline__ void lrn_fwd_run(const float* __restrict__ x, float* 
 template <int SIZE>
 __global__ __launch_bounds__(kLrnThreads) void lrn_fwd_kernel(
     const float* __restrict__ x, float* __restrict__ top, float* __restrict__ scale, int C,
-    int HW, int crun, float aos, float nbeta, float kconst) {
+    int HW, int crun, float aos, float nbeta, float kconst, int stream_out) {
     const LrnBlock blk = lrn_block(HW, C, crun);
-    if (blk.run & 1) lrn_fwd_run<SIZE, true>(x, top, scale, C, HW, blk, crun, aos, nbeta, kconst);
-    else lrn_fwd_run<SIZE, false>(x, top, scale, C, HW, blk, crun, aos, nbeta, kconst);
+    if (blk.run & 1) lrn_fwd_run<SIZE, true>(x, top, scale, C, HW, blk, crun, aos, nbeta, kconst, stream_out != 0);
+    else lrn_fwd_run<SIZE, false>(x, top, scale, C, HW, blk, crun, aos, nbeta, kconst, stream_out != 0);
 }
 
 // Flat variant for large arrays.  The stores are two thirds of the forward
@@ -529,13 +531,16 @@ CGT_API int cgt_amd_lrn_fwd_f32(const float* x, long N, long C, long H, long W, 
     // outputs are stored; with top alone the pixel-per-lane kernel is ahead (37 M floats: 0.057 vs 0.071)
     const bool flat = scale && total >= (16L << 20) && total < (1L << 31) && reinterpret_cast<uintptr_t>(top) % 16 == 0 &&
                       reinterpret_cast<uintptr_t>(scale) % 16 == 0;
+    // an output too large to stay in the last-level cache for its reader is stored past it
+    // (AlexNet conv1 layer, top alone: 0.008 ms of the step, a third of it in the kernels that follow)
+    const int stream_out = total >= (16L << 20) ? 1 : 0;
     const dim3 flat_grid((unsigned)cdiv(cdiv(total, 4), kLrnThreads));
 #define LRN_FWD_CASE(S)                                                                           \
     case S:                                                                                       \
         if (flat)                                                                                 \
             lrn_fwd_flat_kernel<S><<<flat_grid, block, 0, st>>>(x, top, scale, (int)C, HW, (unsigned)total, aos, nbeta, kc); \
         else                                                                                      \
-            lrn_fwd_kernel<S><<<grid, block, 0, st>>>(x, top, scale, (int)C, HW, crun, aos, nbeta, kc); \
+            lrn_fwd_kernel<S><<<grid, block, 0, st>>>(x, top, scale, (int)C, HW, crun, aos, nbeta, kc, stream_out); \
         break;
     switch (size) {
         LRN_FWD_CASE(1) LRN_FWD_CASE(2) LRN_FWD_CASE(3) LRN_FWD_CASE(4) LRN_FWD_CASE(5)

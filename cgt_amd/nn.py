@@ -41,10 +41,24 @@ def conv_algo(name=None):
     return old
 
 
+def _check_geometry(x, channels, kernelshape, pad, stride):
+    """The reference's shape rule, (H + 2p - k) // s + 1 (cgt/nn_ops/im2col.py:36-41), goes to zero or
+    below when the kernel does not fit the padded image; say so here instead of failing in an allocation."""
+    B, K, H, W = x.shape
+    if K != channels:
+        raise ValueError("conv2d: the image has %d channels, the filters take %d" % (K, channels))
+    if min(stride) < 1 or min(pad) < 0 or min(kernelshape) < 1:
+        raise ValueError("conv2d: bad geometry kernel=%s pad=%s stride=%s" % (kernelshape, pad, stride))
+    if H + 2 * pad[0] < kernelshape[0] or W + 2 * pad[1] < kernelshape[1]:
+        raise ValueError("conv2d: the %dx%d kernel is larger than the %dx%d image padded by %s"
+                         % (kernelshape[0], kernelshape[1], H, W, tuple(pad)))
+
+
 def conv2d(x_BKRC, f_LKrc, kernelshape, pad=(0, 0), stride=(1, 1)):
     x_BKRC, f_LKrc = core.as_node(x_BKRC), core.as_node(f_LKrc)
     L, K, r, c = f_LKrc.shape
     assert tuple(kernelshape) == (r, c), "kernelshape must match the filter's last two axes"
+    _check_geometry(x_BKRC, K, tuple(kernelshape), tuple(pad), tuple(stride))
     if _CONV_ALGO == "auto" and conv_same.supported(x_BKRC, f_LKrc, kernelshape, pad, stride):
         return conv_same.conv_same(x_BKRC, f_LKrc, kernelshape)
     if _CONV_ALGO == "auto" and conv_col.patch_supported(x_BKRC, kernelshape, pad, stride):
@@ -111,6 +125,7 @@ class SpatialConvolution(object):
 
     def __call__(self, x):
         x = core.as_node(x)
+        _check_geometry(x, self.weight.shape[1], self.kernelshape, self.pad, self.stride)
         if (_CONV_FUSION and _CONV_ALGO == "auto"
                 and conv_same.supported(x, self.weight, self.kernelshape, self.pad, self.stride)):
             return conv_same.conv_same(x, self.weight, self.kernelshape, bias=self.bias)

@@ -201,6 +201,19 @@ def test_conv2d_grad_through_op_pullbacks(cgt, xshape, fshape, pad, stride):
     assert relfro(gx.get(), gx64) <= TOL and relfro(gf.get(), gf64) <= TOL
 
 
+def test_conv2d_rejects_a_kernel_larger_than_the_padded_image(cgt):
+    from cgt_amd import nn
+    x = cgt.constant(np.zeros((2, 3, 4, 9), np.float32))
+    f = cgt.constant(np.zeros((5, 3, 5, 5), np.float32))
+    with pytest.raises(ValueError, match="larger than"):
+        nn.conv2d(x, f, (5, 5))                       # 4 rows, no padding
+    assert nn.conv2d(x, f, (5, 5), pad=(1, 0)).shape == (2, 5, 2, 5)
+    with pytest.raises(ValueError, match="channels"):
+        nn.conv2d(x, cgt.constant(np.zeros((5, 4, 3, 3), np.float32)), (3, 3))
+    with pytest.raises(ValueError, match="larger than"):
+        nn.SpatialConvolution(3, 5, (5, 5), (0, 0))(x)
+
+
 def test_cifar_shaped_stack_forward_backward(cgt):
     # the CIFAR-shaped stack in miniature: conv 5x5 p2 -> pool 3x3/2 -> LRN(5,1e-4,.75) -> conv 5x5 p2,
     # loss = sum of outputs; gradients wrt input and both weights.  (The ReLU between

@@ -38,6 +38,18 @@ __device__ __forceinline__ LrnBlock lrn_block(int HW, int C, int crun) {
     return b;
 }
 
+// acc + v * v with the product rounded on its own, and k + acc * (alpha / n) as one fused
+// multiply-add: spelled out so that every kernel of this file forms a window sum and a scale
+// with the same roundings, whatever the compiler would otherwise share or fuse between
+// neighbouring windows (a kernel that unrolls the channel walk reuses the squares and adds
+// them; one that does not would fuse each product into its add).
+__device__ __forceinline__ float add_square(float acc, float v) {
+#pragma clang fp contract(off)
+    const float sq = v * v;
+    return acc + sq;
+}
+__device__ __forceinline__ float scale_of(float acc, float aos, float kconst) { return __builtin_fmaf(acc, aos, kconst); }
+
 __device__ __forceinline__ float pow_neg_beta(float s, float nbeta) {
     // s >= k > 0.  exp2(nbeta*log2(s)) on the hardware transcendental units:
     // relative error ~1e-6 for the scale range LRN produces.
@@ -89,8 +101,8 @@ __device__ __forceinline__ void lrn_fwd_run(const float* __restrict__ x, float* 
         for (int u = 0; u < U; ++u) {
             float acc = 0.0f;
 #pragma unroll
-            for (int j = 0; j < SIZE; ++j) acc += win[u + j] * win[u + j];
-            const float s = kconst + acc * aos;
+            for (int j = 0; j < SIZE; ++j) acc = add_square(acc, win[u + j]);
+            const float s = scale_of(acc, aos, kconst);
             if (c0 + u < ce) {
                 if (scale) sp[(c0 + u) * hs] = s;
                 const float t = win[u + PRE] * pow_neg_beta(s, nbeta);
@@ -155,9 +167,13 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_fwd_flat_kernel(
 #pragma unroll
         for (int j = 0; j < SIZE; ++j) {
             const v4f v = ok[j] ? w[j] : zero;
-            acc += v * v;
+            acc.x = add_square(acc.x, v.x);
+            acc.y = add_square(acc.y, v.y);
+            acc.z = add_square(acc.z, v.z);
+            acc.w = add_square(acc.w, v.w);
         }
-        const v4f s = kconst + acc * aos;
+        const v4f s = {scale_of(acc.x, aos, kconst), scale_of(acc.y, aos, kconst), scale_of(acc.z, aos, kconst),
+                       scale_of(acc.w, aos, kconst)};
         const v4f mid = w[PRE];
         if (scale) stream_store4(scale + f, s.x, s.y, s.z, s.w);
         stream_store4(top + f, mid.x * pow_neg_beta(s.x, nbeta), mid.y * pow_neg_beta(s.y, nbeta),
@@ -170,12 +186,10 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_fwd_flat_kernel(
         float acc = 0.0f;
         for (int j = 0; j < SIZE; ++j) {
             const int cc = c - PRE + j;
-            if (cc >= 0 && cc < C) {
-                const float v = x[(long)e + (long)(j - PRE) * HW];
-                acc += v * v;
-            }
+            const float v = (cc >= 0 && cc < C) ? x[(long)e + (long)(j - PRE) * HW] : 0.0f;
+            acc = add_square(acc, v);
         }
-        const float s = kconst + acc * aos;
+        const float s = scale_of(acc, aos, kconst);
         if (scale) scale[e] = s;
         top[e] = x[e] * pow_neg_beta(s, nbeta);
     }
@@ -195,11 +209,8 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_fwd_generic_kernel(
     for (int c = cs; c < ce; ++c) {
         float acc = 0.0f;
         const int lo = max(0, c - pre), hi = min(C - 1, c + post);
-        for (int cc = lo; cc <= hi; ++cc) {
-            const float v = x[base + (long)cc * HW];
-            acc += v * v;
-        }
-        const float s = kconst + acc * aos;
+        for (int cc = lo; cc <= hi; ++cc) acc = add_square(acc, x[base + (long)cc * HW]);
+        const float s = scale_of(acc, aos, kconst);
         if (scale) scale[base + (long)c * HW] = s;
         top[base + (long)c * HW] = x[base + (long)c * HW] * pow_neg_beta(s, nbeta);
     }
@@ -365,8 +376,8 @@ __device__ __forceinline__ void lrn_bwd_x_run(const float* __restrict__ x, const
         for (int j = 0; j < SIZE - 1; ++j) {
             float acc = 0.0f;
 #pragma unroll
-            for (int i = 0; i < SIZE; ++i) acc += xh[j + i] * xh[j + i];
-            const float sc = kconst + acc * aos;
+            for (int i = 0; i < SIZE; ++i) acc = add_square(acc, xh[j + i]);
+            const float sc = scale_of(acc, aos, kconst);
             const float pw = pow_neg_beta(sc, nbeta);
             const float xc = xh[j + FPRE];
             tr[j] = dh[j] * (xc * pw) / sc;
@@ -391,8 +402,8 @@ __device__ __forceinline__ void lrn_bwd_x_run(const float* __restrict__ x, const
         for (int u = 0; u < U; ++u) {
             float acc = 0.0f;
 #pragma unroll
-            for (int i = 0; i < SIZE; ++i) acc += xw[u + i] * xw[u + i];
-            const float sc = kconst + acc * aos;
+            for (int i = 0; i < SIZE; ++i) acc = add_square(acc, xw[u + i]);
+            const float sc = scale_of(acc, aos, kconst);
             const float pw = pow_neg_beta(sc, nbeta);
             const float xc = xw[u + FPRE];
             dr[POST + u] = dn[u];
@@ -444,11 +455,8 @@ __global__ __launch_bounds__(kLrnThreads) void lrn_bwd_x_generic_kernel(
     const long base = n * C * (long)HW + p;
     auto scale_at = [&](int ch) {
         float acc = 0.0f;
-        for (int cc = max(0, ch - fpre); cc <= min(C - 1, ch + fpost); ++cc) {
-            const float v = x[base + (long)cc * HW];
-            acc += v * v;
-        }
-        return kconst + acc * aos;
+        for (int cc = max(0, ch - fpre); cc <= min(C - 1, ch + fpost); ++cc) acc = add_square(acc, x[base + (long)cc * HW]);
+        return scale_of(acc, aos, kconst);
     };
     for (int c = cs; c < ce; ++c) {
         float acc = 0.0f;

@@ -628,6 +628,12 @@ def cpu_baseline(cfg, sample_batch):
     m = O.conv_outsize(x.shape[2], r, pad[0], stride[0])
     n = O.conv_outsize(x.shape[3], c, pad[1], stride[1])
     gy = np.ones((sample_batch, L, m, n), np.float32)
+    # the reference's own loops where they were compiled here (im2col_cpu / col2im_cpu with this
+    # geometry as template constants, pooling.h), the oracle's restatement elsewhere
+    conv_kind = CB.conv_impl((r, c), pad, stride)[1]
+    P, pool_kind = CB.pool_impl()
+    from_reference = ([s for s in ("im2col", "col2im") if conv_kind == "reference"] +
+                      [s for s in ("max_pool_fwd", "max_pool_bwd") if pool_kind == "reference" and cfg["pool"]])
 
     def run():
         y, gx, gf = CB.conv2d_fwd_bwd(x, f, gy, pad, stride)
@@ -637,8 +643,8 @@ def cpu_baseline(cfg, sample_batch):
             act, scale = O.lrn_fwd(y, size, alpha, beta, k)
         if cfg["pool"]:
             pk, pp, ps = cfg["pool"]
-            pool, mask = O.max_pool(act, pk, pp, ps)
-            g = O.max_pool_pullback(act.shape, mask, np.ones_like(pool))
+            pool, mask = P.max_pool(act, pk, pp, ps)
+            g = P.max_pool_pullback(act.shape, mask, np.ones_like(pool))
             if cfg["lrn"]:
                 O.lrn_bwd(y, act, scale, g, size, alpha, beta)
 
@@ -650,11 +656,18 @@ def cpu_baseline(cfg, sample_batch):
         if name.startswith("gemm"):
             per_stage[name] = {"ms": round(sec * 1e3, 3), "TFLOPs": round(work / sec / 1e12, 4)}
         else:
-            per_stage[name] = {"ms": round(sec * 1e3, 3), "GBps": round(work / sec / 1e9, 3)}
+            per_stage[name] = {"ms": round(sec * 1e3, 3), "GBps": round(work / sec / 1e9, 3),
+                               "impl": "reference" if name in from_reference else "port"}
+    # "port": not every stage is the reference's own code (its GEMM library is a build-time download,
+    # its transpose generated C, its LRN CUDA only); `reference_stages` names the ones that are
     return {"value": flops / best / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port", "stages": per_stage,
-            "sample": "%d of %d images of the workload, best of %d passes (%.2f s each); im2col/col2im/"
-                      "transpose/pool/LRN single-threaded C, GEMM %s with %d threads; host %s, %d cores usable"
-                      % (sample_batch, cfg["x"][0], reps, best, CB.blas_config(), threads, CB.cpu_model(), CB.host_cores())}
+            "reference_stages": from_reference,
+            "sample": "%d of %d images of the workload, best of %d passes (%.2f s each); single-threaded C: %s the "
+                      "reference's own loops compiled -O3 (geometry as template constants), transposes/LRN%s the "
+                      "oracle's restatement; GEMM %s with %d threads; host %s, %d cores usable"
+                      % (sample_batch, cfg["x"][0], reps, best, "/".join(from_reference) if from_reference else "none of them",
+                         "" if from_reference else "/im2col/col2im/pool",
+                         CB.blas_config(), threads, CB.cpu_model(), CB.host_cores())}
 
 
 def cpu_gemm_baseline(n=2048):

@@ -5,8 +5,11 @@ cblas_sgemm -> Transpose, with pooling.h for pooling; its OpenBLAS 0.2.14 is
 fetched at build time and is not in the reference tree, so scipy's bundled
 OpenBLAS stands in for it, called row-major with the reference's argument
 mapping (cgt/core.py:2196-2205) and at most 16 threads (CMakeLists.txt:51).
-The single-threaded stages are the oracle's (oracle/cgt_oracle.c).  Only
-bench.py's cpu_baseline leg uses this module.
+The single-threaded stages are the reference's own loops where they exist as
+C++ and were compiled here (oracle/_ref/libcgt_ref.so: im2col_cpu / col2im_cpu
+with the geometry as template constants, max_pool / max_pool_pullback), else
+the oracle's (oracle/cgt_oracle.c: transposes, LRN, geometries that were not
+instantiated).  Only bench.py's cpu_baseline leg uses this module.
 """
 import ctypes
 import glob
@@ -16,8 +19,20 @@ import time
 import numpy as np
 
 from . import oracle as O
+from . import ref as R
 
 _BLAS = None
+
+
+def conv_impl(kernel, pad, stride):
+    """(module with im2col / col2im, "reference" | "port") for a geometry."""
+    if R.available() and tuple(kernel) + tuple(pad) + tuple(stride) in R.GEOMS:
+        return R, "reference"
+    return O, "port"
+
+
+def pool_impl():
+    return (R, "reference") if R.available() else (O, "port")
 
 
 def blas():
@@ -77,13 +92,14 @@ def sgemm(A, B, tA=False, tB=False):
 def conv2d_fwd_bwd(x, f, gy, pad, stride):
     """conv2d forward + both gradients the way the reference's CPU graph runs them."""
     L, K, r, c = f.shape
-    col = O.im2col(x, (r, c), pad, stride)
+    I, _ = conv_impl((r, c), pad, stride)
+    col = I.im2col(x, (r, c), pad, stride)
     B, m, n, Z = col.shape
     f_LZ = f.reshape(L, Z)
     y = O.transpose4(sgemm(col.reshape(B * m * n, Z), f_LZ, False, True).reshape(B, m, n, L), (0, 3, 1, 2))
     gc = O.transpose4(gy, (0, 2, 3, 1)).reshape(B * m * n, L)
     gcol = sgemm(gc, f_LZ, False, False)
-    gx = O.col2im(gcol.reshape(B, m, n, Z), x.shape, (r, c), pad, stride)
+    gx = I.col2im(gcol.reshape(B, m, n, Z), x.shape, (r, c), pad, stride)
     gf = sgemm(gc, col.reshape(B * m * n, Z), True, False).reshape(f.shape)
     return y, gx, gf
 
@@ -106,12 +122,14 @@ def stage_times(x, f, gy, pad, stride, pool=None, lrn=None, min_seconds=0.5):
     order the reference's graph runs them: {stage: (seconds, bytes or flops)}."""
     L, K, r, c = f.shape
     out = {}
-    col = O.im2col(x, (r, c), pad, stride)
+    I, _ = conv_impl((r, c), pad, stride)
+    P, _ = pool_impl()
+    col = I.im2col(x, (r, c), pad, stride)
     B, m, n, Z = col.shape
     col2, f_LZ = col.reshape(B * m * n, Z), f.reshape(L, Z)
     io = 4 * (x.size + col.size)
     flops = 2 * B * m * n * L * Z
-    out["im2col"] = (timed(lambda: O.im2col(x, (r, c), pad, stride), min_seconds, 5)[0], io)
+    out["im2col"] = (timed(lambda: I.im2col(x, (r, c), pad, stride), min_seconds, 5)[0], io)
     out["gemm_fwd_NT"] = (timed(lambda: sgemm(col2, f_LZ, False, True), min_seconds, 5)[0], flops)
     y2 = sgemm(col2, f_LZ, False, True).reshape(B, m, n, L)
     out["transpose_0312"] = (timed(lambda: O.transpose4(y2, (0, 3, 1, 2)), min_seconds, 5)[0], 8 * y2.size)
@@ -124,19 +142,19 @@ def stage_times(x, f, gy, pad, stride, pool=None, lrn=None, min_seconds=0.5):
     g = gy
     if pool:
         pk, pp, ps = pool
-        out["max_pool_fwd"] = (timed(lambda: O.max_pool(act, pk, pp, ps), min_seconds, 5)[0], None)
-        pooled, mask = O.max_pool(act, pk, pp, ps)
+        out["max_pool_fwd"] = (timed(lambda: P.max_pool(act, pk, pp, ps), min_seconds, 5)[0], None)
+        pooled, mask = P.max_pool(act, pk, pp, ps)
         out["max_pool_fwd"] = (out["max_pool_fwd"][0], 4 * (act.size + 2 * pooled.size))
         gp = np.ones_like(pooled)
-        out["max_pool_bwd"] = (timed(lambda: O.max_pool_pullback(act.shape, mask, gp), min_seconds, 5)[0],
+        out["max_pool_bwd"] = (timed(lambda: P.max_pool_pullback(act.shape, mask, gp), min_seconds, 5)[0],
                                4 * (2 * pooled.size + act.size))
-        g = O.max_pool_pullback(act.shape, mask, gp)
+        g = P.max_pool_pullback(act.shape, mask, gp)
     if lrn:
         out["lrn_bwd"] = (timed(lambda: O.lrn_bwd(y, act, scale, g, size, alpha, beta), min_seconds, 5)[0], 20 * y.size)
     out["transpose_0231"] = (timed(lambda: O.transpose4(g, (0, 2, 3, 1)), min_seconds, 5)[0], 8 * y.size)
     gc = O.transpose4(g, (0, 2, 3, 1)).reshape(B * m * n, L)
     out["gemm_dgrad_NN"] = (timed(lambda: sgemm(gc, f_LZ, False, False), min_seconds, 5)[0], flops)
     gcol = sgemm(gc, f_LZ, False, False).reshape(B, m, n, Z)
-    out["col2im"] = (timed(lambda: O.col2im(gcol, x.shape, (r, c), pad, stride), min_seconds, 5)[0], io)
+    out["col2im"] = (timed(lambda: I.col2im(gcol, x.shape, (r, c), pad, stride), min_seconds, 5)[0], io)
     out["gemm_wgrad_TN"] = (timed(lambda: sgemm(gc, col2, True, False), min_seconds, 5)[0], flops)
     return out

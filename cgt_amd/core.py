@@ -752,11 +752,16 @@ class BatchedMul22(Op):
 
 
 class Transpose(Op):
-    """Axis permutation of a 4-d array (reference core.py:1559-1594, cpu-only there)."""
+    """Axis permutation of an array of up to four axes (reference core.py:1559-1594, cpu-only and of
+    any rank there; the conv path transposes 4-d arrays, fewer axes ride along as leading extents of 1)."""
     available_impls = ("native_gpu",)
 
     def __init__(self, axes):
         self.axes = tuple(int(a) for a in axes)
+        if sorted(self.axes) != list(range(len(self.axes))):
+            raise ValueError("Transpose: %s is not a permutation of the axes" % (self.axes,))
+        if len(self.axes) > 4:
+            raise NotImplementedError("Transpose: arrays of more than four axes are not supported on the device")
 
     def get_diff(self, _):
         return [True]
@@ -778,13 +783,25 @@ class Transpose(Op):
         return "Transpose{%s}" % ",".join(map(str, self.axes))
 
     def get_native_compile_info(self, input_types, devtype):
-        assert devtype == "gpu" and input_types[0].ndim == 4 and input_types[0].dtype == "f4"
-        triples = [("a%d" % i, ctypes.c_int, a) for i, a in enumerate(self.axes)]
+        assert devtype == "gpu" and input_types[0].dtype == "f4"
+        if input_types[0].ndim != len(self.axes):
+            raise ValueError("Transpose%s applied to an array of %d axes" % (self.axes, input_types[0].ndim))
+        triples = [("a%d" % i, ctypes.c_int, a) for i, a in enumerate(self.axes + (0,) * (4 - len(self.axes)))]
+        triples.append(("nd", ctypes.c_int, len(self.axes)))
         code = r"""
             CGT_EXPORT_C void $function($closure* cl, cgtArray** reads, cgtArray* write) {
                 cgtArray* in = reads[0];
-                int axes[4] = {cl->a0, cl->a1, cl->a2, cl->a3};
-                int rc = cgt_amd_transpose4_f32((const float*)in->data(), in->shape(), axes,
+                const int given[4] = {cl->a0, cl->a1, cl->a2, cl->a3};
+                const int nd = cl->nd, lead = 4 - nd;
+                cgt_check(in->ndim() == nd && write->size() == in->size(), "Transpose: operand rank or size does not fit");
+                if (cgtGlobalStatus != cgtStatusOK) return;
+                long shape4[4];
+                int axes4[4];
+                for (int i = 0; i < 4; ++i) {       // fewer than four axes: leading extents of 1 that stay in place
+                    shape4[i] = i < lead ? 1 : in->shape()[i - lead];
+                    axes4[i] = i < lead ? i : given[i - lead] + lead;
+                }
+                int rc = cgt_amd_transpose4_f32((const float*)in->data(), shape4, axes4,
                     (float*)write->data(), cgt_get_stream());
                 cgt_check(rc == CGT_AMD_OK, "Transpose: %s", cgt_amd_last_error());
             }"""

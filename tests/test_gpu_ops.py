@@ -201,6 +201,28 @@ def test_conv2d_grad_through_op_pullbacks(cgt, xshape, fshape, pad, stride):
     assert relfro(gx.get(), gx64) <= TOL and relfro(gf.get(), gf64) <= TOL
 
 
+@pytest.mark.parametrize("shape,axes", [((5, 7), (1, 0)), ((3, 4, 5), (2, 0, 1)), ((3, 4, 5), (0, 2, 1)), ((6,), (0,)),
+                                        ((2, 3, 4, 5), (3, 1, 0, 2)), ((1, 9), (1, 0))])
+def test_transpose_of_fewer_than_four_axes(cgt, shape, axes):
+    # the reference's Transpose takes any rank (cgt/core.py:1559-1594); the device kernel is 4-d, fewer axes
+    # ride along as leading extents of 1.  Values, gradient, and a compiled replay at another leading extent
+    rs = np.random.RandomState(len(shape))
+    xv = rs.randn(*shape).astype(np.float32)
+    x = cgt.constant(xv)
+    y = cgt.transpose(x, axes)
+    assert np.array_equal(y.get(), xv.transpose(axes))
+    g = rs.randn(*y.shape).astype(np.float32)
+    gx, = cgt.grad(y, [x], goutput=g)
+    assert np.array_equal(gx.get(), g.transpose(np.argsort(axes)))
+    f = cgt.function([x], y)
+    x2 = rs.randn(*((shape[0] + 2,) + shape[1:])).astype(np.float32)
+    assert np.array_equal(f(x2), x2.transpose(axes))
+    with pytest.raises(ValueError):
+        cgt.transpose(x, (axes[0],) * len(axes) if len(axes) > 1 else (1,))        # not a permutation
+    with pytest.raises(NotImplementedError):
+        cgt.Transpose((0, 1, 2, 3, 4))
+
+
 def test_conv2d_rejects_a_kernel_larger_than_the_padded_image(cgt):
     from cgt_amd import nn
     x = cgt.constant(np.zeros((2, 3, 4, 9), np.float32))

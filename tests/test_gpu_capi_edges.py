@@ -150,6 +150,12 @@ def test_gemm_whole_tiles_with_ragged_k(L, M, N, K, tA, tB):
     (lambda L, p: L.cgt_amd_lrn_fwd_f32(p, 1, 3, 4, 4, 5, 1e-4, 0.75, 1.0, p, p, None), "size"),
     (lambda L, p: L.cgt_amd_lrn_fwd_f32(p, 1, 8, 4, 4, 5, 1e-4, 0.75, 0.0, p, p, None), "k must be positive"),
     (lambda L, p: L.cgt_amd_lrn_bwd_f32(p, p, p, p, 1, 8, 4, 4, 0, 1e-4, 0.75, p, None), "size"),
+    (lambda L, p: L.cgt_amd_lrn_fwd_f32(p, 1, 8, 4, 4, 5, 1e-4, 0.75, 1.0, None, None, None), "null"),     # top may not be null (scale may)
+    (lambda L, p: L.cgt_amd_lrn_bwd_from_x_f32(p, p, 1, 8, 4, 4, 5, 1e-4, 0.75, 0.0, p, None), "k must be positive"),
+    (lambda L, p: L.cgt_amd_lrn_bwd_from_x_f32(p, None, 1, 8, 4, 4, 5, 1e-4, 0.75, 1.0, p, None), "null"),
+    (lambda L, p: L.cgt_amd_lrn_bwd_from_x_f32(p, p, 1, 3, 4, 4, 5, 1e-4, 0.75, 1.0, p, None), "size"),
+    (lambda L, p: L.cgt_amd_lrn_bwd_recompute_f32(p, None, p, 1, 8, 4, 4, 5, 1e-4, 0.75, p, None), "null"),
+    (lambda L, p: L.cgt_amd_conv_same_pad_pool_pullback_f32(p, p, None, 2, 4, 4, 2, 2, 0, 0, 2, 2, 2, 2, 4, 4, p, None), "odd"),
     (lambda L, p: L.cgt_amd_sgemm(0, 0, 4, 4, 4, p, 3, p, 4, p, 4, None), "leading dimension"),
     (lambda L, p: L.cgt_amd_sgemm(0, 0, 4, 4, 4, p, 4, p, 4, None, 4, None), "null"),
     (lambda L, p: L.cgt_amd_sgemm(0, 0, -1, 4, 4, p, 4, p, 4, p, 4, None), "negative"),

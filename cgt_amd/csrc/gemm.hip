@@ -1233,6 +1233,7 @@ static void launch_gather(int which, int shape, dim3 grid, hipStream_t st, const
             case 0: sgemm_kernel<true, false, false, 2, 2, 2, 2, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;
             case 2: sgemm_kernel<true, false, false, 4, 1, 1, 2, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;    // 128 x 64
             case 4: sgemm_kernel<true, false, false, 1, 4, 3, 1, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;    // 96 x 128
+            case 6: sgemm_kernel<true, false, false, 1, 4, 1, 1, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;    // 32 x 128
             default: sgemm_kernel<true, false, false, 1, 4, 2, 1, false, 0, 2, GPAD><<<grid, block, 0, st>>>(a); break;   // 64 x 128
         }
     }
@@ -1307,7 +1308,7 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     int shape = 0;
     double best = 0;
     const bool gather_cols = cv && cv->mode == 4 && cv->patch;     // the gathered weight gradient: tiles of 128 or 64 columns
-    for (int i = 0; i < kPlainShapes; ++i) {
+    for (int i = 0; i < kPlainShapes + (gather_cols ? 1 : 0); ++i) {        // 32 x 128: the gathered weight gradient of 32 or fewer filters
         if (gather_cols && kShapes[i].bn != 128 && kShapes[i].bn != 64) continue;
         const double work = (double)(cdiv(M, kShapes[i].bm) * kShapes[i].bm) *
                             (double)(cdiv(N, kShapes[i].bn) * kShapes[i].bn);

@@ -336,9 +336,11 @@ class Function(object):
         plan = self._plan
         if self.use_graph:
             from .gpuarray import to_gpu
-            vals = [to_gpu(v) if on_gpu and not isinstance(v, GpuArray) else v
-                    for v, (_s, _d, on_gpu) in zip(vals, self._arg_specs)]
+            uploaded = [on_gpu and not isinstance(v, GpuArray) for v, (_s, _d, on_gpu) in zip(vals, self._arg_specs)]
+            vals = [to_gpu(v) if up else v for v, up in zip(vals, uploaded)]
             self._run_graph(vals)
+            if any(uploaded):       # the staging copies read temporaries that die with this call
+                self._stream.synchronize()
         else:
             plan.it.run(vals)
         outs = [plan.it.get_array(s) for s in plan.out_slots]
@@ -358,8 +360,8 @@ class Function(object):
             if s is None:
                 staged.append(v)              # host operand (shape integers): read at capture time
             else:
-                if v.ptr != s.ptr:
-                    capi.check(capi.lib().cgt_amd_memcpy(capi.GPU, capi.GPU, s.ptr, v.ptr, s.nbytes))
+                if v.ptr != s.ptr:      # on the graph's own stream: ordered before the replay, no host wait
+                    capi.check(capi.lib().cgt_amd_memcpy_async(capi.GPU, capi.GPU, s.ptr, v.ptr, s.nbytes, self._stream.handle))
                 staged.append(s)
         rt.set_stream(self._stream.handle)
         try:

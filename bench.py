@@ -139,9 +139,10 @@ def traffic_from_profiles(workload, algo=None, stage_names=("gemm_fwd_NT", "gemm
         for name, mb in rows:
             if "sgemm_kernel" in name:
                 stage = next(order, None)
-            elif "reduce_kernel" not in name:
+            elif "reduce_" not in name:
                 stage = None if stage is None else "-"     # another kernel: later reduce rows are not this GEMM's
-            if stage not in (None, "-") and ("sgemm_kernel" in name or "reduce_kernel" in name):
+            # splitk_reduce_kernel, tail_reduce_kernel, tail_reduce_conv_kernel: the partials' second pass
+            if stage not in (None, "-") and ("sgemm_kernel" in name or "reduce_" in name):
                 total[stage] = total.get(stage, 0.0) + scale * mb * 1e6
     return {k: int(round(v)) for k, v in total.items()}
 
@@ -174,7 +175,10 @@ class Stage(object):
 class LayerOnGpu(object):
     """One configured layer with every buffer pre-allocated on the device."""
 
-    def __init__(self, cfg, overlap=False, glue=False, algo="auto"):
+    def __init__(self, cfg, overlap=False, glue=False, algo="auto", batch=None, seed=0, cotangent="ones"):
+        """batch / seed: another batch size and input stream than the configured ones (the parity
+        gate runs the very stage list that is timed on a 2-image slice); cotangent "ones" is the
+        configured loss (sum of outputs), "random" a seeded N(0,1) one for the gate."""
         from cgt_amd import capi, kernels as K
         from cgt_amd.gpuarray import empty, to_gpu
         # two streams (default priority): the weight-gradient GEMM depends only on
@@ -186,7 +190,10 @@ class LayerOnGpu(object):
         stream = self._main.handle
         self._wgrad_stream = stream
         self.cfg, self.K, self.stream = cfg, K, stream
-        x, f = make_inputs(cfg)
+        x, f = make_inputs(cfg, batch, seed)
+        cot_rs = np.random.RandomState(seed + 1000)
+        self._cot = (lambda shape: np.ones(shape, np.float32)) if cotangent == "ones" else \
+                    (lambda shape: cot_rs.randn(*shape).astype(np.float32))
         B, C, H, W = x.shape
         L, _, r, c = f.shape
         pad, stride = cfg["pad"], cfg["stride"]
@@ -257,7 +264,7 @@ class LayerOnGpu(object):
             pk, pp, ps = cfg["pool"]
             PH, PW = K.pool_outsize(m, pk[0], pp[0], ps[0]), K.pool_outsize(n, pk[1], pp[1], ps[1])
             self.pool, self.mask = empty((B, L, PH, PW)), empty((B, L, PH, PW), np.int32)
-            self.gpool = to_gpu(np.ones((B, L, PH, PW), np.float32))
+            self.gpool = to_gpu(self._cot((B, L, PH, PW)))
             self.gact = empty(self.y.shape)
             pool_in = act
             st.append(Stage("max_pool_fwd", "max_pool_fwd_kernel", lambda: K.max_pool(pool_in, pk, pp, ps, out=(self.pool, self.mask), stream=s),
@@ -267,7 +274,7 @@ class LayerOnGpu(object):
                             4 * (2 * nelem(self.pool) + nelem(self.y)), "hbm"))
             gy = self.gact
         else:
-            gy = to_gpu(np.ones(self.y.shape, np.float32))   # loss = sum of outputs
+            gy = to_gpu(self._cot(self.y.shape))   # "ones": loss = sum of outputs
         if cfg["lrn"]:
             self.gy_lrn = empty(self.y.shape)
             g_in = gy
@@ -370,7 +377,7 @@ class LayerOnGpu(object):
             pk, pp, ps = cfg["pool"]
             PH, PW = K.pool_outsize(H, pk[0], pp[0], ps[0]), K.pool_outsize(W, pk[1], pp[1], ps[1])
             self.pool, self.mask = empty((B, L, PH, PW)), empty((B, L, PH, PW), np.int32)
-            self.gpool = to_gpu(np.ones((B, L, PH, PW), np.float32))
+            self.gpool = to_gpu(self._cot((B, L, PH, PW)))
             st.append(Stage("max_pool_fwd", "max_pool_fwd_kernel", lambda: K.max_pool(act, pk, pp, ps, out=(self.pool, self.mask), stream=s),
                             4 * (nelem(self.y) + 2 * nelem(self.pool)), "hbm"))
             # the pool's pullback writes the padded cotangent itself (what the Op graph builds:
@@ -380,7 +387,7 @@ class LayerOnGpu(object):
                                                                   out=self.gypad, stream=s),
                             4 * (2 * nelem(self.pool) + nelem(self.gypad)), "hbm"))
         else:
-            self.gy = to_gpu(np.ones(self.y.shape, np.float32))
+            self.gy = to_gpu(self._cot(self.y.shape))
             st.append(Stage("pad_gy", "pad_planes_kernel", lambda: K.conv_same_pad(self.gy, (r, c), out=self.gypad, stream=s),
                             4 * (nelem(self.y) + nelem(self.gypad)), "hbm"))
         st.append(Stage("filter_flip", "flip_filters_kernel",
@@ -518,10 +525,12 @@ class GemmOnGpu(object):
 
 def hbm_reference(reps=10):
     """What plain streaming kernels of this library reach on this box, measured in the same
-    run on arrays (1 GiB each) far larger than the 256 MB last-level cache: a device-to-device
-    copy, a pure write (fill), a pure read (sum) and an elementwise add (two reads, one
-    write).  The HBM-bound stages are priced against the published 8 TB/s; these rows say
-    how much of that a kernel with no index arithmetic at all gets here."""
+    run on arrays (1 GiB each) far larger than the 256 MB last-level cache: the library's
+    device-to-device copy kernel (workgroup-contiguous regions, 8 x 16-byte loads in flight
+    per lane, non-temporal stores), the runtime's own memcpy beside it, a pure write (fill),
+    a pure read (sum) and an elementwise add (two reads, one write).  The HBM-bound stages are
+    priced against the published 8 TB/s; these rows say how much of that a kernel with no
+    index arithmetic at all gets here."""
     from cgt_amd import capi, kernels as K
     from cgt_amd.gpuarray import empty
     n = 1 << 28
@@ -546,7 +555,9 @@ def hbm_reference(reps=10):
         rows[name] = {"ms": round(ms, 4), "bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1),
                       "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
 
-    timed("copy_1GiB", lambda: capi.check(lib.cgt_amd_memcpy_async(capi.GPU, capi.GPU, c.ptr, a.ptr, 4 * n, st)), 8 * n)
+    timed("copy_kernel_1GiB", lambda: capi.check(lib.cgt_amd_stream_copy(c.ptr, a.ptr, 4 * n, st)), 8 * n)
+    # overlapping ranges keep the runtime's copy (memmove semantics): this row is hipMemcpyAsync itself
+    timed("runtime_memcpy_1GiB", lambda: capi.check(lib.cgt_amd_memcpy_async(capi.GPU, capi.GPU, a.ptr + 4096, a.ptr, 4 * n - 4096, st)), 8 * n)
     timed("write_fill_1GiB", lambda: K.fill(3.0, (n,), out=c, stream=st), 4 * n)
     timed("read_sum_1GiB", lambda: K.sum_keepdims(a, (0,), out=small, stream=st), 4 * n)
     timed("add_2r1w_1GiB", lambda: K.elwise_binary("+", a, b, out=c, stream=st), 12 * n)
@@ -554,38 +565,105 @@ def hbm_reference(reps=10):
     return rows
 
 
-def check_gemm_against_oracle():
-    from cgt_amd import kernels as K
-    from cgt_amd.gpuarray import to_gpu
-    rs = np.random.RandomState(1)
-    A = rs.uniform(-1, 1, (300, 1000)).astype(np.float32)
-    B = rs.uniform(-1, 1, (200, 1000)).astype(np.float32)
-    C = K.mul22(to_gpu(A), to_gpu(B), False, True).get()
-    ref = A.astype(np.float64) @ B.astype(np.float64).T
-    err = float(np.linalg.norm(C - ref) / np.linalg.norm(ref))
-    return {"mul22_rel_fro": err, "ok": bool(err <= 1e-4)}
+def _relfro(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-300))
 
 
-def check_against_oracle(cfg):
-    """Parity gate run with every measurement, on a 2-image slice of the workload."""
-    from cgt_amd import kernels as K
-    from cgt_amd.gpuarray import to_gpu
+def _same_bits(a, b):
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    return bool(a.shape == b.shape and a.dtype == b.dtype and np.array_equal(a.view(np.uint32), b.view(np.uint32)))
+
+
+TOL = 1e-4      # relative Frobenius error allowed for GEMM, conv and LRN results (north_star)
+
+
+def check_gemm_against_oracle(layer, rows=24):
+    """Parity gate of the raw products, on the operands and launches that are timed: after one
+    step every variant's result is compared, on `rows` sampled rows (and 2 sampled batches),
+    with the oracle's product in float64 (reference argument mapping, cgt/core.py:2196-2205,
+    2272-2285)."""
+    from cgt_amd import capi
     from oracle import oracle as O
-    x, f = make_inputs(cfg, batch=2, seed=1)
-    pad, stride = cfg["pad"], cfg["stride"]
+    A, B = layer.A.get().astype(np.float64), layer.B.get().astype(np.float64)
+    rs = np.random.RandomState(5)
+    pick = np.sort(rs.choice(A.shape[0], rows, replace=False))
+    worst = 0.0
+    for st, (tA, tB) in zip(layer.stages[:4], [(False, False), (False, True), (True, False), (True, True)]):
+        st.fn()
+        capi.synchronize()
+        got = layer.C.get()[pick]
+        Asub = np.ascontiguousarray(A[:, pick] if tA else A[pick])
+        worst = max(worst, _relfro(got, O.mul22(Asub, B, tA, tB)))
+    layer.stages[4].fn()
+    capi.synchronize()
+    bA, bB, bC = layer.bA.get().astype(np.float64), layer.bB.get().astype(np.float64), layer.bC.get()
+    for p in (0, bA.shape[0] - 1):
+        worst = max(worst, _relfro(bC[p], O.batched_mul22(bA[p:p + 1], bB[p:p + 1])[0]))
+    return {"mul22_x4_batched_rel_fro": worst, "ok": bool(worst <= TOL)}
+
+
+def check_layer_against_oracle(cfg, algo):
+    """Parity gate run with every measurement: the stage list that is timed (same algorithm,
+    same entry points, same geometry) runs once on a 2-image slice with a random cotangent, and
+    every stage's output is compared with the oracle applied to that stage's inputs.  Bit-exact:
+    im2col, col2im, padding, pool values, int32 mask, pool pullback (also where it is written
+    into the padded layout).  Relative Frobenius <= 1e-4 against float64: conv output, LRN
+    top / scale / gradient, data gradient, weight gradient.  Reference: cgt/nn.py:87-111,
+    include/im2col.h:6-50, include/pooling.h:24-106, include/lrn.cuh:3-114."""
+    from cgt_amd import capi
+    from oracle import oracle as O
+    layer = LayerOnGpu(cfg, algo=algo, batch=2, seed=1, cotangent="random")
+    layer.step()
+    capi.synchronize()
+    d = np.float64
+    pad, stride = tuple(cfg["pad"]), tuple(cfg["stride"])
+    x, f = layer.x.get(), layer.f.get()
     r, c = f.shape[2:]
-    col = K.im2col(to_gpu(x), (r, c), pad, stride)
-    ocol = O.im2col(x, (r, c), pad, stride)
-    ok = np.array_equal(col.get().view(np.uint32), ocol.view(np.uint32))
-    y = K.conv2d(to_gpu(x), to_gpu(f), pad, stride).get()
-    y64 = O.conv2d(x.astype(np.float64), f.astype(np.float64), pad, stride)
-    err = float(np.linalg.norm(y - y64) / np.linalg.norm(y64))
-    y = K.conv_col_fwd(col, to_gpu(f)).get()        # the fused product over the same column buffer
-    err = max(err, float(np.linalg.norm(y - y64) / np.linalg.norm(y64)))
-    if K.conv_patch_supported(x.shape, (r, c), pad, stride):      # and with the patches gathered from x
-        y = K.conv_patch_fwd(to_gpu(x), to_gpu(f), pad, stride).get()
-        err = max(err, float(np.linalg.norm(y - y64) / np.linalg.norm(y64)))
-    return {"im2col_bit_exact": bool(ok), "conv2d_rel_fro": err, "ok": bool(ok and err <= 1e-4)}
+    exact, err = {}, {}
+    y = layer.y.get()
+    err["conv_fwd"] = _relfro(y, O.conv2d(x.astype(d), f.astype(d), pad, stride))
+    if layer.algo == "direct":
+        exact["pad"] = _same_bits(layer.xpad.get(), O.conv_same_padded(x, (r, c), layer.xpad.size))
+    elif getattr(layer, "col", None) is not None:
+        exact["im2col"] = _same_bits(layer.col.get(), O.im2col(x, (r, c), pad, stride))
+    act = y
+    if cfg["lrn"]:
+        size, alpha, beta, k = cfg["lrn"]
+        top64, scale64 = O.lrn_fwd(y.astype(d), size, alpha, beta, k)
+        act = layer.top.get()
+        err["lrn_fwd"] = _relfro(act, top64)
+        if getattr(layer, "scale", None) is not None:
+            err["lrn_fwd"] = max(err["lrn_fwd"], _relfro(layer.scale.get(), scale64))
+    if cfg["pool"]:
+        pk, pp, ps = cfg["pool"]
+        opool, omask = O.max_pool(act, pk, pp, ps)
+        mask = layer.mask.get()
+        exact["pool_values"] = _same_bits(layer.pool.get(), opool)
+        exact["pool_mask"] = _same_bits(mask, omask)
+        g = O.max_pool_pullback(act.shape, mask, layer.gpool.get())
+        if layer.algo == "direct":      # written straight into the padded cotangent
+            exact["pool_bwd_padded"] = _same_bits(layer.gypad.get(), O.conv_same_padded(g, (r, c), layer.gypad.size))
+        else:
+            exact["pool_bwd"] = _same_bits(layer.gact.get(), g)
+    else:
+        g = layer.gy.get()
+        if layer.algo == "direct":
+            exact["pad_gy"] = _same_bits(layer.gypad.get(), O.conv_same_padded(g, (r, c), layer.gypad.size))
+    if cfg["lrn"]:
+        got = layer.gy_lrn.get()
+        err["lrn_bwd"] = _relfro(got, O.lrn_bwd(y.astype(d), top64, scale64, g.astype(d), size, alpha, beta))
+        g = got
+    gx64, gf64 = O.conv2d_pullback(x.astype(d), f.astype(d), g.astype(d), pad, stride)
+    err["conv_dgrad"] = _relfro(layer.gx.get(), gx64)
+    err["conv_wgrad"] = _relfro(layer.gf.get().reshape(f.shape), gf64)
+    if getattr(layer, "gcol", None) is not None:
+        B, C, H, W = x.shape
+        gcol = layer.gcol.get().reshape(B, layer.dims["m"], layer.dims["n"], layer.dims["Z"])
+        exact["col2im"] = _same_bits(layer.gx.get(), O.col2im(gcol, x.shape, (r, c), pad, stride))
+    ok = all(exact.values()) and all(v <= TOL for v in err.values())
+    return {"ok": bool(ok), "algo": layer.algo, "images": 2, "bit_exact": exact,
+            "rel_fro": {k: float("%.2e" % v) for k, v in err.items()}}
 
 
 def op_api_step_ms(cfg, steps, warmup):
@@ -662,6 +740,9 @@ def cpu_baseline(cfg, sample_batch):
     # its transpose generated C, its LRN CUDA only); `reference_stages` names the ones that are
     return {"value": flops / best / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port", "stages": per_stage,
             "reference_stages": from_reference,
+            "sample_short": "%d of %d images, best of %d passes (%.2f s each); 1-thread C loops (%s: the reference's own, -O3), "
+                            "GEMM %s x%d threads; %s" % (sample_batch, cfg["x"][0], reps, best, "/".join(from_reference) or "none",
+                                                         " ".join(CB.blas_config().split()[:2]), threads, CB.cpu_model()),
             "sample": "%d of %d images of the workload, best of %d passes (%.2f s each); single-threaded C: %s the "
                       "reference's own loops compiled -O3 (geometry as template constants), transposes/LRN%s the "
                       "oracle's restatement; GEMM %s with %d threads; host %s, %d cores usable"
@@ -690,13 +771,13 @@ def measure(workload, args, primary):
     if is_gemm:
         cfg = {"x": [4096, 4096], "f": [4096, 4096], "pad": [], "stride": []}
         layer = GemmOnGpu()
-        parity = {"ok": True, "skipped": True} if args.no_check else check_gemm_against_oracle()
+        parity = {"ok": True, "skipped": True} if args.no_check else check_gemm_against_oracle(layer)
     else:
         base, forced = split_workload(workload)
         cfg = WORKLOADS[base]
         layer = LayerOnGpu(cfg, overlap=primary and args.overlap and not args.no_overlap, glue=primary and args.glue,
                            algo=forced or args.conv_algo)
-        parity = {"ok": True, "skipped": True} if args.no_check else check_against_oracle(cfg)
+        parity = {"ok": True, "skipped": True} if args.no_check else check_layer_against_oracle(cfg, forced or args.conv_algo)
 
     for _ in range(args.warmup):
         layer.step()
@@ -768,8 +849,8 @@ def measure(workload, args, primary):
     traffic = traffic_from_profiles(workload, algo, mfma_stages).get(dominant.name)
     config = {"workload": workload, "x": list(cfg["x"]), "filters": list(cfg["f"]),
               "pad": list(cfg["pad"]), "stride": list(cfg["stride"]),
-              "value_is": "conv GEMM flops (6*B*m*n*L*Z) / whole step time incl. im2col, col2im, "
-                          "transposes, pool and LRN stages",
+              "value_is": "conv GEMM flops 6*B*m*n*L*Z / whole step time, every stage counted: " +
+                          ", ".join(st.name for st in layer.stages if st.bound == "hbm"),
               "schedule": ("one stream" if not getattr(layer, "overlap", False) else
                            "weight-gradient GEMM on a second stream beside col2im")}
     if algo:
@@ -831,6 +912,9 @@ def main():
                     help="auto: what nn.conv2d builds (the fused ops without a column buffer where they apply, else "
                          "im2col + the fused products over the column buffer); col: the latter for every layer; "
                          "im2col: always the literal im2col -> Mul22 -> transpose composition")
+    ap.add_argument("--detail-file", default=None, help="also write the full JSON (stage tables of every workload) here")
+    ap.add_argument("--hbm-reference-only", action="store_true",
+                    help="run only the plain streaming kernels (copy, fill, sum, add over 1 GiB) and print their table")
     ap.add_argument("--only", action="store_true",
                     help="measure --workload alone (profiling runs); by default the headline workload is followed by "
                          "the other configurations, reported under `workloads`")
@@ -841,6 +925,9 @@ def main():
 
     from cgt_amd import capi
     capi.require_gpu()
+    if args.hbm_reference_only:
+        print(json.dumps({"hbm_reference": hbm_reference(), "peak_GBps": HBM_PEAK_GBS, "device": capi.device_name()}))
+        return
     is_gemm = args.workload == GEMM_WORKLOAD
     res, cfg = measure(args.workload, args, primary=True)
     out = {
@@ -869,8 +956,8 @@ def main():
             r["unit"] = "TFLOP/s"
             out["workloads"][name] = r
     if "hbm_reference" in out:
-        # every HBM-bound stage also against what a plain device-to-device copy reaches in this run
-        copy = out["hbm_reference"]["copy_1GiB"]["GBps"]
+        # every HBM-bound stage also against what this library's streaming copy reaches in this run
+        copy = out["hbm_reference"]["copy_kernel_1GiB"]["GBps"]
         for table in [out["stages"]] + [w["stages"] for w in out["workloads"].values()]:
             for row in table:
                 if row["bound"] == "hbm" and "GBps_in_step" in row:
@@ -879,9 +966,77 @@ def main():
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample)
     elif not args.no_cpu:
         out["cpu_baseline"] = cpu_gemm_baseline()
-    print(json.dumps(out))
+    # stdout carries ONE compact line (the contract fields, the roofline, the CPU baseline, the parity
+    # gate and one summary row per other workload); the full stage tables go to stderr as one JSON
+    # line behind the word "detail", and to --detail-file when given
+    detail = json.dumps(out)
+    sys.stderr.write("detail " + detail + "\n")
+    sys.stderr.flush()
+    if args.detail_file:
+        with open(args.detail_file, "w") as fh:
+            fh.write(detail + "\n")
+    print(json.dumps(compact_line(out), separators=(",", ":")))
+    sys.stdout.flush()
     if not parity_ok:
         sys.exit("bench.py: parity gate failed")
+
+
+MAX_LINE = 3500     # characters of the stdout line (a longer one has been cut by a harness that captures a tail)
+
+
+def _clock_frac(row):
+    return row.get("frac_in_step", row.get("frac"))
+
+
+def _summary(res):
+    """One short row per workload: whole-step value, its slowest GEMM launch as fraction of the
+    fp32 MFMA peak, the HBM-bound stage furthest from 8 TB/s, and the gate's verdict."""
+    hbm = [(r["stage"], _clock_frac(r)) for r in res["stages"] if r["bound"] == "hbm" and _clock_frac(r) is not None]
+    row = {"value": res["value"], "ms_per_step": res["ms_per_step"], "gemm_frac": res["roofline"]["frac"],
+           "parity_ok": res["parity"]["ok"]}
+    if hbm:
+        best, worst = max(hbm, key=lambda t: t[1]), min(hbm, key=lambda t: t[1])
+        row["hbm_best"], row["hbm_worst"] = [best[0], round(best[1], 3)], [worst[0], round(worst[1], 3)]
+    return row
+
+
+def compact_line(out):
+    """The stdout line: the contract fields in full, everything else boiled down."""
+    keep = ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+            "vs_baseline", "dtype", "data", "device")
+    line = {k: out[k] for k in keep if k in out}
+    cfg = out["config"]
+    line["config"] = {k: cfg[k] for k in ("workload", "x", "filters", "pad", "stride", "conv_algo", "value_is", "lrn") if k in cfg}
+    roof = out["roofline"]
+    line["roofline"] = {k: roof[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel", "stage",
+                                             "flops_per_launch", "avg_launch_ms", "timing")}
+    line["frac_fp32_mfma_peak"] = out["frac_fp32_mfma_peak"]
+    if "cpu_baseline" in out:
+        cpu = out["cpu_baseline"]
+        line["cpu_baseline"] = {k: cpu[k] for k in ("value", "unit", "cores", "kind") if k in cpu}
+        line["cpu_baseline"]["value"] = round(cpu["value"], 4)
+        line["cpu_baseline"]["sample"] = cpu.get("sample_short", cpu["sample"])[:220]
+    par = out["parity"]
+    line["parity"] = {"ok": bool(par["ok"] and all(w["parity"]["ok"] for w in out.get("workloads", {}).values()))}
+    for k in ("bit_exact", "rel_fro", "mul22_x4_batched_rel_fro", "skipped"):
+        if k in par:
+            line["parity"][k] = par[k]
+    # stage -> [ms inside the step, fraction of its roof (8 TB/s or 157.3 TFLOP/s)]
+    line["stages"] = {r["stage"]: [r.get("ms_in_step", r.get("ms")), _clock_frac(r)] for r in out["stages"]}
+    if "op_api_step" in out:
+        line["op_api_step"] = {k: out["op_api_step"][k] for k in ("ms_per_step", "TFLOPs")}
+    if "hbm_reference" in out:      # fraction of 8 TB/s that plain streaming kernels reach in this run
+        line["hbm_reference"] = {k: v["frac"] for k, v in out["hbm_reference"].items()}
+    if "workloads" in out:
+        line["workloads"] = {name: _summary(r) for name, r in out["workloads"].items()}
+    line["detail"] = "stderr"
+    # never longer than a tail capture holds: drop the optional parts, least needed first
+    for drop in (None, "stages", "hbm_reference", "op_api_step", "workloads"):
+        if drop:
+            line.pop(drop, None)
+        if len(json.dumps(line, separators=(",", ":"))) <= MAX_LINE:
+            break
+    return line
 
 
 if __name__ == "__main__":

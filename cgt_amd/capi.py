@@ -40,6 +40,8 @@ PROTOTYPES = {
     "cgt_amd_graph_destroy": (c_int, [c_void_p]),
     "cgt_amd_event_elapsed_ms": (c_int, [c_void_p, c_void_p, ctypes.POINTER(ctypes.c_float)]),
     "cgt_amd_memcpy_async": (c_int, [c_int, c_int, c_void_p, c_void_p, c_long, c_void_p]),
+    "cgt_amd_stream_copy": (c_int, [c_void_p, c_void_p, c_long, c_void_p]),
+    "cgt_amd_stream_copy_tune": (c_int, [c_long, c_int]),
     "cgt_amd_im2col_f32": (c_int, [c_void_p] + [c_long] * 4 + [c_int] * 6 + [c_void_p, c_void_p]),
     "cgt_amd_col2im_f32": (c_int, [c_void_p] + [c_long] * 4 + [c_int] * 6 + [c_void_p, c_void_p]),
     "cgt_amd_pool_outsize": (c_long, [c_long, c_int, c_int, c_int]),

@@ -16,9 +16,11 @@ void clear_error();
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 
 // Library-owned device workspaces (split-K partials, partial sums): one block per
-// (stream, user), grown on demand.  A block that is outgrown is NOT freed -- a HIP
-// graph recorded earlier may have its address baked in, and hipFree would stall the
-// stream -- it is retired and released with the stream (cgt_amd_stream_destroy).
+// (stream, user), grown on demand and geometrically (at least 1.5 x the block that is
+// outgrown).  An outgrown block is not freed on the spot -- kernels in flight may still
+// use it and hipFree would stall the stream -- it is retired: released at the stream's
+// next cgt_amd_synchronize, or, if it was current when a capture began on the stream (a
+// HIP graph may have its address baked in), with the stream (cgt_amd_stream_destroy).
 // Growth while the stream is being captured is refused (an allocation would break the
 // capture): returns nullptr with the message set.
 enum WorkspaceUser { kWsGemm = 0, kWsSum = 1, kWsConvFilter = 2, kWsConvTable = 3, kWsConvData = 4, kWsUsers = 5 };

@@ -70,6 +70,17 @@ int cgt_amd_memcpy(int dest_devtype, int src_devtype, void *dest, const void *sr
 int cgt_amd_memcpy_async(int dest_devtype, int src_devtype, void *dest, const void *src, long nbytes,
                          void *stream);
 
+/* The device-to-device case of that copy as a kernel of this library (the D2D
+ * branch of cgt_memcpy, src/cgt_common.cpp:146-150, without the runtime's copy
+ * engine path): each workgroup streams its own contiguous region with several
+ * 16-byte loads in flight per lane and non-temporal stores; any alignment and
+ * size, the ranges must not overlap.  It is also the yardstick the measurement
+ * script prices the bandwidth-bound kernels against.  cgt_amd_stream_copy_tune
+ * sets the region per workgroup (a multiple of 4096 bytes) and the loads in
+ * flight per lane (4, 8 or 16) for all later calls. */
+int cgt_amd_stream_copy(void *dest, const void *src, long nbytes, void *stream);
+int cgt_amd_stream_copy_tune(long bytes_per_workgroup, int loads_in_flight);
+
 /* Asynchronous fill of `count` 32-bit words with `value` (a fill kernel, safe
  * to capture in a HIP graph). */
 int cgt_amd_fill_u32(void *dst, unsigned int value, long count, void *stream);

@@ -210,6 +210,23 @@ def conv2d_pullback(x, f, gy, pad=(0, 0), stride=(1, 1)):
     return gx, gf
 
 
+def conv_same_padded(x, kernel, total):
+    """x [B,C,H,W] in the zero-padded plane layout that the library's products without a
+    column buffer read (a layout of this library, no reference counterpart; a copy, so the
+    bar is bit-exact): per plane pw zeros, then H + 2 ph rows of W + pw floats (W pixels, pw
+    zeros -- the zeros that end a row are the left padding of the next), rounded up past 16
+    zero floats to a multiple of 16; `total` floats in all, the rest zero."""
+    B, C, H, W = x.shape
+    ph, pw = (kernel[0] - 1) // 2, (kernel[1] - 1) // 2
+    Hp, Wp = H + 2 * ph, W + pw
+    plane = (pw + Hp * Wp + 16 + 15) // 16 * 16
+    ref = np.zeros(total, x.dtype)
+    img = np.zeros((B * C, Hp, Wp), x.dtype)
+    img[:, ph:ph + H, :W] = x.reshape(B * C, H, W)
+    ref[:B * C * plane].reshape(B * C, plane)[:, pw:pw + Hp * Wp] = img.reshape(B * C, -1)
+    return ref
+
+
 # ---------------------------------------------------------------- conv-layer glue
 
 UNARY_OPS = ["abs", "cos", "exp", "log", "neg", "sign", "sin", "square", "sqrt", "tanh", "sigmoid"]

@@ -188,3 +188,28 @@ def test_pool_outsize_rule(L):
     assert L.cgt_amd_pool_outsize(32, 3, 0, 2) == 15
     assert L.cgt_amd_pool_outsize(2, 5, 0, 1) == 0
     assert L.cgt_amd_pool_outsize(8, 2, 0, 0) == 0
+
+
+@pytest.mark.parametrize("loads_in_flight", [8, 4, 16])
+def test_stream_copy_any_alignment_and_size(L, loads_in_flight):
+    # the copy kernel behind device-to-device transports: bytes before the first and after the
+    # last whole 16-byte unit, source and destination aligned differently (no units at all),
+    # sizes around the region of one workgroup; everything outside the range stays untouched
+    assert L.cgt_amd_stream_copy_tune(8192, loads_in_flight) == OK
+    try:
+        rs = np.random.RandomState(7)
+        total = 3 * 65536 + 64
+        src_h = rs.randint(0, 256, total).astype(np.int8)
+        src = gpu(src_h)
+        for so, do, n in [(0, 0, 0), (0, 0, 1), (3, 3, 15), (5, 5, 16), (5, 5, 17), (0, 0, 8192), (16, 32, 8192 + 16),
+                          (1, 1, 65536 + 5), (7, 23, 3 * 8192 - 1), (9, 10, 40000), (0, 16, 2 * 65536 + 48), (4, 0, 65536 * 2 + 33)]:
+            dst = gpu(np.full(total, 0x55, np.int8))
+            assert L.cgt_amd_stream_copy(dst.ptr + do, src.ptr + so, n, None) == OK, _err(L)
+            want = np.full(total, 0x55, np.int8)
+            want[do:do + n] = src_h[so:so + n]
+            assert np.array_equal(dst.get(), want), (so, do, n)
+        assert L.cgt_amd_stream_copy(src.ptr + 8, src.ptr, 100, None) == ERR_ARG and "overlap" in _err(L)
+        assert L.cgt_amd_stream_copy(None, src.ptr, 100, None) == ERR_ARG
+        assert L.cgt_amd_stream_copy_tune(5000, 8) == ERR_ARG and L.cgt_amd_stream_copy_tune(8192, 3) == ERR_ARG
+    finally:
+        assert L.cgt_amd_stream_copy_tune(16384, 4) == OK

@@ -299,6 +299,140 @@ __global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_block_kernel(
     }
 }
 
+// The same block decomposition with both sides of the memory traffic made linear.  The
+// block kernel above keeps 8 bytes of unread input in flight per thread (its neighbourhood
+// loads overlap those of its neighbours four times) and writes 4-byte pieces at odd
+// alignments; on planes of 55 x 55 it moves 2.7 TB/s from memory (its reads alone take as
+// long as its writes alone, and the two do not overlap).  Here a workgroup (1) copies the
+// (mask, top_diff) of its run of planes into LDS with aligned 16-byte loads, all in flight
+// at once, (2) lets every thread form its blocks' cells from LDS -- same candidates, same
+// ascending (ph, pw) order, hence the same bits -- into an LDS image of the output run laid
+// out at the run's own 16-byte phase, and (3) writes that image as aligned 16-byte units
+// (the few floats before the first and after the last whole unit one by one).
+template <class G>
+__global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_linear_kernel(
+    G, const int* __restrict__ mask, const float* __restrict__ top_diff,
+    float* __restrict__ bottom_diff, long nplanes, int H, int W, int PH, int PW, int BH, int BW,
+    int planes_per_wg, int in_floats, int nt) {
+    constexpr int KH = G::kKH, KW = G::kKW, PDH = G::kPH, PDW = G::kPW, SH = G::kSH, SW = G::kSW;
+    constexpr int DY0 = cceildiv(PDH - KH + 1, SH), DY1 = cfloordiv(SH - 1 + PDH, SH);
+    constexpr int DX0 = cceildiv(PDW - KW + 1, SW), DX1 = cfloordiv(SW - 1 + PDW, SW);
+    constexpr int NY = DY1 - DY0 + 1, NX = DX1 - DX0 + 1;
+    extern __shared__ float tile[];
+    const long p0 = (long)blockIdx.x * planes_per_wg;
+    const long left = nplanes - p0;
+    const int np = left < planes_per_wg ? (int)left : planes_per_wg;
+    const int HW = H * W, PP = PH * PW, per_plane = BH * BW;
+    // LDS: td [in_floats], mk [in_floats], out [rest]; every part a multiple of 4 floats
+    float* td = tile;
+    int* mk = reinterpret_cast<int*>(tile + in_floats);
+    float* outp = tile + 2 * in_floats;
+
+    // (1) the input run [p0 * PP, (p0 + np) * PP) of both arrays, from the 16-byte boundary at or below its start
+    const long in0 = p0 * PP, in_end = nplanes * (long)PP;
+    const int iphase = (int)(in0 & 3);
+    const int nin = np * PP;
+    const int in_units = (iphase + nin + 3) >> 2;
+    const float4* td4 = reinterpret_cast<const float4*>(top_diff + (in0 - iphase));
+    const int4* mk4 = reinterpret_cast<const int4*>(mask + (in0 - iphase));
+    // units that end inside the arrays are loaded four per thread before the first is parked (indices
+    // past the run are clamped to its last such unit and dropped); the unit holding the arrays' last
+    // floats, if it is cut, goes float by float
+    const int safe_units = (int)min((long)in_units, (in_end - (in0 - iphase)) >> 2);
+    for (int base = threadIdx.x; base < safe_units; base += kPoolThreads * 4) {
+        float4 tv4[4];
+        int4 mv4[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int u = min(base + k * kPoolThreads, safe_units - 1);
+            tv4[k] = td4[u];
+            mv4[k] = mk4[u];
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int u = base + k * kPoolThreads;
+            if (u < safe_units) {
+                reinterpret_cast<float4*>(td)[u] = tv4[k];
+                reinterpret_cast<int4*>(mk)[u] = mv4[k];
+            }
+        }
+    }
+    if (safe_units < in_units && threadIdx.x < 4) {
+        const long g = in0 - iphase + 4L * safe_units + threadIdx.x;
+        if (g < in_end) {
+            td[4 * safe_units + threadIdx.x] = top_diff[g];
+            mk[4 * safe_units + threadIdx.x] = mask[g];
+        }
+    }
+    __syncthreads();
+
+    // (2) blocks -> LDS image of the output run, at the run's phase
+    const long out0 = p0 * (long)HW;
+    const int ophase = (int)(out0 & 3);
+    const int n = np * per_plane;
+    const float rPer = 1.0f / per_plane, rBW = 1.0f / BW;
+    for (int j = threadIdx.x; j < n; j += kPoolThreads) {
+        const int pl = fastdiv(j, rPer), r = j - pl * per_plane;
+        const int by = fastdiv(r, rBW), bx = r - by * BW;
+        const int* mkp = mk + iphase + pl * PP;
+        const float* tdp = td + iphase + pl * PP;
+        int mv[NY][NX];
+        float tv[NY][NX];
+#pragma unroll
+        for (int dy = 0; dy < NY; ++dy)
+#pragma unroll
+            for (int dx = 0; dx < NX; ++dx) {
+                const int y = by + DY0 + dy, x = bx + DX0 + dx;
+                const bool ok = y >= 0 && y < PH && x >= 0 && x < PW;
+                const int o = ok ? y * PW + x : 0;
+                const int m = mkp[o];
+                const float t = tdp[o];
+                mv[dy][dx] = ok ? m : -1;
+                tv[dy][dx] = ok ? t : 0.0f;
+            }
+        float* dst = outp + ophase + pl * HW;
+#pragma unroll
+        for (int i = 0; i < SH; ++i) {
+            const int h = by * SH + i;
+            if (h >= H) break;
+#pragma unroll
+            for (int jj = 0; jj < SW; ++jj) {
+                const int cell = h * W + bx * SW + jj;
+                float acc = 0.0f;
+#pragma unroll
+                for (int dy = 0; dy < NY; ++dy)
+#pragma unroll
+                    for (int dx = 0; dx < NX; ++dx) {
+                        const bool covers = DY0 + dy >= cceildiv(i + PDH - KH + 1, SH) && DY0 + dy <= cfloordiv(i + PDH, SH) &&
+                                            DX0 + dx >= cceildiv(jj + PDW - KW + 1, SW) && DX0 + dx <= cfloordiv(jj + PDW, SW);
+                        if (covers) acc = (mv[dy][dx] == cell) ? acc + tv[dy][dx] : acc;
+                    }
+                if (bx * SW + jj < W) dst[cell] = acc;
+            }
+        }
+    }
+    __syncthreads();
+
+    // (3) the image goes out: whole units between the first and the last 16-byte boundary inside the run
+    const int nout = np * HW;
+    float* gbase = bottom_diff + (out0 - ophase);
+    const int first = ophase ? 1 : 0, last = (ophase + nout) >> 2;      // units [first, last) lie inside the run
+    for (int u = first + threadIdx.x; u < last; u += kPoolThreads) {
+        const float4 v = reinterpret_cast<const float4*>(outp)[u];
+        if (nt) stream_store4(gbase + 4 * u, v.x, v.y, v.z, v.w);
+        else *reinterpret_cast<float4*>(gbase + 4 * u) = v;
+    }
+    if (threadIdx.x < 8) {
+        const int e = threadIdx.x & 3;
+        if (threadIdx.x < 4) {      // floats of the first unit that belong to this run
+            if (ophase && e >= ophase && e < ophase + nout) gbase[e] = outp[e];
+        } else {                    // floats behind the last whole unit
+            const int f = 4 * last + e;
+            if (last >= first && f < ophase + nout) gbase[f] = outp[f];
+        }
+    }
+}
+
 template <class G>
 __global__ __launch_bounds__(kPoolThreads) void max_pool_bwd_direct_kernel(
     G g, const int* __restrict__ mask, const float* __restrict__ top_diff,
@@ -591,10 +725,28 @@ static int launch_pool_bwd(G g, const int* mask, const float* top_diff, long npl
                     return CGT_AMD_OK;
                 }
             }
-            // Odd widths (the AlexNet planes of 55 x 55) keep the block kernel with 4-byte stores:
-            // collecting the planes in LDS to write them as one linear region of 16-byte units
-            // measured 0.096 ms inside the AlexNet step against 0.085, and one column per thread
-            // (every store instruction one contiguous run) 0.101.
+            // Rows that are not whole 16-byte units (the AlexNet planes of 55 x 55): both sides linear
+            // through LDS.  Inside the AlexNet conv1 step: 0.042 ms against the block kernel's 0.082
+            // (one plane per workgroup; two planes 0.052, three 0.058: many short-lived workgroups
+            // stream better than few long ones; plain instead of non-temporal stores 0.043 and the
+            // kernel after it 5 % slower).
+            {
+                const long per_plane_floats = 2 * PH * PW + H * W;
+                // at least 8 KB of output per workgroup (tiny planes share one), within 36 KB of LDS
+                const long ppw_l = std::max(1L, std::min({(36 * 1024) / (per_plane_floats * 4), cdiv(8192L, H * W * 4), cdiv(nplanes, 2048L)}));
+                const int nt = 1;
+                const long in_floats = (ppw_l * PH * PW + 6) / 4 * 4, out_floats = (ppw_l * H * W + 6) / 4 * 4;
+                const size_t lds = (size_t)(2 * in_floats + out_floats) * sizeof(float);
+                const bool aligned = reinterpret_cast<uintptr_t>(bottom_diff) % 16 == 0 && reinterpret_cast<uintptr_t>(mask) % 16 == 0 &&
+                                     reinterpret_cast<uintptr_t>(top_diff) % 16 == 0;
+                if (ppw_l > 0 && aligned && lds <= 64 * 1024 && ppw_l * BH * BW < kFastdivLimit && ppw_l * H * W < kFastdivLimit) {
+                    max_pool_bwd_linear_kernel<G><<<dim3((unsigned)cdiv(nplanes, ppw_l)), dim3(kPoolThreads), lds, st>>>(
+                        g, mask, top_diff, bottom_diff, nplanes, (int)H, (int)W, (int)PH, (int)PW, (int)BH, (int)BW,
+                        (int)ppw_l, (int)in_floats, nt);
+                    CGT_LAUNCH_CHECK("max_pool_bwd_linear_kernel");
+                    return CGT_AMD_OK;
+                }
+            }
             const int vec2 = W % 2 == 0 && reinterpret_cast<uintptr_t>(bottom_diff) % 8 == 0;
             max_pool_bwd_block_kernel<G><<<dim3((unsigned)blocks), dim3(kPoolThreads), 0, st>>>(
                 g, mask, top_diff, bottom_diff, nplanes, (int)H, (int)W, (int)PH, (int)PW, (int)BH,

@@ -167,6 +167,14 @@ POOL_CASES = [
     ((2, 3, 12, 16), (3, 3), (1, 1), (2, 2)),      # W % 4 == 0: the pullback writes 16-byte rows (overlapping windows, padding)
     ((3, 5, 4, 4), (2, 2), (0, 0), (2, 2)),        # one 16-byte unit per row
     ((2, 2, 9, 8), (3, 3), (0, 0), (2, 2)),
+    # odd planes, overlapping windows: the pullback goes through LDS in runs of planes that start at
+    # every 16-byte phase; input runs whose last 16-byte unit is cut by the end of the arrays
+    ((7, 3, 5, 7), (3, 3), (0, 0), (2, 2)),
+    ((5, 13, 9, 11), (3, 3), (1, 1), (2, 2)),
+    ((1, 1, 3, 5), (3, 3), (0, 0), (2, 2)),
+    ((37, 59, 7, 7), (3, 3), (0, 0), (2, 2)),      # several planes per workgroup, the last workgroup short
+    ((3, 1, 55, 55), (3, 3), (0, 0), (2, 2)),
+    ((1, 5, 1, 9), (3, 3), (1, 1), (2, 2)),
 ]
 
 

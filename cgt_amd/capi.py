@@ -66,6 +66,8 @@ PROTOTYPES = {
                                       c_void_p, c_long, c_long, c_void_p, c_long, c_long,
                                       c_void_p, c_long, c_long, c_void_p]),
     "cgt_amd_conv_same_supported": (c_int, [c_long, c_long] + [c_int] * 6),
+    "cgt_amd_conv_same_fits": (c_int, [c_long] * 5 + [c_int, c_int]),
+    "cgt_amd_conv_col_fits": (c_int, [c_long] * 4),
     "cgt_amd_conv_same_padded_size": (c_long, [c_long, c_long, c_long, c_int, c_int]),
     "cgt_amd_conv_same_pad_f32": (c_int, [c_void_p, c_long, c_long, c_long, c_int, c_int, c_void_p, c_void_p]),
     "cgt_amd_conv_same_filter_f32": (c_int, [c_void_p, c_long, c_long, c_int, c_int, c_int, c_void_p, c_void_p]),

@@ -20,7 +20,7 @@ from . import build as _build
 from . import core, rt
 
 # bump when the object model in csrc/include/cgt_common.h changes layout
-CPP_ABI_VERSION = 1
+CPP_ABI_VERSION = 2
 # headers every closure is compiled against: cgtArray's accessors are inline, so
 # their text is part of each cached library and therefore of its cache key
 _ABI_HEADERS = ("cgt_common.h", "cgt_amd.h")
@@ -245,6 +245,7 @@ def prebuild_standard_ops():
         (core.Repeat((0, 2, 3)), [T4, S, S, S]),
         (core.Sum((0, 2, 3)), [T4]),
         (core.Fill(0.0), [S, S, S, S]),
+        (core.ExtentAsFloat(), [S]),
         # by-value closures a compiled `function` replays
         (core.Reshape(), [T4, S, S]),
         (core.TupleIndex(0), [core.TupleType(T4, I4)]),

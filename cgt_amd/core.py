@@ -828,7 +828,9 @@ class Reshape(Op):
                     n *= newshape[i];
                 }
                 cgt_check(n == in->size(), "Reshape: size mismatch (%ld vs %ld)", n, in->size());
-                return new cgtArray(cldata->ndim, newshape, in->dtype(), in->devtype(), in->data(), false);
+                cgtArray* view = new cgtArray(cldata->ndim, newshape, in->dtype(), in->devtype(), in->data(), false);
+                view->set_base(in);     // the view keeps the array it shows alive
+                return view;
             }"""
         return NativeCompileInfo(code, closure_triples=[("ndim", ctypes.c_int, len(input_types) - 1)],
                                  gpu_deref_mask=(False,) * len(input_types))
@@ -1077,10 +1079,59 @@ class ElwiseBinary(Op):
                                  gpu_deref_mask=(True, True))
 
 
+class ExtentAsFloat(Op):
+    """An int64 host scalar (an extent, or integer arithmetic over extents) as a 0-d float32
+    device array.  The reference's cgt.size is a symbolic i8 scalar that elementwise ops
+    promote (cgt/core.py:1319-1333, 1614-1640), so `x / cgt.size(x, 0)` is right at any
+    shape; here extents are python ints that carry their expression, and this op keeps
+    that expression alive inside a compiled function instead of freezing the traced value
+    into a constant.  The scalar is read on the host (like the shape operands of Reshape
+    and Fill) and written by the fill kernel."""
+    available_impls = ("native_gpu",)
+
+    def get_diff(self, num_inputs):
+        return [False] * num_inputs
+
+    def __repr__(self):
+        return "ExtentAsFloat"
+
+    def pullback(self, inputs, output, goutput):
+        raise MethodNotDefined("an extent is not differentiable")
+
+    def shp_apply(self, inputs):
+        return []
+
+    def typ_apply(self, input_types):
+        assert len(input_types) == 1 and input_types[0].dtype == "i8" and input_types[0].ndim == 0, \
+            "ExtentAsFloat takes one integer scalar"
+        return TensorType(floatX, 0)
+
+    def get_native_compile_info(self, input_types, devtype):
+        assert devtype == "gpu"
+        code = r"""
+            CGT_EXPORT_C void $function(void* cl, cgtArray** reads, cgtArray* write) {
+                int rc = cgt_amd_fill_f32((float*)write->data(), (float)reads[0]->at<long>(0), 1, cgt_get_stream());
+                cgt_check(rc == CGT_AMD_OK, "ExtentAsFloat: %s", cgt_amd_last_error());
+            }"""
+        return NativeCompileInfo(code, includes=["cgt_amd.h"], gpu_deref_mask=(False,))
+
+
+def extent_as_float(n):
+    """float32 scalar node holding the extent `n`; a plain constant when `n` does not depend
+    on any array's shape."""
+    n = ShapeInt._lift(n)
+    if n.is_constant():
+        return constant(np.float32(int(n)))
+    return Result(ExtentAsFloat(), [constant(n)])
+
+
 def _scalar_operand(v, like):
-    """python numbers become 0-d device arrays of the other operand's float type."""
+    """python numbers become 0-d device arrays of the other operand's float type; an extent
+    that depends on an array's shape stays an expression (ExtentAsFloat)."""
     if isinstance(v, Node):
         return v
+    if isinstance(v, ShapeInt) and not v.is_constant():
+        return extent_as_float(v)
     if isinstance(v, (int, float, np.integer, np.floating)) or (isinstance(v, np.ndarray) and v.ndim == 0):
         return constant(np.float32(v))
     return as_node(v)
@@ -1312,12 +1363,8 @@ def mean(x, axis=None, keepdims=False):
     n = 1
     for ax in axes:
         n *= size(x, ax)
-    divisor = constant(np.float32(n))
-    # the divisor's VALUE comes from extents: a function compiled from this graph serves
-    # other shapes only if those extents do not depend on its arguments
-    divisor.shape_baked = not ShapeInt._lift(n).is_constant()
-    divisor.baked_expr = ShapeInt._lift(n).expr
-    return sum(x, axis=axes, keepdims=keepdims) / divisor
+    # the divisor follows the extents at every call of a compiled function
+    return sum(x, axis=axes, keepdims=keepdims) / extent_as_float(n)
 
 
 def fill(val, shp):

@@ -222,6 +222,7 @@ struct Interpreter {
         if (in.backing && need <= in.backing_bytes) {
             cgtArray* b = static_cast<cgtArray*>(in.backing.get());
             out = new cgtArray(ndim, shape, dtype, in.write.devtype, b->data(), false);
+            out->set_base(b);       // whoever keeps the view keeps the buffer
         } else {
             out = new cgtArray(ndim, shape, dtype, in.write.devtype);
             in.backing = out;

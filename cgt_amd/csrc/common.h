@@ -55,6 +55,8 @@ struct ConvGemm {
     const PatchGeom* patch = nullptr;      // modes 1, 4: gather the column buffer's elements from the image
 };
 int sgemm_conv(const ConvGemm& cv, long M, long N, const float* A, const float* B, float* C, long ldc, void* stream);
+// out[i] = ws[0][i] + ... + ws[n - 1][i], i < count, added in that order (gemm.hip's split-K reduce)
+int reduce_partials(const float* ws, float* out, long count, int n, void* stream);
 // 1 if sgemm_conv has a tile shape for these extents (output channels of the product, channels of the image)
 bool sgemm_conv_supported(int mode, long filters, long channels);
 

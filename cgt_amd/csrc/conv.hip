@@ -103,6 +103,22 @@ static int check_same(const char* what, SameGeom& g, long B, long C, long H, lon
 
 using namespace cgt_amd;
 
+CGT_API int cgt_amd_conv_same_fits(long B, long C, long H, long W, long L, int kh, int kw) {
+    SameGeom g;
+    if (B < 0 || C < 1 || H < 1 || W < 1 || L < 1 || !make_geom(g, B, C, H, W, L, kh, kw)) return 0;
+    // reciprocal index arithmetic of the pad kernels; 32-bit lane offsets of the products (a tile's rows
+    // span the channels of a whole image in the weight gradient, whose operands are x and the cotangent)
+    if (g.plane >= (1L << 21) || C * g.plane >= (1L << 30) || L * g.plane >= (1L << 30)) return 0;
+    return B * g.tpi * 128 < (1L << 31) - 128 && B * g.spi * 16 < (1L << 31) - 128 ? 1 : 0;
+}
+
+CGT_API int cgt_amd_conv_col_fits(long B, long P, long Z, long L) {
+    if (B < 0 || P < 1 || Z < 1 || L < 1) return 0;
+    // forward product: a lane's 32-bit offset spans the images a tile of 128 columns touches
+    if (B * P >= (1L << 31) - 128 || (127 / P + 2) * L * P >= (1L << 30)) return 0;
+    return Z < (1L << 31) - 128 && L * Z < (1L << 29) ? 1 : 0;
+}
+
 CGT_API int cgt_amd_conv_same_supported(long C, long L, int kh, int kw, int ph, int pw, int sh, int sw) {
     if (sh != 1 || sw != 1 || kh % 2 == 0 || kw % 2 == 0 || ph != (kh - 1) / 2 || pw != (kw - 1) / 2) return 0;
     // forward: C channels in, L filters; data gradient: L channels in, C "filters"; weight gradient: both
@@ -245,6 +261,30 @@ CGT_API int cgt_amd_conv_same_bwd_filter_f32(const float* gypad, const float* xp
     return cgt_amd_transpose4_f32(wk, ws, ax, gf, stream);
 }
 
+// The weight gradient's K axis is cut per image, so its partial sums are at least one [L][Z]
+// block per image.  While those fit 256 MiB (and the product's own limits) the batch is one
+// product; beyond that it runs in groups of images, each group's result goes to a second
+// workspace and the groups are summed in order: any batch size, fixed order of additions.
+template <class F>
+static int wgrad_in_groups(long B, long P, long Z, long L, float* gf, void* stream, const char* what, F&& product) {
+    CGT_ARG_CHECK(P < (1L << 31) - 128, "%s: too many output pixels per image", what);
+    const long per_image = L * Z;
+    long group = std::max(1L, (64L << 20) / per_image);                 // 256 MiB of partial sums
+    group = std::min({group, ((1L << 31) - 129) / P, (1L << 19)});      // the product's own limits on pixels and splits
+    CGT_ARG_CHECK(group >= 1, "%s: image too large", what);
+    if (B <= group) return product(0, B, gf);
+    const long ngroups = cdiv(B, group);
+    CGT_ARG_CHECK(ngroups < (1L << 30), "%s: too many images", what);
+    float* part = stream_workspace(stream, kWsConvData, (size_t)ngroups * per_image * sizeof(float), what);
+    if (!part) return CGT_AMD_ERR_NOMEM;
+    for (long gi = 0; gi < ngroups; ++gi) {
+        const long b0 = gi * group;
+        int rc = product(b0, std::min(group, B - b0), part + gi * per_image);
+        if (rc) return rc;
+    }
+    return reduce_partials(part, gf, per_image, (int)ngroups, stream);
+}
+
 // ---- any geometry, over the column buffer of im2col: the three products of conv2d with the
 // NCHW side read and written in place (no [B*m*n, L] intermediate, no transposes).
 //   col [B * P][Z] (P = m * n output pixels per image, Z = C * kh * kw), f [L][Z] (= [L,C,kh,kw]),
@@ -285,9 +325,10 @@ CGT_API int cgt_amd_conv_col_bwd_filter_f32(const float* gy, const float* col, l
     CGT_ARG_CHECK(gf, "conv_col_bwd_filter: null pointer");
     if (B == 0 || P == 0) return cgt_amd_fill_u32(gf, 0u, L * Z, stream);
     CGT_ARG_CHECK(gy && col, "conv_col_bwd_filter: null pointer");
-    CGT_ARG_CHECK(B * P < (1L << 31) - 128, "conv_col_bwd_filter: too many output pixels");
-    ConvGemm cv = {4, B, Z, P, 0, 1, 1, 0, 0, 0, 0, nullptr, 0, nullptr};
-    return sgemm_conv(cv, L, Z, gy, col, gf, Z, stream);
+    return wgrad_in_groups(B, P, Z, L, gf, stream, "conv_col_bwd_filter", [&](long b0, long nb, float* out) {
+        ConvGemm cv = {4, nb, Z, P, 0, 1, 1, 0, 0, 0, 0, nullptr, 0, nullptr};
+        return sgemm_conv(cv, L, Z, gy + b0 * L * P, col + b0 * P * Z, out, Z, stream);
+    });
 }
 
 // ---- any geometry, no column buffer for the forward product and the weight gradient: the two
@@ -338,6 +379,10 @@ CGT_API int cgt_amd_conv_patch_bwd_filter_f32(const float* gy, const float* x, l
     CGT_ARG_CHECK(gf, "conv_patch_bwd_filter: null pointer");
     if (B == 0) return cgt_amd_fill_u32(gf, 0u, L * Z, stream);
     CGT_ARG_CHECK(gy && x, "conv_patch_bwd_filter: null pointer");
-    ConvGemm cv = {4, B, Z, P, 0, 1, 1, 0, 0, 0, 0, nullptr, 0, nullptr, &pg};
-    return sgemm_conv(cv, L, Z, gy, x, gf, Z, stream);
+    return wgrad_in_groups(B, P, Z, L, gf, stream, "conv_patch_bwd_filter", [&](long b0, long nb, float* out) {
+        PatchGeom part = pg;
+        part.x = x + b0 * C * H * W;
+        ConvGemm cv = {4, nb, Z, P, 0, 1, 1, 0, 0, 0, 0, nullptr, 0, nullptr, &part};
+        return sgemm_conv(cv, L, Z, gy + b0 * L * P, part.x, out, Z, stream);
+    });
 }

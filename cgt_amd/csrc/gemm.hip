@@ -1124,6 +1124,21 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     }
 }
 
+// out[i] = ws[0][i] + ws[1][i] + ... + ws[n - 1][i] for i < count, added in that order (the split-K
+// reduce kernel on a caller's partial results: the weight gradient of a very large batch sums
+// per-group results with it).
+int reduce_partials(const float* ws, float* out, long count, int n, void* stream) {
+    const bool vec = count % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && reinterpret_cast<uintptr_t>(ws) % 16 == 0;
+    const long blocks = cdiv(count, vec ? 256L : 64L);
+    CGT_ARG_CHECK(blocks < (1L << 31), "reduce_partials: too many elements");
+    hipStream_t st = as_stream(stream);
+    // the kernel addresses its output as rows of N floats ldc apart: rows of 1024 back to back are the flat array
+    if (vec) splitk_reduce_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(ws, out, count, 1024, 1024, n);
+    else splitk_reduce_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(ws, out, count, 1024, 1024, n);
+    CGT_LAUNCH_CHECK("splitk_reduce_kernel");
+    return CGT_AMD_OK;
+}
+
 // Split-K / tail workspaces: one per stream, owned by the library (see common.h).
 static float* get_workspace(void* stream, size_t bytes) {
     return stream_workspace(stream, kWsGemm, bytes, "sgemm");

@@ -159,6 +159,13 @@ public:
     }
     void print();
 
+    // A view (ownsdata() false) may name the object whose storage it shows: that object then
+    // lives at least as long as the view.  The interpreter's views of its instruction buffers
+    // and Reshape's results do, so an output a caller keeps stays valid when a later call
+    // makes the interpreter drop the buffer for a larger one.
+    void set_base(cgtObject* base) { base_ = base; }
+    cgtObject* base() const { return base_.get(); }
+
 private:
     int ndim_;
     long* shape_;
@@ -166,6 +173,7 @@ private:
     cgtDevtype devtype_;
     bool owns_;
     void* data_;
+    IRC<cgtObject> base_;       // last member: the offsets of the fields above are those of earlier builds
 };
 
 class CGT_EXPORT cgtTuple : public cgtObject {

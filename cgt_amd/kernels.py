@@ -305,6 +305,20 @@ def conv_same_supported(C, L, kernel, pad, stride):
     return bool(capi.lib().cgt_amd_conv_same_supported(int(C), int(L), *_geom(kernel, pad, stride)))
 
 
+def conv_same_fits(xshape, L, kernel):
+    """Whether a batch of images of this shape is inside what the products over the padded image index."""
+    B, C, H, W = (int(v) for v in xshape)
+    return bool(capi.lib().cgt_amd_conv_same_fits(B, C, H, W, int(L), int(kernel[0]), int(kernel[1])))
+
+
+def conv_col_fits(xshape, L, kernel, pad, stride):
+    """Whether the products over the column buffer of this layer are inside what they index."""
+    B, C, H, W = (int(v) for v in xshape)
+    g = _geom(kernel, pad, stride)
+    m, n = conv_outsize(H, g[0], g[2], g[4]), conv_outsize(W, g[1], g[3], g[5])
+    return bool(capi.lib().cgt_amd_conv_col_fits(B, m * n, C * g[0] * g[1], int(L)))
+
+
 def conv_same_padded_size(planes, H, W, kernel):
     n = capi.lib().cgt_amd_conv_same_padded_size(int(planes), int(H), int(W), int(kernel[0]), int(kernel[1]))
     if n < 0:

@@ -61,10 +61,13 @@ def conv2d(x_BKRC, f_LKrc, kernelshape, pad=(0, 0), stride=(1, 1)):
     _check_geometry(x_BKRC, K, tuple(kernelshape), tuple(pad), tuple(stride))
     if _CONV_ALGO == "auto" and conv_same.supported(x_BKRC, f_LKrc, kernelshape, pad, stride):
         return conv_same.conv_same(x_BKRC, f_LKrc, kernelshape)
-    if _CONV_ALGO == "auto" and conv_col.patch_supported(x_BKRC, kernelshape, pad, stride):
+    # extents beyond what the fused products index fall through: padded-image products ->
+    # products over a column buffer -> the literal composition, which takes any size
+    fits_col = conv_col.col_supported(x_BKRC, f_LKrc, kernelshape, pad, stride)
+    if _CONV_ALGO == "auto" and fits_col and conv_col.patch_supported(x_BKRC, kernelshape, pad, stride):
         return conv_col.conv_patch(x_BKRC, f_LKrc, kernelshape, pad, stride)
     col_BmnZ = im2col(x_BKRC, kernelshape, pad, stride)
-    if _CONV_ALGO != "im2col":
+    if _CONV_ALGO != "im2col" and fits_col:
         return conv_col.conv_col(col_BmnZ, f_LKrc)
     f_LZ = f_LKrc.reshape([L, K * r * c])
     B, m, n, Z = col_BmnZ.shape
@@ -129,9 +132,11 @@ class SpatialConvolution(object):
         if (_CONV_FUSION and _CONV_ALGO == "auto"
                 and conv_same.supported(x, self.weight, self.kernelshape, self.pad, self.stride)):
             return conv_same.conv_same(x, self.weight, self.kernelshape, bias=self.bias)
-        if _CONV_FUSION and _CONV_ALGO == "auto" and conv_col.patch_supported(x, self.kernelshape, self.pad, self.stride):
+        fits_col = conv_col.col_supported(x, self.weight, self.kernelshape, self.pad, self.stride)
+        if (_CONV_FUSION and _CONV_ALGO == "auto" and fits_col
+                and conv_col.patch_supported(x, self.kernelshape, self.pad, self.stride)):
             return conv_col.conv_patch(x, self.weight, self.kernelshape, self.pad, self.stride, bias=self.bias)
-        if _CONV_FUSION and _CONV_ALGO != "im2col":
+        if _CONV_FUSION and _CONV_ALGO != "im2col" and fits_col:
             col = im2col(x, self.kernelshape, self.pad, self.stride)
             return conv_col.conv_col(col, self.weight, bias=self.bias)
         tmp = conv2d(x, self.weight, self.kernelshape, self.pad, self.stride)

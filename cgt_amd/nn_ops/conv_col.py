@@ -315,13 +315,20 @@ class ConvPatchBackwardFilter(core.Op):
                                       gpu_deref_mask=(True, True, False))
 
 
+def col_supported(x, f, kernelshape, pad, stride):
+    """Whether the products over the column buffer cover a layer of these extents
+    (cgt_amd_conv_col_fits); the literal composition has no such limits."""
+    from .. import kernels
+    return kernels.conv_col_fits(core.shape(x), core.size(f, 0), kernelshape, pad, stride)
+
+
 def patch_supported(x, kernelshape, pad, stride):
     """Whether the layer is one for the patch-gather products: few input channels (the image is small
     and re-read from cache, and a patch row is a long enough run to gather) and extents the
     32-bit offsets of the gather cover (cgt_amd_conv_patch_supported)."""
     from .. import kernels
     shp = [int(v) for v in core.shape(x)]
-    return shp[1] < 16 and kernels.conv_patch_supported(shp, kernelshape, pad, stride)
+    return shp[1] < 16 and kernels.conv_patch_supported(shp, kernelshape, pad, stride)      # (filter count: see nn.conv2d)
 
 
 def conv_patch(x, f, kernelshape, pad, stride, bias=None, relu=False):

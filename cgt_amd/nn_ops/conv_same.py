@@ -278,7 +278,8 @@ class ConvBackwardFilter(core.Op):
 def supported(x, f, kernelshape, pad, stride):
     """Whether these ops cover the layer (see cgt_amd_conv_same_supported)."""
     from .. import kernels
-    return kernels.conv_same_supported(core.size(x, 1), core.size(f, 0), kernelshape, pad, stride)
+    return (kernels.conv_same_supported(core.size(x, 1), core.size(f, 0), kernelshape, pad, stride)
+            and kernels.conv_same_fits(core.shape(x), core.size(f, 0), kernelshape))
 
 
 def conv_same(x, f, kernelshape, bias=None, relu=False):

@@ -224,10 +224,20 @@ class Interpreter(object):
 
 
 class _Borrowed(object):
-    """Device memory owned by a runtime object; `owner` keeps that object alive."""
+    """Device memory owned by a runtime object: holds one reference on that object (a view
+    holds one on the buffer it shows), so the memory outlives later calls of the function
+    that handed it out; `owner` (the interpreter) is kept alive as well."""
 
-    def __init__(self, ptr, nbytes, owner):
-        self.ptr, self.nbytes, self.owner = ptr, nbytes, owner
+    def __init__(self, ptr, nbytes, owner, handle=None):
+        self.ptr, self.nbytes, self.owner, self.handle = ptr, nbytes, owner, handle
+        if handle:
+            lib().cgt_rt_retain(handle)
+
+    def __del__(self):
+        h = getattr(self, "handle", None)
+        if h and _LIB is not None:
+            _LIB.cgt_rt_release(h)
+            self.handle = None
 
 
 def from_cgt_handle(h, owner=None):
@@ -242,6 +252,6 @@ def from_cgt_handle(h, owner=None):
     data = L.cgt_rt_array_data(h)
     nbytes = L.cgt_rt_array_nbytes(h)
     if L.cgt_rt_array_devtype(h) == GPU:
-        return GpuArray(shape, dtype, _buffer=_Borrowed(data, nbytes, owner))
+        return GpuArray(shape, dtype, _buffer=_Borrowed(data, nbytes, owner, h))
     buf = (ctypes.c_char * max(1, nbytes)).from_address(data)
     return np.frombuffer(buf, dtype=dtype, count=int(np.prod(shape)) if shape else 1).reshape(shape).copy()

@@ -346,6 +346,14 @@ int cgt_amd_sgemm_batched(int tA, int tB, long P, long M, long N, long K,
  * col2im. */
 int cgt_amd_conv_same_supported(long C, long L, int kh, int kw, int ph, int pw, int sh, int sw);
 
+/* 1 if, besides that, the extents of this batch of images are inside what the
+ * three entry points index (padded plane below 2^21 floats, the channels of one
+ * padded image below 2^30 floats, pixel tiles of the batch below 2^31): a host
+ * that finds 0 here builds the layer from im2col and the column-buffer products
+ * or cgt_amd_sgemm instead.  No counterpart in the reference (its cuDNN branch
+ * takes any descriptor, cgt/nn_ops/cudnn_ops.py:58-143). */
+int cgt_amd_conv_same_fits(long B, long C, long H, long W, long L, int kh, int kw);
+
 /* Floats in the padded copy of `planes` planes of H x W (tail included); -1 on bad arguments. */
 long cgt_amd_conv_same_padded_size(long planes, long H, long W, int kh, int kw);
 
@@ -415,6 +423,14 @@ int cgt_amd_conv_same_bwd_filter_f32(const float *gypad, const float *xpad, long
  * K axis differs).  In all three: col [B*P][Z] is cgt_amd_im2col_f32's
  * result (P = m*n output pixels per image, Z = C*kh*kw), f [L][Z] is the
  * filter bank [L,C,kh,kw] as it is stored, y / gy are [B,L,m,n]. */
+
+/* 1 if the extents are inside what these products index (B*P pixels below
+ * 2^31, a filter bank of fewer than 2^29 floats, and -- for the forward
+ * product's NCHW epilogue -- about L*P below 2^29); otherwise build the layer
+ * from cgt_amd_sgemm and cgt_amd_transpose4_f32.  The weight gradient takes any
+ * batch size: beyond 256 MiB of per-image partial sums it runs in groups of
+ * images whose results are added in order. */
+int cgt_amd_conv_col_fits(long B, long P, long Z, long L);
 
 /* y = conv(x, f) from col.  bias / relu / mask as in cgt_amd_conv_same_fwd_f32. */
 int cgt_amd_conv_col_fwd_f32(const float *col, const float *f, const float *bias, int relu,

@@ -298,3 +298,62 @@ def test_nn_conv2d_gathers_patches_for_a_layer_with_few_channels():
     x2 = rs.randn(7, 3, 29, 23).astype(np.float32)
     for a, u in zip(f_patch(x2), f_col(x2)):
         assert np.array_equal(a.view(np.uint32), u.view(np.uint32))
+
+
+def test_weight_gradient_of_a_large_batch_runs_in_groups_of_images(K):
+    # the weight gradient's K axis is cut per image, one [L][Z] block of partial sums per image:
+    # 2000 images x 64 x 576 floats is more than the 256 MiB those may take, so the batch runs in two
+    # groups whose results are added in order -- the same entry point, any batch size
+    from cgt_amd.gpuarray import to_gpu
+    rs = np.random.RandomState(8)
+    B, C, H, W, L = 2000, 64, 4, 4, 64
+    x = rs.randn(B, C, H, W).astype(np.float32)
+    gy = rs.randn(B, L, 2, 2).astype(np.float32)
+    f = (rs.randn(L, C, 3, 3) / 24).astype(np.float32)
+    assert B * L * C * 9 * 4 > 256 << 20
+    col = K.im2col(to_gpu(x), (3, 3), (0, 0), (1, 1))
+    gf = K.conv_col_bwd_filter(to_gpu(gy), col, f.shape)
+    d = np.float64
+    _, gf64 = O.conv2d_pullback(x.astype(d), f.astype(d), gy.astype(d), (0, 0), (1, 1))
+    assert relfro(gf.get(), gf64) <= TOL
+    # deterministic, and the gathered form (no column buffer) groups the same way
+    assert np.array_equal(K.conv_col_bwd_filter(to_gpu(gy), col, f.shape).get().view(np.uint32), gf.get().view(np.uint32))
+    x3 = rs.randn(1500, 3, 9, 9).astype(np.float32)
+    gy3 = rs.randn(1500, 512, 3, 3).astype(np.float32)
+    assert 1500 * 512 * 3 * 49 * 4 > 256 << 20
+    gf3 = K.conv_patch_bwd_filter(to_gpu(gy3), to_gpu(x3), (512, 3, 7, 7), (0, 0), (1, 1))
+    _, gf64 = O.conv2d_pullback(x3.astype(d), np.zeros((512, 3, 7, 7), d), gy3.astype(d), (0, 0), (1, 1))
+    assert relfro(gf3.get(), gf64) <= TOL
+
+
+def test_nn_conv2d_falls_through_when_a_layer_outgrows_the_fused_products(K):
+    # a 16-channel 1449 x 1449 same-padding layer: its padded plane has more than 2^21 floats, which the
+    # products over the padded image do not index; nn.conv2d then builds the products over a column
+    # buffer (and beyond their limits the literal composition) instead of raising
+    import cgt_amd as cgt
+    from cgt_amd import nn
+    from cgt_amd.nn_ops import conv_col, conv_same
+    assert K.conv_same_fits((1, 16, 1440, 1440), 16, (3, 3)) and not K.conv_same_fits((1, 16, 1449, 1449), 16, (3, 3))
+    assert K.conv_same_fits((64, 128, 56, 56), 128, (3, 3))
+    assert not K.conv_same_fits((1, 1024, 1024, 1024), 16, (3, 3))          # one image's channels: 2^30 floats
+    assert K.conv_col_fits((128, 3, 227, 227), 96, (11, 11), (0, 0), (4, 4))
+    assert not K.conv_col_fits((1, 16, 2048, 2048), 256, (3, 3), (1, 1), (1, 1))   # L * P = 2^30
+    rs = np.random.RandomState(9)
+    x = rs.randn(1, 16, 1449, 1449).astype(np.float32)
+    f = (rs.randn(16, 16, 3, 3) / 12).astype(np.float32)
+    xn, fn = cgt.constant(x), cgt.constant(f)
+    y = nn.conv2d(xn, fn, (3, 3), pad=(1, 1))
+    assert isinstance(y.op, conv_col.ConvColForward) and not isinstance(y.op, conv_same.ConvForward)
+    gy = rs.randn(*y.shape).astype(np.float32)
+    gx, gf = cgt.grad(y, [xn, fn], goutput=gy)
+    yv, gxv, gfv = y.get(), gx.get(), gf.get()
+    d = np.float64
+    # rows of the result against a float64 correlation of the rows they read
+    xp = np.pad(x[0].astype(d), ((0, 0), (1, 1), (1, 1)))
+    for h in (0, 700, 1448):
+        want = np.einsum("lcij,cijw->lw", f.astype(d),
+                         np.stack([np.stack([xp[:, h + i, j:j + 1449] for j in range(3)], 1) for i in range(3)], 1))
+        assert relfro(yv[0, :, h, :], want) <= TOL
+    lhs = float(np.vdot(yv.astype(d), gy.astype(d)))
+    assert abs(lhs - float(np.vdot(x.astype(d), gxv.astype(d)))) <= 1e-5 * abs(lhs)
+    assert abs(lhs - float(np.vdot(f.astype(d), gfv.astype(d)))) <= 1e-5 * abs(lhs)

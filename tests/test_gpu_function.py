@@ -191,21 +191,52 @@ def test_function_is_shape_generic(cgt):
         assert np.array_equal(g.get().view(np.uint32), node.get().view(np.uint32))
 
 
-def test_function_with_a_baked_extent_keeps_the_traced_shapes(cgt):
-    # mean() divides by a constant computed from the extents: such a function must refuse
-    # other shapes instead of dividing by the wrong count
+def test_extents_used_as_values_follow_the_call_shapes(cgt):
+    # the reference's cgt.size is a symbolic scalar, so sum(x) / size(x, 0), x * x.shape[1] and
+    # mean() are right at any shape (cgt/core.py:1614-1640); here an extent that depends on an
+    # argument enters a value through ExtentAsFloat, which a compiled function re-evaluates per call
+    from cgt_amd import core
     x0 = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
     xn = cgt.constant(x0)
-    f = cgt.function([xn], cgt.mean(xn * xn))
-    assert not f.shape_generic
-    assert abs(float(f(x0)) - (x0 * x0).mean()) <= 1e-4 * (x0 * x0).mean()
-    with pytest.raises(ValueError):
-        f(x0[:1])
-    # an extent of a weight (not an argument) is a constant: still generic in the argument
+
+    def graph(xn):
+        return [cgt.mean(xn * xn), cgt.sum(xn) / cgt.size(xn, 0), xn * xn.shape[1],
+                (cgt.size(xn, 0) * cgt.size(xn, 2) - 1) * cgt.sum(xn, axis=0), cgt.mean(xn, axis=(0, 2))]
+
+    f = cgt.function([xn], graph(xn))
+    assert f.shape_generic
+    assert any(isinstance(n.op, core.ExtentAsFloat) for n in f._order)
+    rs = np.random.RandomState(3)
+    for shape in [(2, 3, 4), (5, 3, 4), (1, 7, 2), (2, 3, 4)]:
+        xv = rs.randn(*shape).astype(np.float32)
+        got = f(xv)
+        want = graph(cgt.constant(xv))                    # node-by-node evaluation at this shape
+        ref = [np.mean(xv.astype(np.float64) ** 2), xv.sum(dtype=np.float64) / shape[0], xv * shape[1],
+               (shape[0] * shape[2] - 1) * xv.sum(axis=0, dtype=np.float64), xv.mean(axis=(0, 2), dtype=np.float64)]
+        for g, w, r in zip(got, want, ref):
+            assert np.array_equal(np.asarray(g).view(np.uint32), w.get().view(np.uint32)), shape
+            assert np.allclose(np.asarray(g), r, rtol=1e-5, atol=1e-5), shape
+    # an extent of a weight (not an argument) is a constant
     wn = cgt.constant(np.ones((3, 4), np.float32))
     g = cgt.function([xn], cgt.sum(xn * 2.0) * cgt.mean(wn))
     assert g.shape_generic
     assert abs(float(g(x0[:1])) - 2 * x0[:1].sum()) <= 1e-3
+
+
+def test_function_with_a_baked_extent_keeps_the_traced_shapes(cgt):
+    # a value computed outside the graph from an extent (a node flagged shape_baked) cannot follow
+    # the call's shapes: such a function refuses other shapes instead of using the wrong count
+    from cgt_amd import core
+    x0 = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
+    xn = cgt.constant(x0)
+    n = cgt.size(xn, 0) * cgt.size(xn, 1)
+    divisor = cgt.constant(np.float32(1.0 / n))
+    divisor.shape_baked, divisor.baked_expr = True, core.ShapeInt._lift(n).expr
+    f = cgt.function([xn], cgt.sum(xn) * divisor)
+    assert not f.shape_generic
+    assert abs(float(f(x0)) - x0.sum() / 6) <= 1e-4 * x0.sum()
+    with pytest.raises(ValueError):
+        f(x0[:1])
 
 
 def test_function_transports_follow_the_gpu_deref_mask(cgt):
@@ -369,3 +400,39 @@ def test_function_as_hip_graph_matches_eager_on_every_replay(cgt):
           % (t_plain, t_graph, plain.n_instructions))
     for a, b in zip(graph_dev(xg), plain_dev(xg)):
         assert np.array_equal(a.get(), b.get())
+
+
+def test_kept_device_outputs_survive_a_later_call_that_needs_larger_buffers(cgt):
+    # device_outputs=True hands out the interpreter's own buffers.  A later call at a larger shape
+    # makes the interpreter drop those buffers for larger ones; an output kept from the earlier
+    # call holds a reference on its buffer (a view holds one on the buffer it shows), so it still
+    # reads the values of its call
+    from cgt_amd import nn
+    rs = np.random.RandomState(12)
+    w = (rs.randn(16, 16, 3, 3) / 12).astype(np.float32)
+    wn = cgt.constant(w)
+
+    def graph(xn):
+        y = nn.conv2d(xn, wn, (3, 3), pad=(1, 1))
+        return [y, cgt.reshape(y * 2.0, [cgt.size(y, 0), cgt.size(y, 1) * cgt.size(y, 2) * cgt.size(y, 3)])]
+
+    x_small = rs.randn(2, 16, 9, 9).astype(np.float32)
+    xn = cgt.constant(x_small)
+    f = cgt.function([xn], graph(xn), device_outputs=True)
+    kept = f(x_small)
+    want = [g.get().copy() for g in kept]
+    ptr_small = kept[0].ptr
+    for batch in (5, 9, 33):                       # each call outgrows the buffers of the one before
+        big = f(rs.randn(batch, 16, 9, 9).astype(np.float32))
+        assert big[0].shape[0] == batch
+    assert big[0].ptr != ptr_small
+    # allocate and scribble: freed memory would be handed out again
+    from cgt_amd.gpuarray import to_gpu
+    junk = [to_gpu(np.full(want[0].shape, 7.0, np.float32)) for _ in range(8)]
+    for g, w_ in zip(kept, want):
+        assert np.array_equal(g.get().view(np.uint32), w_.view(np.uint32))
+    del junk, kept, big
+    # a smaller call after the growth is a view of the large buffer; keeping it keeps that buffer
+    small_again = f(x_small)
+    del f
+    assert np.array_equal(small_again[0].get().view(np.uint32), want[0].view(np.uint32))

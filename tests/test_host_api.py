@@ -99,7 +99,7 @@ def test_closure_struct_layouts():
 
 def test_prebuild_standard_ops_exports_call_symbols():
     built = compilation.prebuild_standard_ops()
-    assert len(built) == 33
+    assert len(built) == 34
     for c in built:
         assert c.fptr_address and c.return_type in ("byref", "byval") and c.kind == "native"
     assert [c.return_type for c in built].count("byval") == 2

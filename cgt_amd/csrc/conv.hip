@@ -92,6 +92,204 @@ __global__ __launch_bounds__(256) void flip_filters_kernel(const float* __restri
     }
 }
 
+// ---- weight gradient of a first layer with few filters (the CIFAR / MNIST first layers: 32
+// filters, patches of 75 and 9 floats).  The result is a few thousand floats and the reduction runs
+// over every output pixel of the batch, so as a GEMM it is one row tile by one to four column
+// tiles with an enormous K: the tiled product spends its time on prologues and partial tiles
+// (0.045 ms for 0.63 GFLOP).  Here it is a reduction: a workgroup takes (image, band of output
+// rows) units in turn, stages the band's cotangent [L][pixels] and the patch of the image under it
+// (zero-padded, all channels) in LDS, and its four wavefronts walk the band's pixels four at a
+// time, each accumulating the whole [32][32 * NB] result block with v_mfma_f32_32x32x2_f32:
+// A operand = cotangent (lane -> filter, k -> pixel), B operand = patch element (lane -> patch
+// index z, its (channel, row, column) offset fixed per lane; k -> pixel, whose tile offset comes
+// from a small table).  The four wavefronts' blocks are added in order 0..3, each workgroup
+// writes one partial result and the split-K reduce kernel adds those in order: deterministic.
+struct SmallWgrad {
+    const float* gy;      // [B][L][OH * OW]
+    const float* x;       // [B][C][H][W]
+    float* part;          // [workgroups][L][Z]
+    int B, C, H, W, L, OH, OW, Z, kh, kw, ph, pw, sh, sw;
+    int band_rows, bands, units;      // output rows per unit, units per image, B * bands
+    int rows_in, twp;                 // the image tile under a band: C x rows_in x twp floats
+    int pbpad;                        // floats between two filters' rows in the cotangent tile (even)
+    int vec4;                         // every row of every unit's cotangent tile is whole aligned 16-byte units
+    int off_x, off_pix;               // LDS offsets (floats) of the image tile and the pixel table
+};
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+template <int NB>
+__global__ __launch_bounds__(256) void wgrad_small_kernel(SmallWgrad a) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    float* gyt = lds;                                   // [32][pbpad]
+    float* xt = lds + a.off_x;                          // [C][rows_in][twp]
+    int* pixoff = reinterpret_cast<int*>(lds + a.off_pix);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, half = lane >> 5;
+    const int taps = a.kh * a.kw, P = a.OH * a.OW;
+    int offz[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int z = nb * 32 + l32;
+        offz[nb] = 0;                                   // columns past Z read valid LDS; they are never stored
+        if (z < a.Z) {
+            const int c = z / taps, r = z - c * taps, ho = r / a.kw, wo = r - ho * a.kw;
+            offz[nb] = (c * a.rows_in + ho) * a.twp + wo;
+        }
+    }
+    v16f acc[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[nb][e] = 0.0f;
+
+    for (int u = blockIdx.x; u < a.units; u += gridDim.x) {
+        const int b = u / a.bands, bd = u - b * a.bands;
+        const int r0 = bd * a.band_rows, r1 = min(a.OH, r0 + a.band_rows);
+        const int PB = (r1 - r0) * a.OW, PB4 = (PB + 3) & ~3;
+        // cotangent tile: filter l's pixels are contiguous in memory; wavefront w takes rows w, w + 4, ...
+        // (8 rows x up to 4 floats per lane, all loads issued before the first is parked; rows past L
+        // and pixels past PB are loaded from clamped addresses and parked as zeros)
+        const float* gsrc = a.gy + (long)b * a.L * P + (long)r0 * a.OW;
+        const int nx = a.C * a.rows_in * a.twp;
+        const float* xsrc = a.x + (long)b * a.C * a.H * a.W;
+        // image tile: input rows r0 * sh - ph ..., columns -pw ..., zero outside the image
+        auto stage_image = [&]() __attribute__((always_inline)) {
+            for (int i = threadIdx.x; i < nx; i += 256) {
+                const int c = i / (a.rows_in * a.twp), r = i - c * (a.rows_in * a.twp);
+                const int ri = r / a.twp, wi = r - ri * a.twp;
+                const int hh = r0 * a.sh - a.ph + ri, ww = wi - a.pw;
+                const bool in = hh >= 0 && hh < a.H && ww >= 0 && ww < a.W;
+                const float v = xsrc[((long)c * a.H + (in ? hh : 0)) * a.W + (in ? ww : 0)];
+                xt[i] = in ? v : 0.0f;
+            }
+            for (int p = threadIdx.x; p < PB4; p += 256) {
+                const int q = min(p, PB - 1);               // (pixels past PB carry a zero cotangent)
+                const int h = q / a.OW, w = q - h * a.OW;
+                pixoff[p] = h * a.sh * a.twp + w * a.sw;
+            }
+        };
+        if (a.vec4) {
+            // every filter's run of PB floats starts on a 16-byte boundary and is whole units: one
+            // 16-byte load per lane and row (PB <= 256), all eight rows in flight
+            float4 gv[8];
+            const int u = min(lane, PB / 4 - 1);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) gv[i] = *reinterpret_cast<const float4*>(gsrc + (long)min(wave + 4 * i, a.L - 1) * P + 4 * u);
+            stage_image();
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int l = wave + 4 * i;
+                if (4 * lane < PB4) {
+                    const float4 v = l < a.L ? gv[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+                    float2* d = reinterpret_cast<float2*>(gyt + l * a.pbpad + 4 * lane);
+                    d[0] = make_float2(v.x, v.y);
+                    d[1] = make_float2(v.z, v.w);
+                }
+            }
+        } else {
+            float gv[8][4];
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int l = min(wave + 4 * i, a.L - 1), p = min(lane + 64 * k, PB - 1);
+                    gv[i][k] = gsrc[(long)l * P + p];
+                }
+            stage_image();
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int l = wave + 4 * i, p = lane + 64 * k;
+                    if (p < PB4) gyt[l * a.pbpad + p] = (l < a.L && p < PB) ? gv[i][k] : 0.0f;
+                }
+        }
+        __syncthreads();
+        // lanes 0..31 carry pixels q, q + 1 of a quad, lanes 32..63 pixels q + 2, q + 3: the two
+        // MFMAs of a quad pair (q, q + 2) and (q + 1, q + 3) on the k axis, for both operands
+        for (int q = 4 * wave; q < PB4; q += 16) {
+            const int p_lo = q + 2 * half;
+            const float2 av = *reinterpret_cast<const float2*>(gyt + l32 * a.pbpad + p_lo);
+            const int2 po = *reinterpret_cast<const int2*>(pixoff + p_lo);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const float b0 = xt[offz[nb] + po.x], b1 = xt[offz[nb] + po.y];
+                acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, b0, acc[nb], 0, 0, 0);
+                acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, b1, acc[nb], 0, 0, 0);
+            }
+        }
+        __syncthreads();                                // the next unit's tiles go over these
+    }
+    // the four wavefronts' blocks, added in order; element e of a block: row 8 * (e / 4) + 4 * half + e % 4, column l32
+    float* red = lds;
+    for (int w = 0; w < 4; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int i = (nb * 16 + e) * 64 + lane;
+                    red[i] = w == 0 ? acc[nb][e] : red[i] + acc[nb][e];
+                }
+        }
+        __syncthreads();
+    }
+    float* out = a.part + (long)blockIdx.x * a.L * a.Z;
+    for (int i = threadIdx.x; i < NB * 1024; i += 256) {
+        const int nb = i >> 10, e = (i >> 6) & 15, ln = i & 63;
+        const int l = 8 * (e >> 2) + 4 * (ln >> 5) + (e & 3), z = nb * 32 + (ln & 31);
+        if (l < a.L && z < a.Z) out[l * a.Z + z] = red[i];
+    }
+}
+
+// 0 if the reduction kernel does not cover the layer (then the tiled product runs); else the plan
+static bool small_wgrad_plan(SmallWgrad& a, size_t& lds_bytes, int& grid, long B, long C, long H, long W, long L,
+                             const PatchGeom& pg) {
+    const long Z = C * pg.kh * pg.kw;
+    if (L < 1 || L > 32 || Z > 128 || pg.OW > 256 || B < 1 || B >= (1L << 24)) return false;
+    // bands of whole output rows, at most 256 pixels each; more, shorter bands while the chip has workgroups to spare
+    int band_rows = std::max(1, std::min(pg.OH, 256 / pg.OW));
+    int bands = (int)cdiv(pg.OH, band_rows);
+    band_rows = (int)cdiv(pg.OH, bands);
+    while (B * bands < 2 * kNumCU && band_rows > 1 && (band_rows / 2) * pg.OW >= 64) {
+        band_rows = (band_rows + 1) / 2;
+        bands = (int)cdiv(pg.OH, band_rows);
+    }
+    const int rows_in = (band_rows - 1) * pg.sh + pg.kh, twp = (pg.OW - 1) * pg.sw + pg.kw;
+    const long xt_floats = C * rows_in * twp;
+    if (xt_floats > 8192 || B * bands >= (1L << 30)) return false;
+    const int pb4 = (band_rows * pg.OW + 3) & ~3;
+    a.pbpad = pb4 + 2;        // even (8-byte reads and stores), and 2 mod 32 for the largest band: consecutive filters two banks apart
+    a.off_x = (32 * a.pbpad + 3) & ~3;
+    a.off_pix = (int)((a.off_x + xt_floats + 3) & ~3);
+    const long total = a.off_pix + pb4 + 4;
+    lds_bytes = (size_t)std::max(total, 4L * 1024) * sizeof(float);       // the cross-wavefront sum needs NB * 1024 floats
+    if (lds_bytes > 64 * 1024) return false;
+    a.B = (int)B; a.C = (int)C; a.H = (int)H; a.W = (int)W; a.L = (int)L; a.OH = pg.OH; a.OW = pg.OW; a.Z = (int)Z;
+    a.kh = pg.kh; a.kw = pg.kw; a.ph = pg.ph; a.pw = pg.pw; a.sh = pg.sh; a.sw = pg.sw;
+    a.band_rows = band_rows; a.bands = bands; a.units = (int)(B * bands);
+    a.rows_in = rows_in; a.twp = twp;
+    grid = (int)std::min((long)a.units, 4L * kNumCU);
+    return true;
+}
+
+static int small_wgrad(const SmallWgrad& plan, size_t lds_bytes, int grid, const float* gy, const float* x, float* gf, void* stream) {
+    SmallWgrad a = plan;
+    a.gy = gy; a.x = x;
+    // 16-byte loads of the cotangent: pixel runs that start and end on 16-byte boundaries in every unit
+    a.vec4 = (((long)a.OH * a.OW) % 4 == 0 && (a.band_rows * a.OW) % 4 == 0 && reinterpret_cast<uintptr_t>(gy) % 16 == 0) ? 1 : 0;
+    a.part = stream_workspace(stream, kWsConvData, (size_t)grid * a.L * a.Z * sizeof(float), "conv_patch_bwd_filter");
+    if (!a.part) return CGT_AMD_ERR_NOMEM;
+    hipStream_t st = as_stream(stream);
+    const int nb = (a.Z + 31) / 32;
+    if (nb == 1) wgrad_small_kernel<1><<<dim3((unsigned)grid), dim3(256), lds_bytes, st>>>(a);
+    else if (nb == 2) wgrad_small_kernel<2><<<dim3((unsigned)grid), dim3(256), lds_bytes, st>>>(a);
+    else if (nb == 3) wgrad_small_kernel<3><<<dim3((unsigned)grid), dim3(256), lds_bytes, st>>>(a);
+    else wgrad_small_kernel<4><<<dim3((unsigned)grid), dim3(256), lds_bytes, st>>>(a);
+    CGT_LAUNCH_CHECK("wgrad_small_kernel");
+    return reduce_partials(a.part, gf, (long)a.L * a.Z, grid, stream);
+}
+
 static int check_same(const char* what, SameGeom& g, long B, long C, long H, long W, long L, int kh, int kw) {
     CGT_ARG_CHECK(B >= 0 && C > 0 && H > 0 && W > 0 && L > 0, "%s: bad shape", what);
     CGT_ARG_CHECK(make_geom(g, B, C, H, W, L, kh, kw), "%s: the kernel must be odd x odd (pad = (kernel - 1) / 2)", what);
@@ -379,6 +577,12 @@ CGT_API int cgt_amd_conv_patch_bwd_filter_f32(const float* gy, const float* x, l
     CGT_ARG_CHECK(gf, "conv_patch_bwd_filter: null pointer");
     if (B == 0) return cgt_amd_fill_u32(gf, 0u, L * Z, stream);
     CGT_ARG_CHECK(gy && x, "conv_patch_bwd_filter: null pointer");
+    {
+        SmallWgrad plan;
+        size_t lds_bytes = 0;
+        int grid = 0;
+        if (small_wgrad_plan(plan, lds_bytes, grid, B, C, H, W, L, pg)) return small_wgrad(plan, lds_bytes, grid, gy, x, gf, stream);
+    }
     return wgrad_in_groups(B, P, Z, L, gf, stream, "conv_patch_bwd_filter", [&](long b0, long nb, float* out) {
         PatchGeom part = pg;
         part.x = x + b0 * C * H * W;

@@ -1124,10 +1124,47 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     }
 }
 
-// out[i] = ws[0][i] + ws[1][i] + ... + ws[n - 1][i] for i < count, added in that order (the split-K
-// reduce kernel on a caller's partial results: the weight gradient of a very large batch sums
-// per-group results with it).
+// Many partial results of a small array (hundreds of [32][75] blocks): the kernel above would put
+// all of it on a dozen workgroups whose four wavefronts each walk a quarter of the partials, one
+// long chain of load latencies (13 us for 512 x 2400 floats).  Here a workgroup of 16 wavefronts
+// owns 64 outputs; wavefront g adds partials [g * per, (g + 1) * per) in order, 8 loads in flight,
+// and the 16 sums are added in order: the same fixed order on every run.
+__global__ __launch_bounds__(1024) void reduce_many_kernel(const float* __restrict__ ws, float* __restrict__ out,
+                                                           long count, int n) {
+    __shared__ float part[16][64];
+    const int col = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const long i = (long)blockIdx.x * 64 + col;
+    const int per = (n + 15) / 16;
+    const int s0 = g * per, s1 = min(n, s0 + per);
+    float acc = 0.0f;
+    if (i < count) {
+        for (int sb = s0; sb < s1; sb += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = ws[(long)min(sb + u, s1 - 1) * count + i];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (sb + u < s1) acc += v[u];
+        }
+    }
+    part[g][col] = acc;
+    __syncthreads();
+    if (g != 0 || i >= count) return;
+    float tot = part[0][col];
+#pragma unroll
+    for (int k = 1; k < 16; ++k) tot += part[k][col];
+    out[i] = tot;
+}
+
+// out[i] = ws[0][i] + ws[1][i] + ... + ws[n - 1][i] for i < count, added in a fixed order (groups of
+// consecutive partials, then the group sums): the weight gradient of a very large batch sums
+// per-group results with it, the reduction-shaped weight gradient its workgroups' results.
 int reduce_partials(const float* ws, float* out, long count, int n, void* stream) {
+    if (n >= 64 && count <= (1L << 16)) {
+        reduce_many_kernel<<<dim3((unsigned)cdiv(count, 64L)), dim3(1024), 0, as_stream(stream)>>>(ws, out, count, n);
+        CGT_LAUNCH_CHECK("reduce_many_kernel");
+        return CGT_AMD_OK;
+    }
     const bool vec = count % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && reinterpret_cast<uintptr_t>(ws) % 16 == 0;
     const long blocks = cdiv(count, vec ? 256L : 64L);
     CGT_ARG_CHECK(blocks < (1L << 31), "reduce_partials: too many elements");
@@ -1507,7 +1544,10 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     else if (conv_kernel) launch_conv(cv->mode, shape, grid, st, a);
     else launch_trans(tA, tB, pipe, deep, shape, grid, st, a);
     CGT_LAUNCH_CHECK("sgemm_kernel");
-    if (a.splits > 1) {
+    if (a.splits >= 64 && M * N <= (1L << 16) && ldc == N) {
+        int rc = reduce_partials(a.ws, C, M * N, a.splits, stream);      // hundreds of partials of a small result
+        if (rc) return rc;
+    } else if (a.splits > 1) {
         const long MN = M * N;
         const bool vec = N % 4 == 0 && ldc % 4 == 0 && aligned16(C) && aligned16(a.ws);
         const long blocks = cdiv(MN, vec ? 256L : 64L);

@@ -42,6 +42,14 @@ CASES = [
     (5, 3, 20, 17, 33, (4, 6), (3, 5), (3, 2)),         # padding wider than half the kernel, patches hanging over every edge
     (2, 6, 40, 40, 200, (7, 7), (3, 3), (2, 2)),
     (10, 2, 63, 57, 100, (10, 11), (9, 9), (2, 2)),     # the two weight-gradient variants pick different tile shapes
+    # few filters and short patches: the gathered weight gradient is the reduction kernel (bands of output
+    # rows staged in LDS) -- bands that do not divide the rows, 17 filters, patches of exactly 128, a
+    # stride, more (image, band) units than workgroups, rows too wide for it (the tiled product again)
+    (3, 3, 33, 70, 32, (5, 5), (2, 2), (1, 1)),
+    (5, 2, 31, 29, 17, (8, 8), (3, 3), (2, 2)),
+    (1300, 1, 6, 6, 8, (3, 3), (1, 1), (1, 1)),
+    (2, 1, 9, 300, 32, (3, 3), (1, 1), (1, 1)),
+    (4, 3, 24, 24, 1, (3, 5), (0, 2), (1, 3)),
 ]
 
 

@@ -323,3 +323,17 @@ def test_vgg_layer_full_size_through_the_fused_ops(K):
     lhs = float(np.vdot(y.astype(d), gy.astype(d)))
     assert abs(lhs - float(np.vdot(x.astype(d), gx.astype(d)))) <= 1e-5 * abs(lhs)
     assert abs(lhs - float(np.vdot(f.astype(d), gf.astype(d)))) <= 1e-5 * abs(lhs)
+    # the weight gradient itself: sampled (channel, tap) columns over all filters and the whole batch
+    # against float64 -- gf[l, c, ho, wo] = sum over (b, h, w) of gy[b, l, h, w] * x[b, c, h + ho - 1, w + wo - 1];
+    # every tap, first / last / interior channels of the blocks of 16 the product walks
+    gy64 = gy.astype(d)
+    xp = np.pad(x, ((0, 0), (0, 0), (1, 1), (1, 1)))
+    samples = [(c, ho, wo) for c in (0, 15, 16, 77, 127) for ho in range(3) for wo in range(3)][::2]
+    got = np.stack([gf[:, c, ho, wo] for c, ho, wo in samples], 1)
+    want = np.stack([np.einsum("blhw,bhw->l", gy64, xp[:, c, ho:ho + H, wo:wo + W].astype(d)) for c, ho, wo in samples], 1)
+    assert relfro(got, want) <= TOL
+    assert np.max(np.abs(got - want)) <= 1e-4 * np.max(np.abs(want))
+    # the same launches again: same bits (split-K partial sums are reduced in a fixed order)
+    assert np.array_equal(K.conv_same_bwd_filter(gypad, xpad, x.shape, f.shape).get().view(np.uint32), gf.view(np.uint32))
+    assert np.array_equal(K.conv_same_fwd(xpad, fg, x.shape).get().view(np.uint32), y.view(np.uint32))
+    assert np.array_equal(K.conv_same_bwd_data(gypad, fg, x.shape).get().view(np.uint32), gx.view(np.uint32))

@@ -356,3 +356,31 @@ def test_conv2d_fwd_bwd_equals_torch(k, p, s):
     gx, gf = O.conv2d_pullback(x, f, gy, p, s)
     np.testing.assert_allclose(gx, xt.grad.numpy(), rtol=1e-10, atol=1e-10)
     np.testing.assert_allclose(gf, ft.grad.numpy(), rtol=1e-10, atol=1e-10)
+
+
+@pytest.mark.parametrize("shape,kernel", [((2, 3, 5, 7), (3, 3)), ((1, 2, 4, 9), (5, 3)), ((3, 1, 6, 6), (1, 7)), ((1, 1, 1, 1), (3, 5))])
+def test_padded_plane_layout_puts_every_tap_at_a_plain_offset(shape, kernel):
+    # the layout the column-buffer-free products read (no reference counterpart): tap (ho, wo) of the
+    # padded-grid pixel q = h * Wp + w must be the float at q + ho * Wp + wo of its plane, equal to
+    # x[h + ho - ph, w + wo - pw] or zero outside the image -- checked against numpy's own padding
+    from cgt_amd import capi
+    B, C, H, W = shape
+    kh, kw = kernel
+    ph, pw = (kh - 1) // 2, (kw - 1) // 2
+    rs = np.random.RandomState(kh * 10 + W)
+    x = rs.randn(*shape).astype(np.float32)
+    total = capi.lib().cgt_amd_conv_same_padded_size(B * C, H, W, kh, kw)
+    flat = O.conv_same_padded(x, kernel, total)
+    Wp = W + pw
+    plane = (total - (256 + kh * Wp + 3) // 4 * 4) // (B * C)
+    assert plane * B * C + (256 + kh * Wp + 3) // 4 * 4 == total and plane % 16 == 0
+    ref = np.pad(x.reshape(B * C, H, W), ((0, 0), (ph, ph), (pw, pw)))
+    planes = np.concatenate([flat, np.zeros(kh * Wp + kw, np.float32)])      # reads of the last plane's taps run into the tail
+    for p in range(B * C):
+        for ho in range(kh):
+            for wo in range(kw):
+                for h in range(H):
+                    got = planes[p * plane + h * Wp + ho * Wp + wo: p * plane + h * Wp + ho * Wp + wo + W]
+                    assert np.array_equal(got, ref[p, h + ho, wo:wo + W]), (p, ho, wo, h)
+    # everything that is not a pixel is zero, and every pixel appears exactly once
+    assert np.count_nonzero(flat) == np.count_nonzero(x) and abs(float(flat.sum(dtype=np.float64)) - float(x.sum(dtype=np.float64))) < 1e-3

@@ -334,7 +334,19 @@ __global__ __launch_bounds__(kSumThreads) void sum_finish_kernel(const float* __
                                                                  long P, long stride_k, long stride_p) {
     const long k = blockIdx.x;
     float acc = 0.0f;
-    for (long p = threadIdx.x; p < P; p += kSumThreads) acc += ws[k * stride_k + p * stride_p];
+    // eight loads in flight per lane (clamped, unconditional), added in ascending p as before:
+    // thousands of partials of a large sum are otherwise one chain of load latencies
+    for (long p = threadIdx.x; p < P; p += kSumThreads * 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const long q = p + (long)u * kSumThreads;
+            v[u] = ws[k * stride_k + (q < P ? q : P - 1) * stride_p];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (p + (long)u * kSumThreads < P) acc += v[u];
+    }
     const float total = block_sum(acc);
     if (threadIdx.x == 0) out[k] = total;
 }

@@ -213,3 +213,33 @@ def test_stream_copy_any_alignment_and_size(L, loads_in_flight):
         assert L.cgt_amd_stream_copy_tune(5000, 8) == ERR_ARG and L.cgt_amd_stream_copy_tune(8192, 3) == ERR_ARG
     finally:
         assert L.cgt_amd_stream_copy_tune(16384, 4) == OK
+
+
+@pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_tiles_loaded_straight_into_lds_match_the_register_path(L, tA, tB):
+    # Whole tiles reach LDS through global_load_lds_dwordx4, whose LDS base travels in m0 and is set
+    # from inline asm (the compiler is not told: it reserves m0 and refuses it in a clobber list).
+    # If a toolchain ever kept a value of its own in m0 across that asm, or scheduled around it, the
+    # direct loads would land in the wrong place -- in whole tiles only.  Edge tiles take the
+    # register path (ordinary loads + ds_write), which does not touch m0: the same product with one
+    # row / column fewer computes the same dot products in the same order, so its rows and columns
+    # must have the bits of the whole-tile product.  Several K so that the pipelined loop (both
+    # operands k-contiguous, many tiles), the plain loop and a ragged last slice are all covered.
+    rs = np.random.RandomState(31)
+    for M, N, K in [(256, 256, 256), (384, 1664, 96), (256, 128, 363)]:
+        A = rs.uniform(-1, 1, (K, M) if tA else (M, K)).astype(np.float32)
+        B = rs.uniform(-1, 1, (N, K) if tB else (K, N)).astype(np.float32)
+
+        def product(m, n):
+            a = np.ascontiguousarray(A[:, :m] if tA else A[:m])
+            b = np.ascontiguousarray(B[:n] if tB else B[:, :n])
+            ga, gb, gc = gpu(a), gpu(b), gpu(np.full((m, n), np.nan, np.float32))
+            assert L.cgt_amd_sgemm(tA, tB, m, n, K, ga.ptr, a.shape[1], gb.ptr, b.shape[1], gc.ptr, n, None) == OK, _err(L)
+            return gc.get()
+
+        whole = product(M, N)
+        ref = (A.T if tA else A).astype(np.float64) @ (B.T if tB else B).astype(np.float64)
+        assert np.linalg.norm(whole - ref) <= 1e-5 * np.linalg.norm(ref)
+        fewer_rows, fewer_cols = product(M - 1, N), product(M, N - 1)
+        assert np.array_equal(fewer_rows.view(np.uint32), whole[:M - 1].view(np.uint32)), (tA, tB, M, N, K)
+        assert np.array_equal(fewer_cols.view(np.uint32), whole[:, :N - 1].view(np.uint32)), (tA, tB, M, N, K)

@@ -162,9 +162,11 @@ __global__ __launch_bounds__(kElwThreads) void elwise_binary_kernel(const TX* __
         for (long k = i; k < n; ++k) z[k] = F::apply((P)x[xs ? 0 : k], (P)y[ys ? 0 : k]);
 }
 
+// One trip per workgroup up to 4 M workgroups: many short-lived workgroups stream faster on this chip
+// than a resident-sized grid striding through the array (1 GiB add: 5.5-5.6 TB/s against 5.05).
 static unsigned elw_grid(long n) {
     const long per_block = (long)kElwThreads * kElwPerThread;
-    return (unsigned)std::max(1L, std::min(cdiv(n, per_block), 16L * kNumCU));
+    return (unsigned)std::max(1L, std::min(cdiv(n, per_block), 1L << 22));
 }
 
 static bool aligned_to(const void* p, int a) { return reinterpret_cast<uintptr_t>(p) % a == 0; }

@@ -1,6 +1,7 @@
 // Runtime entry points: device memory for cgtGPU arrays, copies, streams,
 // events, error reporting.
 #include "common.h"
+#include <algorithm>
 #include <cstring>
 #include <mutex>
 #include <unordered_map>
@@ -162,10 +163,21 @@ int launch_stream_copy(void* dest, const void* src, long nbytes, void* stream) {
     return CGT_AMD_OK;
 }
 
-__global__ void fill_u32_kernel(unsigned int* __restrict__ dst, unsigned int v, long n) {
-    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    long stride = (long)gridDim.x * blockDim.x;
-    for (; i < n; i += stride) dst[i] = v;
+// A workgroup fills 4096 words: the words before the first 16-byte boundary and after the last one
+// singly (first workgroup), the rest as aligned 16-byte units, four per thread.
+__global__ __launch_bounds__(256) void fill_u32_kernel(unsigned int* __restrict__ dst, unsigned int v, long n, long head, long units) {
+    v4u* body = reinterpret_cast<v4u*>(dst + head);
+    const v4u q = {v, v, v, v};
+    const long u0 = (long)blockIdx.x * 1024 + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const long u = u0 + k * 256;
+        if (u < units) body[u] = q;
+    }
+    if (blockIdx.x == 0) {
+        for (long i = threadIdx.x; i < head; i += 256) dst[i] = v;
+        for (long i = head + 4 * units + threadIdx.x; i < n; i += 256) dst[i] = v;
+    }
 }
 
 }  // namespace cgt_amd
@@ -286,10 +298,14 @@ CGT_API int cgt_amd_fill_u32(void* dst, unsigned int value, long count, void* st
     CGT_ARG_CHECK(count >= 0, "fill: negative count");
     if (count == 0) return CGT_AMD_OK;
     CGT_ARG_CHECK(dst, "fill: null pointer");
-    long blocks = cdiv(count, 256);
-    if (blocks > 4096) blocks = 4096;
+    CGT_ARG_CHECK(reinterpret_cast<uintptr_t>(dst) % 4 == 0, "fill: the destination must be 4-byte aligned");
+    long head = (long)((16 - (reinterpret_cast<uintptr_t>(dst) & 15)) & 15) / 4;
+    if (head > count) head = count;
+    const long units = (count - head) / 4;
+    const long blocks = std::max(1L, cdiv(units, 1024L));
+    CGT_ARG_CHECK(blocks < (1L << 31), "fill: too many words");
     fill_u32_kernel<<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(
-        static_cast<unsigned int*>(dst), value, count);
+        static_cast<unsigned int*>(dst), value, count, head, units);
     CGT_LAUNCH_CHECK("fill_u32");
     return CGT_AMD_OK;
 }

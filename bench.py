@@ -991,7 +991,9 @@ def _clock_frac(row):
 def _summary(res):
     """One short row per workload: whole-step value, its slowest GEMM launch as fraction of the
     fp32 MFMA peak, the HBM-bound stage furthest from 8 TB/s, and the gate's verdict."""
-    hbm = [(r["stage"], _clock_frac(r)) for r in res["stages"] if r["bound"] == "hbm" and _clock_frac(r) is not None]
+    # (stages that move less than 4 MB -- the filter permutes -- are launches, not bandwidth figures)
+    hbm = [(r["stage"], _clock_frac(r)) for r in res["stages"]
+           if r["bound"] == "hbm" and _clock_frac(r) is not None and r.get("bytes", 0) >= 4e6]
     row = {"value": res["value"], "ms_per_step": res["ms_per_step"], "gemm_frac": res["roofline"]["frac"],
            "parity_ok": res["parity"]["ok"]}
     if hbm:

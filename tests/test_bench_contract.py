@@ -75,7 +75,7 @@ def test_compact_line_stays_short_whatever_the_detail_holds():
     # the stdout line is built from the detail by dropping, never by cutting: a detail far larger
     # than any real one still gives a line a tail capture holds, with the contract fields intact
     import bench
-    stage = {"stage": "s" * 30, "bound": "hbm", "ms_in_step": 0.1234, "frac_in_step": 0.5678}
+    stage = {"stage": "s" * 30, "bound": "hbm", "ms_in_step": 0.1234, "frac_in_step": 0.5678, "bytes": 10 ** 8}
     gemm = {"stage": "gemm_fwd", "bound": "mfma", "ms_in_step": 0.4, "frac_in_step": 0.85}
     roof = {"bound": "mfma", "achieved": 130.0, "peak": 157.3, "unit": "TFLOP/s", "frac": 0.8264, "traffic": 3 * 10 ** 8,
             "kernel": "sgemm_kernel", "stage": "gemm_fwd", "flops_per_launch": 59190000000, "avg_launch_ms": 0.45,

@@ -23,6 +23,7 @@ PROTOTYPES = {
     "cgt_amd_last_error": (c_char_p, []),
     "cgt_amd_device_count": (c_int, []),
     "cgt_amd_device_name": (c_int, [c_char_p, c_int]),
+    "cgt_amd_mem_info": (c_int, [ctypes.POINTER(c_long), ctypes.POINTER(c_long)]),
     "cgt_amd_alloc": (c_void_p, [c_long]),
     "cgt_amd_free": (c_int, [c_void_p]),
     "cgt_amd_memcpy": (c_int, [c_int, c_int, c_void_p, c_void_p, c_long]),

@@ -208,6 +208,15 @@ CGT_API int cgt_amd_device_name(char* buf, int buflen) {
     return CGT_AMD_OK;
 }
 
+CGT_API int cgt_amd_mem_info(long* free_bytes, long* total_bytes) {
+    CGT_ARG_CHECK(free_bytes && total_bytes, "mem_info: null pointer");
+    size_t f = 0, t = 0;
+    CGT_HIP_TRY(hipMemGetInfo(&f, &t));
+    *free_bytes = (long)f;
+    *total_bytes = (long)t;
+    return CGT_AMD_OK;
+}
+
 CGT_API void* cgt_amd_alloc(long nbytes) {
     if (nbytes < 0) {
         set_error("alloc: negative size %ld", nbytes);

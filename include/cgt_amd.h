@@ -58,6 +58,11 @@ int cgt_amd_device_name(char *buf, int buflen);
 void *cgt_amd_alloc(long nbytes);
 int cgt_amd_free(void *ptr);
 
+/* Free and total device memory of the current device in bytes (no counterpart in
+ * the reference; lets a host size its batches and lets the tests watch the
+ * library's workspaces). */
+int cgt_amd_mem_info(long *free_bytes, long *total_bytes);
+
 /* Synchronous copy between host and device memory.  Replaces the cudaMemcpy
  * branch of cgt_memcpy (src/cgt_common.cpp:138-153). */
 int cgt_amd_memcpy(int dest_devtype, int src_devtype, void *dest, const void *src, long nbytes);

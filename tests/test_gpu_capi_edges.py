@@ -243,3 +243,32 @@ def test_tiles_loaded_straight_into_lds_match_the_register_path(L, tA, tB):
         fewer_rows, fewer_cols = product(M - 1, N), product(M, N - 1)
         assert np.array_equal(fewer_rows.view(np.uint32), whole[:M - 1].view(np.uint32)), (tA, tB, M, N, K)
         assert np.array_equal(fewer_cols.view(np.uint32), whole[:, :N - 1].view(np.uint32)), (tA, tB, M, N, K)
+
+
+def test_workspaces_of_rising_sizes_do_not_pile_up(L):
+    # split-K products whose partial sums grow call by call (a shape-generic function fed rising batch
+    # sizes): the stream's workspace grows geometrically and blocks it has outgrown are freed at the
+    # next synchronize -- the memory held afterwards is about the largest workspace, not the sum of all
+    from cgt_amd import capi
+    def free_bytes():
+        f, t = ctypes.c_long(), ctypes.c_long()
+        assert L.cgt_amd_mem_info(ctypes.byref(f), ctypes.byref(t)) == OK
+        return f.value
+    s = capi.Stream()
+    K = 64 * 1024
+    sizes = [64 + 16 * i for i in range(24)]              # M = N: 64 .. 432, 112 splits each -> 1.8 .. 84 MB of partials
+    a = gpu(np.ones((max(sizes), K), np.float32))
+    b = gpu(np.ones((max(sizes), K), np.float32))
+    c = gpu(np.zeros((max(sizes), max(sizes)), np.float32))
+    L.cgt_amd_synchronize(None)
+    before = free_bytes()
+    total_asked = 0
+    for m in sizes:
+        assert L.cgt_amd_sgemm(0, 1, m, m, K, a.ptr, K, b.ptr, K, c.ptr, m, s.handle) == OK, _err(L)
+        total_asked += m * m * 4 * 64
+    assert L.cgt_amd_synchronize(s.handle) == OK
+    held = before - free_bytes()
+    assert np.array_equal(c.get().reshape(-1)[:sizes[-1] ** 2], np.full(sizes[-1] ** 2, K, np.float32))
+    largest = sizes[-1] ** 2 * 4 * 256        # an upper bound on one call's workspace (<= 256 MiB cap)
+    assert held <= min(2 * largest, 600 << 20), (held, largest, total_asked)
+    del s

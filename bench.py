@@ -169,7 +169,7 @@ class Stage(object):
         # HBM stages whose op moves fewer arrays than the reference's algorithm does (`work` is what
         # the op as built has to move): the reference algorithm's bytes, the unit its figures are quoted in
         self.ref_bytes = ref_bytes
-        self.ms = self.ms_median = self.ms_min = self.ms_in_step = None
+        self.ms = self.ms_median = self.ms_min = self.ms_in_step = self.ms_copy_in_step = None
 
 
 class LayerOnGpu(object):
@@ -467,6 +467,35 @@ class LayerOnGpu(object):
         capi.synchronize()
         for i, st in enumerate(self.stages):
             st.ms_in_step = sum(ev[k][i].elapsed_ms(ev[k][i + 1]) for k in range(steps)) / steps
+
+    def time_copy_in_step(self, steps, min_bytes=4e6):
+        """The yardstick for the HBM-bound stages: each one in turn is replaced by this library's
+        streaming copy moving the same number of bytes (half read, half written, between two
+        scratch arrays) and that copy is timed where the stage runs, with the same kernels in
+        front of it and behind it.  -> st.ms_copy_in_step"""
+        from cgt_amd import capi
+        from cgt_amd.gpuarray import empty
+        if self.overlap:
+            return
+        todo = [st for st in self.stages if st.bound == "hbm" and st.work >= min_bytes]
+        if not todo:
+            return
+        half = max(st.work for st in todo) // 2 // 16 * 16
+        src, dst = empty((half // 4,)), empty((half // 4,))
+        self.K.fill(1.0, src.shape, out=src, stream=self.stream)
+        lib, keep = capi.lib(), [st.ms_in_step for st in self.stages]
+        for st in todo:
+            nbytes = st.work // 2 // 16 * 16
+            fn, st.fn = st.fn, (lambda nbytes=nbytes: capi.check(lib.cgt_amd_stream_copy(dst.ptr, src.ptr, nbytes, self.stream)))
+            try:
+                self.time_stages_in_step(steps)
+                st.ms_copy_in_step = st.ms_in_step
+            finally:
+                st.fn = fn
+        for st, ms in zip(self.stages, keep):
+            st.ms_in_step = ms
+        self.step()         # every buffer holds a real step's values again
+        capi.synchronize()
 
     def time_stages(self, reps):
         from cgt_amd import capi
@@ -801,6 +830,8 @@ def measure(workload, args, primary):
         layer.time_stages(max(stage_reps, 1))
     if not is_gemm:
         layer.time_stages_in_step(in_step_steps)
+        if not args.no_copy_yardstick:
+            layer.time_copy_in_step(in_step_steps)
 
     def clock(st):          # the stage's duration for the roofline: inside the step where measured
         t = getattr(st, "ms_in_step", None)
@@ -822,6 +853,11 @@ def measure(workload, args, primary):
             rate = st.work / (st.ms_in_step * 1e-3) / scale
             row.update({"ms_in_step": round(st.ms_in_step, 4), unit + "_in_step": round(rate, 2),
                         "frac_in_step": round(rate / peak, 4)})
+        if getattr(st, "ms_copy_in_step", None) is not None and getattr(st, "ms_in_step", None):
+            # the same bytes moved by the plain streaming copy at this place in the step
+            row.update({"ms_copy_same_bytes_in_step": round(st.ms_copy_in_step, 4),
+                        "frac_copy_same_bytes_in_step": round(st.work / (st.ms_copy_in_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                        "vs_copy_in_step": round(st.ms_copy_in_step / st.ms_in_step, 3)})
         if st.bound == "hbm" and getattr(st, "ref_bytes", None):
             row.update({"bytes_reference_algorithm": st.ref_bytes,
                         "GBps_in_reference_bytes": round(st.ref_bytes / (clock(st) * 1e-3) / 1e9, 1)})
@@ -906,6 +942,8 @@ def main():
                     help="also time the conv-layer glue kernels (bias add, ReLU, their gradients, loss sum) on the "
                          "layer's activation; they appear in `glue_stages`, outside the step")
     ap.add_argument("--no-op-api", action="store_true", help="skip timing the same step through the Op API")
+    ap.add_argument("--no-copy-yardstick", action="store_true",
+                    help="skip timing a plain copy of the same bytes in place of each HBM-bound stage")
     ap.add_argument("--no-check", action="store_true",
                     help="skip the parity gate (profiling runs: keeps its small launches out of the kernel statistics)")
     ap.add_argument("--conv-algo", default="auto", choices=["auto", "patch", "col", "im2col"],
@@ -992,13 +1030,14 @@ def _summary(res):
     """One short row per workload: whole-step value, its slowest GEMM launch as fraction of the
     fp32 MFMA peak, the HBM-bound stage furthest from 8 TB/s, and the gate's verdict."""
     # (stages that move less than 4 MB -- the filter permutes -- are launches, not bandwidth figures)
-    hbm = [(r["stage"], _clock_frac(r)) for r in res["stages"]
+    hbm = [(r["stage"], _clock_frac(r), r.get("vs_copy_in_step")) for r in res["stages"]
            if r["bound"] == "hbm" and _clock_frac(r) is not None and r.get("bytes", 0) >= 4e6]
     row = {"value": res["value"], "ms_per_step": res["ms_per_step"], "gemm_frac": res["roofline"]["frac"],
            "parity_ok": res["parity"]["ok"]}
     if hbm:
         best, worst = max(hbm, key=lambda t: t[1]), min(hbm, key=lambda t: t[1])
-        row["hbm_best"], row["hbm_worst"] = [best[0], round(best[1], 3)], [worst[0], round(worst[1], 3)]
+        # [stage, fraction of 8 TB/s, fraction of what a plain copy of the same bytes reaches there]
+        row["hbm_best"], row["hbm_worst"] = ([t[0], round(t[1], 3)] + ([t[2]] if t[2] is not None else []) for t in (best, worst))
     return row
 
 
@@ -1024,7 +1063,9 @@ def compact_line(out):
         if k in par:
             line["parity"][k] = par[k]
     # stage -> [ms inside the step, fraction of its roof (8 TB/s or 157.3 TFLOP/s)]
-    line["stages"] = {r["stage"]: [r.get("ms_in_step", r.get("ms")), _clock_frac(r)] for r in out["stages"]}
+    # (HBM stages: and the time of a plain copy of the same bytes at that place in the step / the stage's time)
+    line["stages"] = {r["stage"]: [r.get("ms_in_step", r.get("ms")), _clock_frac(r)] +
+                      ([r["vs_copy_in_step"]] if "vs_copy_in_step" in r else []) for r in out["stages"]}
     if "op_api_step" in out:
         line["op_api_step"] = {k: out["op_api_step"][k] for k in ("ms_per_step", "TFLOPs")}
     if "hbm_reference" in out:      # fraction of 8 TB/s that plain streaming kernels reach in this run

@@ -75,7 +75,8 @@ def test_compact_line_stays_short_whatever_the_detail_holds():
     # the stdout line is built from the detail by dropping, never by cutting: a detail far larger
     # than any real one still gives a line a tail capture holds, with the contract fields intact
     import bench
-    stage = {"stage": "s" * 30, "bound": "hbm", "ms_in_step": 0.1234, "frac_in_step": 0.5678, "bytes": 10 ** 8}
+    stage = {"stage": "s" * 30, "bound": "hbm", "ms_in_step": 0.1234, "frac_in_step": 0.5678, "bytes": 10 ** 8,
+             "vs_copy_in_step": 0.987}
     gemm = {"stage": "gemm_fwd", "bound": "mfma", "ms_in_step": 0.4, "frac_in_step": 0.85}
     roof = {"bound": "mfma", "achieved": 130.0, "peak": 157.3, "unit": "TFLOP/s", "frac": 0.8264, "traffic": 3 * 10 ** 8,
             "kernel": "sgemm_kernel", "stage": "gemm_fwd", "flops_per_launch": 59190000000, "avg_launch_ms": 0.45,
@@ -103,6 +104,7 @@ def test_compact_line_stays_short_whatever_the_detail_holds():
     back = bench.compact_line(out)
     assert set(back["workloads"]) == set(out["workloads"]) and "stages" in back and "hbm_reference" in back
     assert back["workloads"]["workload_0"]["hbm_worst"][0].startswith("stage_")
+    assert back["workloads"]["workload_0"]["hbm_worst"][1:] == [0.568, 0.987] and back["stages"]["stage_0"] == [0.1234, 0.5678, 0.987]
     assert len(json.dumps(back, separators=(",", ":"))) <= bench.MAX_LINE
 
 
@@ -181,6 +183,10 @@ def test_default_workload_prints_the_contract_line():
         assert len(gemms) == 3 and all(r["roof"] in ("hbm", "mfma") and r["frac_hbm"] > 0 and r["frac_in_step"] > 0 for r in gemms)
         assert [r["roof"] for r in gemms if r["stage"] == "gemm_dgrad"] == ["hbm"]
     assert all("vs_measured_copy" in r for r in full["stages"] if r["bound"] == "hbm")
+    # ... and against a plain copy of the same bytes timed in the stage's place inside the step
+    big = [r for r in full["stages"] if r["bound"] == "hbm" and r["bytes"] >= 4e6]
+    assert big and all(0.5 < r["vs_copy_in_step"] < 1.5 and r["ms_copy_same_bytes_in_step"] > 0 for r in big)
+    assert all(len(out["stages"][r["stage"]]) == 3 for r in big)
     assert full["cpu_baseline"]["stages"]
 
 
@@ -192,6 +198,6 @@ def test_in_step_clock_alone():
     assert proc.returncode == 0, proc.stderr[-2000:]
     out = json.loads([ln for ln in proc.stdout.splitlines() if ln.strip()][0])
     assert out["roofline"]["achieved"] > 0 and "inside" in out["roofline"]["timing"]
-    assert all(ms > 0 for ms, _frac in out["stages"].values())
+    assert all(v[0] > 0 for v in out["stages"].values())
     for row in _detail(proc)["stages"]:
         assert row["ms_in_step"] > 0 and "ms" not in row

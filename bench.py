@@ -695,7 +695,22 @@ def check_layer_against_oracle(cfg, algo):
             "rel_fro": {k: float("%.2e" % v) for k, v in err.items()}}
 
 
-def op_api_step_ms(cfg, steps, warmup):
+def settle_clock(step, settle_ms):
+    """Untimed steps until the device has been under load for settle_ms milliseconds.  After an
+    idle stretch (the host-side parity gate, compilation) the power manager takes about 25 ms of
+    load to reach the clock it then sustains: the first step runs 14 % slower than the sixteenth,
+    and five warm-up steps of 1.4 ms end in the middle of that ramp.  Returns the steps run."""
+    from cgt_amd import capi
+    n, t0 = 0, time.perf_counter()
+    while settle_ms > 0 and (time.perf_counter() - t0) * 1e3 < settle_ms:
+        for _ in range(5):
+            step()
+        capi.synchronize()
+        n += 5
+    return n
+
+
+def op_api_step_ms(cfg, steps, warmup, settle_ms=0):
     """The same layer built with the Op API (nn.conv2d / cross_channel_lrn /
     max_pool_2d, grad through the ops' pullbacks), compiled with cgt.function and
     replayed by the C++ interpreter on one stream: ms per step."""
@@ -714,6 +729,7 @@ def op_api_step_ms(cfg, steps, warmup):
     fun = cgt.function([xn, fn], [out, gx, gf], device_outputs=True)
     args = (xn.value, fn.value)
     del out, gx, gf
+    settle_clock(lambda: fun(*args), settle_ms)
     for _ in range(warmup):
         fun(*args)
     capi.synchronize()
@@ -808,6 +824,7 @@ def measure(workload, args, primary):
                            algo=forced or args.conv_algo)
         parity = {"ok": True, "skipped": True} if args.no_check else check_layer_against_oracle(cfg, forced or args.conv_algo)
 
+    settle_steps = settle_clock(layer.step, args.settle_ms)
     for _ in range(args.warmup):
         layer.step()
     capi.synchronize()
@@ -901,6 +918,8 @@ def measure(workload, args, primary):
         config["lrn"] = dict(zip(("size", "alpha", "beta", "k"), cfg["lrn"]))
     res = {
         "value": round(value, 3), "ms_per_step": round(ms_per_step, 4), "config": config,
+        # untimed steps run before the warm-up steps so that the timed ones see the sustained clock
+        "clock_settle": {"ms": args.settle_ms, "steps": settle_steps},
         "frac_fp32_mfma_peak": round(value / FP32_MFMA_PEAK_TFLOPS, 4),
         # the dominant kernel: the slowest MFMA GEMM launch of a step
         "roofline": {"bound": "mfma", "kernel": dominant.kernel, "stage": dominant.name,
@@ -930,6 +949,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--settle-ms", type=float, default=60.0,
+                    help="milliseconds of untimed steps before the warm-up steps (0: none): the device reaches the "
+                         "clock it sustains only after about 25 ms under load")
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS) + [GEMM_WORKLOAD])
     ap.add_argument("--stage-reps", type=int, default=20)
     ap.add_argument("--cpu-sample", type=int, default=16, help="images in the CPU baseline sample")
@@ -978,7 +1000,7 @@ def main():
     out["device"] = capi.device_name()
     parity_ok = res["parity"]["ok"]
     if not is_gemm and not args.no_op_api:
-        ms, n_instr = op_api_step_ms(cfg, args.steps, args.warmup)
+        ms, n_instr = op_api_step_ms(cfg, args.steps, args.warmup, args.settle_ms)
         out["op_api_step"] = {"ms_per_step": round(ms, 4), "TFLOPs": round(res["value"] * res["ms_per_step"] / ms, 3),
                               "instructions": n_instr,
                               "what": "the same step through nn.conv2d / cross_channel_lrn / max_pool_2d + grad, compiled "
@@ -1052,6 +1074,8 @@ def compact_line(out):
     line["roofline"] = {k: roof[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel", "stage",
                                              "flops_per_launch", "avg_launch_ms", "timing")}
     line["frac_fp32_mfma_peak"] = out["frac_fp32_mfma_peak"]
+    if "clock_settle" in out:       # untimed steps before the warm-up steps: {"ms": asked for, "steps": run}
+        line["clock_settle"] = out["clock_settle"]
     if "cpu_baseline" in out:
         cpu = out["cpu_baseline"]
         line["cpu_baseline"] = {k: cpu[k] for k in ("value", "unit", "cores", "kind") if k in cpu}

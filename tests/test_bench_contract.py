@@ -142,6 +142,8 @@ def test_default_workload_prints_the_contract_line():
     for name, row in out["workloads"].items():
         assert row["value"] > 0 and row["ms_per_step"] > 0 and row["gemm_frac"] > 0 and row["parity_ok"] is True
         assert name.startswith("raw_gemm") or 0 < row["hbm_worst"][1] <= row["hbm_best"][1] < 1.2
+    # untimed steps in front of the warm-up steps (the clock ramps for ~25 ms after an idle stretch) are declared
+    assert out["clock_settle"]["ms"] == 60.0 and out["clock_settle"]["steps"] >= 5
     assert set(out["hbm_reference"]) == {"copy_kernel_1GiB", "runtime_memcpy_1GiB", "write_fill_1GiB", "read_sum_1GiB", "add_2r1w_1GiB"}
     assert all(0.2 < v < 1.0 for v in out["hbm_reference"].values())
 

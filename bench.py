@@ -357,7 +357,7 @@ class LayerOnGpu(object):
         s = self.stream
         self.xpad = empty((K.conv_same_padded_size(B * C, H, W, (r, c)),))
         self.gypad = empty((K.conv_same_padded_size(B * L, H, W, (r, c)),))
-        self.fk, self.fflip, self.gfk = empty((L, r * c, C)), empty((C, r * c, L)), empty((L, r, c, C))
+        self.fk, self.fflip = empty((L, r * c, C)), empty((C, r * c, L))
         self.y, self.gx, self.gf = empty((B, L, H, W)), empty(self.x.shape), empty(self.f.shape)
 
         def call(fn, *a):
@@ -395,10 +395,9 @@ class LayerOnGpu(object):
         st.append(Stage("gemm_dgrad", "sgemm_kernel",
                         lambda: call(lib.cgt_amd_conv_same_product_f32, self.gypad.ptr, self.fflip.ptr, None, 0, B, L, H, W, C, r, c, self.gx.ptr, None, s),
                         gemm_flops, "mfma", gemm_bytes))
-        st.append(Stage("gemm_wgrad", "sgemm_kernel", lambda: call(lib.cgt_amd_conv_same_wgrad_f32, self.gypad.ptr, self.xpad.ptr, B, C, H, W, L, r, c, self.gfk.ptr, s),
+        # (the kernel that sums the product's K pieces stores the gradient in the filters' own layout)
+        st.append(Stage("gemm_wgrad", "sgemm_kernel", lambda: call(lib.cgt_amd_conv_same_bwd_filter_f32, self.gypad.ptr, self.xpad.ptr, B, C, H, W, L, r, c, self.gf.ptr, s),
                         gemm_flops, "mfma", gemm_bytes))
-        st.append(Stage("filter_grad_layout", "batched_transpose_kernel",
-                        lambda: K.transpose4(self.gfk, (0, 3, 1, 2), out=self.gf, stream=s), 8 * L * Z, "hbm"))
         self.stages = st
         self.conv_flops = 6 * Bmn * L * Z
         self.extra_stages = []

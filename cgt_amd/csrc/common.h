@@ -53,10 +53,13 @@ struct ConvGemm {
     int relu;              // mode 3: x * (x >= 0) on the way out
     signed char* mask;     // mode 3: (x >= 0) as int8, same shape as the output, or null
     const PatchGeom* patch = nullptr;      // modes 1, 4: gather the column buffer's elements from the image
+    int out_taps = 0;      // mode 2: > 0 = store the result [M][taps * C] as [M][C][taps], the filters' own layout (ldc == N)
 };
 int sgemm_conv(const ConvGemm& cv, long M, long N, const float* A, const float* B, float* C, long ldc, void* stream);
 // out[i] = ws[0][i] + ... + ws[n - 1][i], i < count, added in that order (gemm.hip's split-K reduce)
-int reduce_partials(const float* ws, float* out, long count, int n, void* stream);
+// taps > 0: the array is rows of row_len floats whose columns are ordered (tap, channel), and the sums are
+// stored as [row][channel][tap], the layout of the filters
+int reduce_partials(const float* ws, float* out, long count, int n, void* stream, int row_len = 0, int taps = 0);
 // 1 if sgemm_conv has a tile shape for these extents (output channels of the product, channels of the image)
 bool sgemm_conv_supported(int mode, long filters, long channels);
 

@@ -450,13 +450,11 @@ CGT_API int cgt_amd_conv_same_bwd_filter_f32(const float* gypad, const float* xp
     const long taps = (long)kh * kw;
     if (B == 0) return cgt_amd_fill_u32(gf, 0u, L * C * taps, stream);
     CGT_ARG_CHECK(cgt_amd_conv_same_supported(C, L, kh, kw, g.ph, g.pw, 1, 1), "conv_same_bwd_filter: unsupported extents C=%ld L=%ld", C, L);
-    float* wk = stream_workspace(stream, kWsConvFilter, (size_t)L * C * taps * sizeof(float), "conv_same_bwd_filter");
-    if (!wk) return CGT_AMD_ERR_NOMEM;
-    if ((rc = cgt_amd_conv_same_wgrad_f32(gypad, xpad, B, C, H, W, L, kh, kw, wk, stream))) return rc;
-    // [L][tap][C] -> [L][C][kh][kw]
-    const long ws[4] = {L, kh, kw, C};
-    const int ax[4] = {0, 3, 1, 2};
-    return cgt_amd_transpose4_f32(wk, ws, ax, gf, stream);
+    CGT_ARG_CHECK(gypad && xpad && gf, "conv_same_bwd_filter: null pointer");
+    // the product's columns are (tap, channel); the kernel that sums its K pieces stores [L][C][kh][kw]
+    ConvGemm cv = {2, B, C, g.plane, (int)g.Wp, kh, kw, g.tpi, g.spi, H, W, nullptr, 0, nullptr};
+    cv.out_taps = (int)taps;
+    return sgemm_conv(cv, L, taps * C, gypad + g.ph * g.Wp + g.pw, xpad, gf, taps * C, stream);
 }
 
 // The weight gradient's K axis is cut per image, so its partial sums are at least one [L][Z]

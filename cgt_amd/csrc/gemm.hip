@@ -1070,10 +1070,20 @@ __global__ __launch_bounds__(256) void tail_reduce_conv_kernel(const float* __re
 // sum per output would be one long chain of load latencies.
 constexpr int kReduceGroups = 4;
 
+// A weight gradient computed with its columns ordered (tap, channel) and stored as the filters are,
+// [row][channel][tap]: flat index row * n + tap * (n / taps) + channel -> (row * (n / taps) + channel) * taps + tap.
+__device__ __forceinline__ long filter_layout_index(long i, int n, int taps) {
+    const long r = i / n;
+    const int c = (int)(i - r * n), channels = n / taps;
+    const int tap = c / channels, ch = c - tap * channels;
+    return (r * channels + ch) * taps + tap;
+}
+
+// taps > 0: the sums are stored through filter_layout_index (C dense, ldc == N).
 template <bool VEC>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws,
                                                             float* __restrict__ C, long MN, int N,
-                                                            long ldc, int splits) {
+                                                            long ldc, int splits, int taps = 0) {
     typedef typename std::conditional<VEC, float4, float>::type T;
     constexpr int W = VEC ? 4 : 1;
     __shared__ T part[kReduceGroups][64];
@@ -1114,6 +1124,17 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
             tot += p;
         }
     }
+    if (taps > 0) {
+        if constexpr (VEC) {
+            C[filter_layout_index(i, N, taps)] = tot.x;
+            C[filter_layout_index(i + 1, N, taps)] = tot.y;
+            C[filter_layout_index(i + 2, N, taps)] = tot.z;
+            C[filter_layout_index(i + 3, N, taps)] = tot.w;
+        } else {
+            C[filter_layout_index(i, N, taps)] = tot;
+        }
+        return;
+    }
     if constexpr (VEC) {
         // N % 4 == 0: the four outputs share a row of C
         const long r = i / N, c = i - r * N;
@@ -1130,7 +1151,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 // owns 64 outputs; wavefront g adds partials [g * per, (g + 1) * per) in order, 8 loads in flight,
 // and the 16 sums are added in order: the same fixed order on every run.
 __global__ __launch_bounds__(1024) void reduce_many_kernel(const float* __restrict__ ws, float* __restrict__ out,
-                                                           long count, int n) {
+                                                           long count, int n, int row_len = 0, int taps = 0) {
     __shared__ float part[16][64];
     const int col = threadIdx.x & 63, g = threadIdx.x >> 6;
     const long i = (long)blockIdx.x * 64 + col;
@@ -1153,16 +1174,25 @@ __global__ __launch_bounds__(1024) void reduce_many_kernel(const float* __restri
     float tot = part[0][col];
 #pragma unroll
     for (int k = 1; k < 16; ++k) tot += part[k][col];
-    out[i] = tot;
+    out[taps > 0 ? filter_layout_index(i, row_len, taps) : i] = tot;
 }
 
 // out[i] = ws[0][i] + ws[1][i] + ... + ws[n - 1][i] for i < count, added in a fixed order (groups of
 // consecutive partials, then the group sums): the weight gradient of a very large batch sums
 // per-group results with it, the reduction-shaped weight gradient its workgroups' results.
-int reduce_partials(const float* ws, float* out, long count, int n, void* stream) {
+int reduce_partials(const float* ws, float* out, long count, int n, void* stream, int row_len, int taps) {
     if (n >= 64 && count <= (1L << 16)) {
-        reduce_many_kernel<<<dim3((unsigned)cdiv(count, 64L)), dim3(1024), 0, as_stream(stream)>>>(ws, out, count, n);
+        reduce_many_kernel<<<dim3((unsigned)cdiv(count, 64L)), dim3(1024), 0, as_stream(stream)>>>(ws, out, count, n, row_len, taps);
         CGT_LAUNCH_CHECK("reduce_many_kernel");
+        return CGT_AMD_OK;
+    }
+    if (taps > 0) {         // rows of row_len floats, stored in the filters' layout
+        const bool vec4 = row_len % 4 == 0 && reinterpret_cast<uintptr_t>(ws) % 16 == 0;
+        const long nblocks = cdiv(count, vec4 ? 256L : 64L);
+        CGT_ARG_CHECK(nblocks < (1L << 31), "reduce_partials: too many elements");
+        if (vec4) splitk_reduce_kernel<true><<<dim3((unsigned)nblocks), dim3(256), 0, as_stream(stream)>>>(ws, out, count, row_len, row_len, n, taps);
+        else splitk_reduce_kernel<false><<<dim3((unsigned)nblocks), dim3(256), 0, as_stream(stream)>>>(ws, out, count, row_len, row_len, n, taps);
+        CGT_LAUNCH_CHECK("splitk_reduce_kernel");
         return CGT_AMD_OK;
     }
     const bool vec = count % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && reinterpret_cast<uintptr_t>(ws) % 16 == 0;
@@ -1498,6 +1528,18 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
             if (!a.ws) return ws_rc;
         }
     }
+    // a weight gradient wanted in the filters' layout: the reduce kernel stores it that way; a product
+    // that is not split writes its one "partial" to the workspace and the same kernel moves it
+    const int out_taps = cv && cv->mode == 2 ? cv->out_taps : 0;
+    float* const C_final = C;
+    if (out_taps > 0) {
+        CGT_ARG_CHECK(P == 1 && ldc == N && N % out_taps == 0, "sgemm_conv: the filters' layout needs a dense [M][taps * C] result");
+        if (a.splits == 1) {
+            C = workspace((size_t)M * N * sizeof(float));
+            if (!C) return ws_rc;
+            a.C = C;
+        }
+    }
     // tail split (single product, no split-K): tiles beyond the last full
     // round of the chip are cut along K so the partial round is balanced
     a.main_wgs = (int)(tiles * P);
@@ -1505,7 +1547,8 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     a.tail_kchunk = a.kchunk;
     long tail_tiles = 0;
     const long nk = cdiv(K, KT);
-    if (P == 1 && a.splits == 1 && tiles >= kNumCU && tiles < 24L * kNumCU && tiles % kNumCU != 0 && nk >= 16) {
+    if (P == 1 && a.splits == 1 && tiles >= kNumCU && tiles < 24L * kNumCU && tiles % kNumCU != 0 && nk >= 16 &&
+        out_taps == 0) {     // (there the workspace holds the product itself)
         const long r = tiles % kNumCU;
         long best_s = 1;
         double best_t = (double)cdiv(r, kNumCU);             // tail time in units of one whole tile
@@ -1544,7 +1587,10 @@ static int gemm_dispatch(int tA, int tB, long P, long M, long N, long K, const f
     else if (conv_kernel) launch_conv(cv->mode, shape, grid, st, a);
     else launch_trans(tA, tB, pipe, deep, shape, grid, st, a);
     CGT_LAUNCH_CHECK("sgemm_kernel");
-    if (a.splits >= 64 && M * N <= (1L << 16) && ldc == N) {
+    if (out_taps > 0) {
+        int rc = reduce_partials(a.splits > 1 ? a.ws : C, C_final, M * N, a.splits, stream, (int)N, out_taps);
+        if (rc) return rc;
+    } else if (a.splits >= 64 && M * N <= (1L << 16) && ldc == N) {
         int rc = reduce_partials(a.ws, C, M * N, a.splits, stream);      // hundreds of partials of a small result
         if (rc) return rc;
     } else if (a.splits > 1) {

@@ -412,7 +412,8 @@ int cgt_amd_conv_same_wgrad_f32(const float *gypad, const float *xpad, long B, l
 int cgt_amd_conv_same_bwd_data_f32(const float *gypad, const float *f, long B, long C, long H, long W,
                                    long L, int kh, int kw, float *gx, void *stream);
 
-/* gf [L,C,kh,kw] from the padded cotangent and the padded input. */
+/* gf [L,C,kh,kw] from the padded cotangent and the padded input (the wgrad product above, its
+ * split-K reduce kernel storing the filters' layout: no separate transpose). */
 int cgt_amd_conv_same_bwd_filter_f32(const float *gypad, const float *xpad, long B, long C, long H,
                                      long W, long L, int kh, int kw, float *gf, void *stream);
 

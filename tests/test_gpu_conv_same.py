@@ -58,6 +58,9 @@ CASES = [
     (1, 160, 6, 6, 96, (3, 3)),
     (2, 96, 5, 13, 208, (1, 3)),
     (3, 64, 13, 13, 64, (3, 3)),
+    # many K pieces of a small weight gradient (the kernel that sums them stores the filters' layout)
+    (48, 16, 20, 22, 16, (3, 3)),
+    (40, 32, 15, 15, 48, (5, 3)),
 ]
 
 

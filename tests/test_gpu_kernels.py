@@ -204,6 +204,28 @@ def test_max_pool_all_negative_and_constant(K):
         assert np.array_equal(mask.get(), rmask) and bits_equal(top.get(), rtop)
 
 
+@pytest.mark.parametrize("xshape,k,p,s", [((2, 3, 13, 17), (3, 3), (0, 0), (2, 2)), ((2, 16, 56, 56), (2, 2), (0, 0), (2, 2)),
+                                         ((1, 96, 55, 55), (3, 3), (0, 0), (2, 2)), ((2, 5, 9, 9), (3, 3), (1, 1), (1, 1)),
+                                         ((3, 4, 20, 31), (4, 4), (0, 0), (1, 1))])
+def test_max_pool_and_im2col_with_nan_and_infinite_inputs(K, xshape, k, p, s):
+    # the reference's scan starts from -FLT_MAX / index -1 and keeps a cell only if it compares
+    # greater (include/pooling.h:46-54): NaN and -inf never win, a window of nothing else yields
+    # (-FLT_MAX, -1).  Selection and copying carry the bits through unchanged.
+    rs = np.random.RandomState(7)
+    x = rs.randn(*xshape).astype(np.float32)
+    m = rs.rand(*xshape)
+    x[m < 0.15] = np.nan
+    x[(m >= 0.15) & (m < 0.25)] = -np.inf
+    x[(m >= 0.25) & (m < 0.3)] = np.inf
+    x[0, 0, :4, :4] = np.nan
+    x[0, 0, 4:8, :4] = -np.inf
+    rtop, rmask = O.max_pool(x, k, p, s)
+    assert rmask.min() == -1 and (rtop == -np.finfo(np.float32).max).any()
+    top, mask = K.max_pool(gpu(x), k, p, s)
+    assert np.array_equal(mask.get(), rmask) and bits_equal(top.get(), rtop)
+    assert bits_equal(K.im2col(gpu(x), k, p, s).get(), O.im2col(x, k, p, s))
+
+
 # ---------------------------------------------------------------- LRN vs oracle
 
 LRN_CASES = [
@@ -283,6 +305,45 @@ def test_lrn_forward_large_arrays(K, shape, size):
     # top alone (no scale array): the pixel-per-lane kernel at this size too
     top_only = K.lrn_fwd(gpu(x), size, 0.3, 0.75, 1.0, want_scale=False).get()
     assert relfro(top_only, rtop) <= 5e-6 and np.max(np.abs(top_only - rtop) / (np.abs(rtop) + 1e-6)) <= 1e-4
+
+
+def test_lrn_confines_non_finite_inputs_to_their_windows(K):
+    # A documented difference.  The reference keeps a running window sum down the channels
+    # (include/lrn.cuh:22-50: add the entering square, subtract the leaving one), so once an
+    # infinite or NaN input has entered, inf - inf leaves NaN in the sum for every later channel
+    # of that pixel.  The kernels here sum every window afresh: the same values wherever the
+    # reference's are finite, and non-finite results only for the windows that hold the input.
+    rs = np.random.RandomState(3)
+    x = rs.randn(2, 16, 9, 9).astype(np.float32)
+    x[0, 3, 2, 2], x[1, 5, 4, 4], x[1, 7, 1, 1] = np.inf, np.nan, -np.inf
+    rtop, rscale = O.lrn_fwd(x, 5, 1e-4, 0.75)
+    top, scale = K.lrn_fwd(gpu(x), 5, 1e-4, 0.75)
+    top, scale = top.get(), scale.get()
+    fin = np.isfinite(rtop) & np.isfinite(rscale)
+    assert fin.sum() > 0.9 * fin.size
+    assert np.allclose(top[fin], rtop[fin], rtol=1e-5, atol=1e-7) and np.allclose(scale[fin], rscale[fin], rtol=1e-6)
+    bad = ~np.isfinite(scale)
+    assert not (bad & np.isfinite(rscale)).any()            # never non-finite where the reference is finite
+    for (n, c, h, w) in [(0, 3, 2, 2), (1, 5, 4, 4), (1, 7, 1, 1)]:
+        assert bad[n, max(0, c - 2):c + 3, h, w].all()      # the windows that contain the input
+        assert np.isfinite(scale[n, c + 3:, h, w]).all() and not np.isfinite(rscale[n, c + 3:, h, w]).any()
+
+
+def test_lrn_window_sums_do_not_inherit_the_running_sums_cancellation(K):
+    # The second documented difference, same cause.  One channel of 1e4 among ones: the
+    # reference's running sum holds 1e8 while that square is in the window, the ones added
+    # meanwhile fall below its last bit, and after the subtraction the sum is 0 (later even
+    # negative) where it should be 5.  The oracle, which restates the reference, shows it; the
+    # kernels match the float64 window sums.  (On inputs of ordinary range the two agree to
+    # rounding: every other LRN test compares the kernels with the oracle.)
+    x = np.ones((1, 12, 3, 3), np.float32)
+    x[0, 0] = 1e4
+    _, rscale = O.lrn_fwd(x, 5, 0.1, 0.75)
+    _, scale = K.lrn_fwd(gpu(x), 5, 0.1, 0.75)
+    sq = x.astype(np.float64) ** 2
+    exact = np.stack([1 + 0.1 / 5 * sq[0, max(0, c - 2):c + 3].sum(axis=0) for c in range(12)])[None]
+    assert np.allclose(scale.get(), exact, rtol=1e-6)
+    assert abs(rscale[0, 5, 0, 0] - 1.0) < 1e-6 and abs(exact[0, 5, 0, 0] - 1.1) < 1e-12 and rscale[0, 11, 0, 0] < 1.0
 
 
 def test_lrn_rejects_size_above_channels(K):

@@ -272,3 +272,51 @@ def test_workspaces_of_rising_sizes_do_not_pile_up(L):
     largest = sizes[-1] ** 2 * 4 * 256        # an upper bound on one call's workspace (<= 256 MiB cap)
     assert held <= min(2 * largest, 600 << 20), (held, largest, total_asked)
     del s
+
+
+def test_host_threads_on_their_own_streams_get_the_bits_of_the_calls_made_alone(L):
+    # the library keeps per-stream workspaces and a thread-local error string: four host threads,
+    # each launching a mixed sequence (fused conv products with their split-K / tail workspaces,
+    # pooling, im2col / col2im, LRN, ragged Mul22) on a stream of its own, must neither disturb each
+    # other nor change a bit of what the same calls give one after another on the null stream
+    import threading
+    from cgt_amd import capi, kernels as K
+
+    def work(seed, stream, out):
+        rs = np.random.RandomState(seed)
+        res = []
+        for _ in range(6):
+            B, C, Lf = rs.randint(1, 9), 16 * rs.randint(1, 5), 16 * rs.randint(1, 5)
+            H, W = rs.randint(5, 40), rs.randint(5, 40)
+            x = rs.randn(B, C, H, W).astype(np.float32)
+            f = (rs.randn(Lf, C, 3, 3) / 12).astype(np.float32)
+            xg, fg = gpu(x), gpu(f)
+            xpad = K.conv_same_pad(xg, (3, 3), stream=stream)
+            y = K.conv_same_fwd(xpad, fg, x.shape, stream=stream)
+            top, mask = K.max_pool(y, (2, 2), (0, 0), (2, 2), stream=stream)
+            gyp = K.conv_same_pad(gpu(rs.randn(*y.shape).astype(np.float32)), (3, 3), stream=stream)
+            gx = K.conv_same_bwd_data(gyp, fg, x.shape, stream=stream)
+            gf = K.conv_same_bwd_filter(gyp, xpad, x.shape, f.shape, stream=stream)
+            col = K.im2col(xg, (3, 3), (1, 1), (1, 1), stream=stream)
+            im = K.col2im(col, x.shape, (3, 3), (1, 1), (1, 1), stream=stream)
+            lt, ls = K.lrn_fwd(y, 5, 1e-4, 0.75, stream=stream)
+            M, N, Kk = rs.randint(1, 300), rs.randint(1, 300), rs.randint(1, 3000)
+            c = K.mul22(gpu(rs.randn(M, Kk).astype(np.float32)), gpu(rs.randn(Kk, N).astype(np.float32)), stream=stream)
+            capi.synchronize(stream)
+            res.append([t.get() for t in (y, top, mask, gx, gf, col, im, lt, ls, c)])
+        out[seed] = res
+
+    alone, together = {}, {}
+    for s in range(4):
+        work(s, None, alone)
+    streams = [capi.Stream() for _ in range(4)]
+    threads = [threading.Thread(target=work, args=(s, streams[s].handle, together)) for s in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert sorted(together) == [0, 1, 2, 3]
+    for s in range(4):
+        for ra, rb in zip(alone[s], together[s]):
+            for a, b in zip(ra, rb):
+                assert a.shape == b.shape and np.array_equal(a.view(np.uint32), b.view(np.uint32))

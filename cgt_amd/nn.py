@@ -143,6 +143,36 @@ class SpatialConvolution(object):
         return core.broadcast("+", tmp, self.bias, "xxxx,1x11")
 
 
+class Affine(object):
+    """x.dot(W) + b with W [input_size, output_size], b [1, output_size] (reference cgt/nn.py:198-213): the
+    fully connected layer that ends the reference's convolutional examples.  Weights default to zero as there."""
+
+    def __init__(self, input_size, output_size, name=None, weight_init=None, bias_init=None):
+        import numpy as np
+        input_size, output_size = int(input_size), int(output_size)
+        self.name = "unnamed" if name is None else name
+        w = np.zeros((input_size, output_size), np.float32) if weight_init is None else \
+            np.asarray(weight_init, np.float32).reshape(input_size, output_size)
+        b = np.zeros((1, output_size), np.float32) if bias_init is None else np.asarray(bias_init, np.float32).reshape(1, output_size)
+        self.weight = core.constant(w)
+        self.bias = core.constant(b)
+
+    def __call__(self, x):
+        return core.broadcast("+", core.dot(core.as_node(x), self.weight), self.bias, "xx,1x")
+
+
+def softmax(x, axis=1):
+    """exp(x) / sum(exp(x), axis) for a matrix, without the shift by the row maximum -- as the
+    reference computes it (cgt/nn.py:55-59)."""
+    out = core.exp(core.as_node(x))
+    return core.broadcast("/", out, core.sum(out, axis=axis, keepdims=True), "xx,x1" if axis == 1 else "xx,1x")
+
+
+def logsoftmax(x, axis=1):
+    """log(softmax(x)) (cgt/nn.py:61-62)."""
+    return core.log(softmax(x, axis=axis))
+
+
 def max_pool_2d(x, kernelshape, pad=(0, 0), stride=(1, 1)):
     kernel_h, kernel_w = kernelshape
     pad_h, pad_w = pad

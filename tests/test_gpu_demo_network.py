@@ -58,7 +58,7 @@ def torch_steps(params, batches, stepsize, rho, eps, want_grads=False):
         logprobs = torch.log(e / e.sum(1, keepdim=True))
         loss = -(logprobs * onehot).sum() / x.shape[0]
         grads = torch.autograd.grad(loss, [p[k] for k in sorted(p)])
-        losses.append(float(loss))
+        losses.append(float(loss.detach()))
         if want_grads:
             return losses, {k: g.numpy() for k, g in zip(sorted(p), grads)}
         with torch.no_grad():
